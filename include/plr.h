@@ -1,0 +1,115 @@
+/*
+ * plr -- C ABI of the MI355X logistic-regression shard kernels.
+ *
+ * A worker keeps its local shard (samples X, labels y) resident in HBM and,
+ * once per round, hands over theta and receives the shard's loss and batch
+ * gradient.  These entry points replace the inline loops of the reference's
+ * worker (the reference has no FFI/plugin interface around this compute; the
+ * loops sit between paracel_read and paracel_bupdate inside
+ * logistic_regression::dgd_learning), so each declaration cites the
+ * reference lines whose result it returns.
+ *
+ * Conventions: plain C types only; every pointer is caller-owned HOST memory,
+ * valid for the duration of the call; calls are synchronous (they return
+ * after the context's stream has drained); one context per worker process,
+ * not thread-safe (as the reference's kvclt is not); results are bitwise
+ * reproducible for a fixed (n, d, device).  All functions returning int give
+ * PLR_OK (0) or a negative plr_status; plr_last_error() describes the last
+ * failure on that context.
+ */
+#ifndef PLR_H
+#define PLR_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct plr_ctx plr_ctx; /* opaque: device buffers + one HIP stream */
+
+typedef enum {
+  PLR_OK = 0,
+  PLR_ERR_INVALID = -1,     /* null pointer, bad shape, bad flag            */
+  PLR_ERR_HIP = -2,         /* a HIP runtime call failed                    */
+  PLR_ERR_NOMEM = -3,       /* device or pinned allocation failed           */
+  PLR_ERR_NODATA = -4,      /* no shard resident yet                        */
+  PLR_ERR_UNSUPPORTED = -5  /* shape outside what the kernels cover         */
+} plr_status;
+
+/* loss formula selector for plr_loss_grad / plr_calc_loss */
+#define PLR_LOSS_REFERENCE 0u /* -log(h) / -log(1-h): lr.cpp:325-329; may be
+                                 +inf for saturated rows, like the reference */
+#define PLR_LOSS_STABLE 1u    /* log1p(exp(-|z|)) + max(-/+z, 0): same value,
+                                 finite for any z                            */
+#define PLR_LOSS_NONE 2u      /* skip the loss (loss_sum receives 0)         */
+
+/* Create a context on HIP device `device_id`.  Replaces nothing in the
+ * reference (which has no device); it is the constructor-time set-up a
+ * worker does next to paralg's (include/ps.hpp:102-125). */
+int plr_create(plr_ctx** out, int device_id);
+void plr_destroy(plr_ctx* ctx);
+
+/* Make the shard resident: n rows of d doubles, row-major with pitch
+ * ldx >= d (in doubles), plus n labels.  Copies; the caller keeps its
+ * buffers.  This is the layout lr.cpp:76-93 (local_parser) produces in
+ * `samples`/`labels` (lr.hpp:75-76), flattened.  n may be 0. */
+int plr_set_data(plr_ctx* ctx, const double* X, int64_t n, int64_t d,
+                 int64_t ldx, const double* y);
+
+/* Streaming form of the same: reserve an n x d shard, then fill row ranges
+ * in any order (each row exactly once before the first compute call). */
+int plr_alloc_data(plr_ctx* ctx, int64_t n, int64_t d);
+int plr_set_data_chunk(plr_ctx* ctx, int64_t row0, int64_t nrows,
+                       const double* X, int64_t ldx, const double* y);
+
+/* One fused pass over the shard with theta (d doubles):
+ *   gsum[j]  = sum_i (h_i - y_i) * x_ij,  h_i = 1/(1+exp(-x_i.theta))
+ *              (lr.cpp:69-72 with ext_utility.hpp:171-174; the data term of
+ *               lr.cpp:133-137 with the sign of the residual flipped and
+ *               alpha factored out)
+ *   loss_sum = sum_i l_i as lr.cpp:322-330 accumulates it (before the
+ *              all-reduce and the division of lr.cpp:331-335)
+ *   n_out    = number of rows summed.
+ * gsum, loss_sum, n_out may each be NULL. */
+int plr_loss_grad(plr_ctx* ctx, const double* theta, double* gsum,
+                  double* loss_sum, int64_t* n_out, unsigned flags);
+
+/* One round's delta exactly as lr.cpp:119,125-138 leaves it in `delta`
+ * (reference signs): delta = alpha*X^T(y-h) - 2*alpha*beta*n*theta.
+ * loss_sum (nullable) as above with the reference formula. */
+int plr_dgd_delta(plr_ctx* ctx, const double* theta, double alpha, double beta,
+                  double* delta, double* loss_sum);
+
+/* lr.cpp:322-330: the loss pass alone (no gradient). */
+int plr_calc_loss(plr_ctx* ctx, const double* theta, double* loss_sum,
+                  int64_t* n_out, unsigned flags);
+
+/* lr.cpp:361-363: h_i for every resident row (n doubles out). */
+int plr_predict(plr_ctx* ctx, const double* theta, double* h_out);
+
+/* Shape of the resident shard (0,0 before plr_set_data). */
+int plr_get_shape(const plr_ctx* ctx, int64_t* n, int64_t* d);
+
+/* Timing of the streaming kernel, measured with HIP events recorded on the
+ * context's own stream around the kernel launch only: milliseconds of the
+ * last launch and, since the last plr_reset_timing, the sum and the count.
+ * Any pointer may be NULL. */
+int plr_get_timing(const plr_ctx* ctx, double* last_ms, double* sum_ms,
+                   int64_t* launches);
+int plr_reset_timing(plr_ctx* ctx);
+
+/* Human-readable description of the kernel variant chosen for the resident
+ * shape (tile shape, grid), for logs.  Context-owned, never freed. */
+const char* plr_kernel_info(const plr_ctx* ctx);
+
+/* Context-owned message of the last error ("" if none); never freed.
+ * plr_last_error(NULL) describes the last plr_create failure. */
+const char* plr_last_error(const plr_ctx* ctx);
+
+const char* plr_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PLR_H */

@@ -1,0 +1,47 @@
+"""Build steps for the native parts of the package (run on CPU; hipcc
+cross-compiles gfx950 without a GPU).  Outputs land in-tree next to this file.
+"""
+import os
+import shutil
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(_HERE)
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # keep packed-fp32 instructions out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+]
+
+
+def _run(cmd, cwd=None):
+    print("+", " ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True, cwd=cwd)
+
+
+def hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found")
+    return exe
+
+
+def build_libplr():
+    """HIP kernels + C ABI -> paracel_amd/libplr.so"""
+    out = os.path.join(_HERE, "libplr.so")
+    _run([hipcc()] + HIPCC_FLAGS + ["-o", out, os.path.join(_HERE, "csrc", "plr_capi.hip")])
+    return out
+
+
+def build_libplr_gen():
+    """Seeded shard generator (host C) -> paracel_amd/libplr_gen.so"""
+    out = os.path.join(_HERE, "libplr_gen.so")
+    _run(["gcc", "-O2", "-ffp-contract=off", "-fPIC", "-shared", "-pthread", "-Wall", "-Wextra",
+          "-o", out, os.path.join(_HERE, "datagen", "plr_gen.c"), "-lm"])
+    return out
+
+
+def build_all():
+    return [build_libplr(), build_libplr_gen()]

@@ -1,0 +1,440 @@
+// C ABI (include/plr.h) over the gfx950 shard kernels: context, resident
+// shard, variant selection, launches.  Host C++ only sees plain pointers and
+// sizes; nothing here falls back to a CPU path -- if HIP fails, the call
+// fails.
+#include "../../include/plr.h"
+
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <string>
+
+#include "plr_kernels.hpp"
+
+namespace {
+
+using plr::FinishArgs;
+using plr::PassArgs;
+
+typedef void (*pass_fn)(PassArgs);
+
+struct Variant {
+  int nch, R, wcol, wrow;
+  pass_fn grad, nograd;
+};
+
+#define PLR_VARIANT(NCH, R, WCOL, WROW, MINW)                          \
+  {NCH, R, WCOL, WROW, plr::shard_pass<NCH, R, WCOL, WROW, MINW, true>, \
+   plr::shard_pass<NCH, R, WCOL, WROW, MINW, false>}
+
+// Ordered by the number of 128-column chunks they cover (wcol * nch).
+const Variant kVariants[] = {
+    PLR_VARIANT(1, 16, 1, 4, 4),   // d <= 128
+    PLR_VARIANT(2, 16, 1, 4, 2),   // d <= 256
+    PLR_VARIANT(4, 8, 1, 4, 2),    // d <= 512
+    PLR_VARIANT(8, 4, 1, 4, 2),    // d <= 1024
+    PLR_VARIANT(8, 4, 2, 1, 2),    // d <= 2048
+    PLR_VARIANT(8, 4, 4, 1, 2),    // d <= 4096
+    PLR_VARIANT(8, 4, 8, 1, 2),    // d <= 8192
+    PLR_VARIANT(16, 1, 8, 1, 2),   // d <= 16384
+    PLR_VARIANT(20, 1, 8, 1, 2),   // d <= 20480
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+constexpr int64_t kMaxCols = 20480;
+
+std::string g_create_error;
+
+}  // namespace
+
+struct plr_ctx {
+  int device = 0;
+  int num_cu = 0;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+
+  // resident shard
+  double* dX = nullptr;
+  double* dy = nullptr;
+  int64_t n = 0, d = 0, pitch = 0;
+  bool have_data = false;
+
+  // per-shape workspace
+  const Variant* var = nullptr;
+  int nch_rt = 0;
+  int grid = 0, grid_nograd = 0;
+  int64_t theta_len = 0;
+  double* d_theta = nullptr;    // theta_len doubles, zero padded
+  double* d_part_g = nullptr;   // grid x pitch
+  double* d_part_loss = nullptr;  // max(grid, grid_nograd)
+  double* d_out = nullptr;      // d + 1
+  double* d_h = nullptr;        // n (predict), lazily allocated
+  double* h_theta = nullptr;    // pinned, theta_len
+  double* h_out = nullptr;      // pinned, d + 1
+
+  double last_ms = 0., sum_ms = 0.;
+  int64_t launches = 0;
+
+  std::string err;
+  std::string info;
+};
+
+namespace {
+
+int fail(plr_ctx* c, int code, const std::string& msg) {
+  if (c) c->err = msg;
+  return code;
+}
+
+#define PLR_HIP(c, call)                                                     \
+  do {                                                                       \
+    hipError_t e_ = (call);                                                  \
+    if (e_ != hipSuccess) {                                                  \
+      char b_[512];                                                          \
+      snprintf(b_, sizeof b_, "%s failed: %s (%s:%d)", #call,                \
+               hipGetErrorString(e_), __FILE__, __LINE__);                   \
+      (void)hipGetLastError();                                               \
+      return fail((c), (e_ == hipErrorOutOfMemory) ? PLR_ERR_NOMEM           \
+                                                   : PLR_ERR_HIP, b_);       \
+    }                                                                        \
+  } while (0)
+
+void free_shape(plr_ctx* c) {
+  (void)hipSetDevice(c->device);
+  if (c->dX) (void)hipFree(c->dX);
+  if (c->dy) (void)hipFree(c->dy);
+  if (c->d_theta) (void)hipFree(c->d_theta);
+  if (c->d_part_g) (void)hipFree(c->d_part_g);
+  if (c->d_part_loss) (void)hipFree(c->d_part_loss);
+  if (c->d_out) (void)hipFree(c->d_out);
+  if (c->d_h) (void)hipFree(c->d_h);
+  if (c->h_theta) (void)hipHostFree(c->h_theta);
+  if (c->h_out) (void)hipHostFree(c->h_out);
+  c->dX = c->dy = c->d_theta = c->d_part_g = c->d_part_loss = c->d_out =
+      c->d_h = c->h_theta = c->h_out = nullptr;
+  c->n = c->d = c->pitch = 0;
+  c->have_data = false;
+  c->var = nullptr;
+  c->info.clear();
+}
+
+int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Pick the kernel variant and persistent grid for an n x d shard.
+int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
+  if (d > kMaxCols)
+    return fail(c, PLR_ERR_UNSUPPORTED,
+                "d = " + std::to_string(d) + " exceeds the widest kernel variant (" +
+                    std::to_string(kMaxCols) + " columns)");
+  const int64_t pitch = (d + 1) & ~int64_t(1);
+  const int64_t chunks = ceil_div(pitch, plr::kChunkCols);
+  const Variant* v = nullptr;
+  for (int i = 0; i < kNumVariants; ++i)
+    if ((int64_t)kVariants[i].nch * kVariants[i].wcol >= chunks) {
+      v = &kVariants[i];
+      break;
+    }
+  if (!v) return fail(c, PLR_ERR_UNSUPPORTED, "no kernel variant covers this width");
+  c->var = v;
+  c->pitch = pitch;
+  c->nch_rt = (int)ceil_div(chunks, v->wcol);
+  c->theta_len = (int64_t)v->wcol * c->nch_rt * plr::kChunkCols;
+  const int threads = plr::kWave * v->wcol * v->wrow;
+  const int64_t ntiles = ceil_div(n, v->R);
+  const int64_t want = ceil_div(ntiles, v->wrow);
+  int occ = 0, occ_ng = 0;
+  PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                 &occ, reinterpret_cast<const void*>(v->grad), threads, 0));
+  PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                 &occ_ng, reinterpret_cast<const void*>(v->nograd), threads, 0));
+  if (occ < 1 || occ_ng < 1)
+    return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
+  int64_t g = (int64_t)c->num_cu * occ, g2 = (int64_t)c->num_cu * occ_ng;
+  if (g > want) g = want;
+  if (g2 > want) g2 = want;
+  if (g < 1) g = 1;
+  if (g2 < 1) g2 = 1;
+  c->grid = (int)g;
+  c->grid_nograd = (int)g2;
+  char b[256];
+  snprintf(b, sizeof b,
+           "shard_pass<NCH=%d,R=%d,WCOL=%d,WROW=%d> nch_rt=%d pitch=%lld grid=%d x %d "
+           "threads (occupancy %d blocks/CU, %d CUs)",
+           v->nch, v->R, v->wcol, v->wrow, c->nch_rt, (long long)pitch, c->grid,
+           threads, occ, c->num_cu);
+  c->info = b;
+  return PLR_OK;
+}
+
+int alloc_shape(plr_ctx* c, int64_t n, int64_t d) {
+  if (n < 0 || d < 1)
+    return fail(c, PLR_ERR_INVALID, "need n >= 0 and d >= 1");
+  PLR_HIP(c, hipSetDevice(c->device));
+  free_shape(c);
+  int rc = plan_shape(c, n, d);
+  if (rc != PLR_OK) return rc;
+  c->n = n;
+  c->d = d;
+  // lanes of the chunk that straddles the end of the last row read (and then
+  // discard) up to one slab past it: keep that much slack mapped
+  const size_t xbytes = (size_t)n * c->pitch * sizeof(double) +
+                        (size_t)c->theta_len * sizeof(double);
+  if (n > 0) {
+    PLR_HIP(c, hipMalloc(&c->dX, xbytes));
+    PLR_HIP(c, hipMalloc(&c->dy, (size_t)n * sizeof(double)));
+  }
+  const int gmax = c->grid > c->grid_nograd ? c->grid : c->grid_nograd;
+  PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)c->theta_len * sizeof(double)));
+  PLR_HIP(c, hipMalloc(&c->d_part_g, (size_t)c->grid * c->pitch * sizeof(double)));
+  PLR_HIP(c, hipMalloc(&c->d_part_loss, (size_t)gmax * sizeof(double)));
+  PLR_HIP(c, hipMalloc(&c->d_out, (size_t)(d + 1) * sizeof(double)));
+  PLR_HIP(c, hipHostMalloc(&c->h_theta, (size_t)c->theta_len * sizeof(double), hipHostMallocDefault));
+  PLR_HIP(c, hipHostMalloc(&c->h_out, (size_t)(d + 1) * sizeof(double), hipHostMallocDefault));
+  memset(c->h_theta, 0, (size_t)c->theta_len * sizeof(double));
+  PLR_HIP(c, hipMemsetAsync(c->d_theta, 0, (size_t)c->theta_len * sizeof(double), c->stream));
+  if (n > 0 && c->pitch != d)  // the pad column must read as zero
+    PLR_HIP(c, hipMemset2DAsync(c->dX + d, (size_t)c->pitch * sizeof(double), 0,
+                                (size_t)(c->pitch - d) * sizeof(double), (size_t)n,
+                                c->stream));
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  c->have_data = true;
+  return PLR_OK;
+}
+
+int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
+                int64_t ldx, const double* y) {
+  if (nrows == 0) return PLR_OK;
+  if (!X || !y) return fail(c, PLR_ERR_INVALID, "X and y must not be NULL");
+  if (ldx < c->d) return fail(c, PLR_ERR_INVALID, "ldx must be >= d");
+  if (row0 < 0 || nrows < 0 || row0 + nrows > c->n)
+    return fail(c, PLR_ERR_INVALID, "row range outside the reserved shard");
+  PLR_HIP(c, hipSetDevice(c->device));
+  PLR_HIP(c, hipMemcpy2D(c->dX + row0 * c->pitch, (size_t)c->pitch * sizeof(double), X,
+                         (size_t)ldx * sizeof(double), (size_t)c->d * sizeof(double),
+                         (size_t)nrows, hipMemcpyHostToDevice));
+  PLR_HIP(c, hipMemcpy(c->dy + row0, y, (size_t)nrows * sizeof(double),
+                       hipMemcpyHostToDevice));
+  return PLR_OK;
+}
+
+enum PassKind { kPassGrad, kPassDelta, kPassLoss, kPassPredict };
+
+// theta -> device, streaming kernel (timed), finishing kernel, results ->
+// pinned host.  Returns after the stream has drained.
+int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
+             double alpha, double beta) {
+  if (!c->have_data) return fail(c, PLR_ERR_NODATA, "no shard resident: call plr_set_data first");
+  if (!theta) return fail(c, PLR_ERR_INVALID, "theta must not be NULL");
+  if (loss_mode > plr::kLossNone) return fail(c, PLR_ERR_INVALID, "unknown loss flag");
+  PLR_HIP(c, hipSetDevice(c->device));
+  const Variant* v = c->var;
+  const bool grad = (kind == kPassGrad || kind == kPassDelta);
+  const int grid = grad ? c->grid : c->grid_nograd;
+  const int threads = plr::kWave * v->wcol * v->wrow;
+
+  memcpy(c->h_theta, theta, (size_t)c->d * sizeof(double));
+  PLR_HIP(c, hipMemcpyAsync(c->d_theta, c->h_theta, (size_t)c->d * sizeof(double),
+                            hipMemcpyHostToDevice, c->stream));
+  if (kind == kPassPredict && !c->d_h && c->n > 0)
+    PLR_HIP(c, hipMalloc(&c->d_h, (size_t)c->n * sizeof(double)));
+
+  PassArgs pa;
+  pa.X = c->dX;
+  pa.y = (kind == kPassPredict) ? nullptr : c->dy;
+  pa.theta = c->d_theta;
+  pa.part_g = c->d_part_g;
+  pa.part_loss = c->d_part_loss;
+  pa.h_out = (kind == kPassPredict) ? c->d_h : nullptr;
+  pa.n = c->n;
+  pa.pitch = c->pitch;
+  pa.ntiles = ceil_div(c->n, v->R);
+  pa.nch_rt = c->nch_rt;
+  pa.loss_mode = (kind == kPassPredict) ? (unsigned)plr::kLossNone : loss_mode;
+
+  PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
+  hipLaunchKernelGGL(grad ? v->grad : v->nograd, dim3(grid), dim3(threads), 0,
+                     c->stream, pa);
+  PLR_HIP(c, hipGetLastError());
+  PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
+
+  if (kind != kPassPredict) {
+    FinishArgs fa;
+    fa.part_g = c->d_part_g;
+    fa.part_loss = c->d_part_loss;
+    fa.theta = c->d_theta;
+    fa.out = c->d_out;
+    fa.pitch = c->pitch;
+    fa.d = c->d;
+    fa.n = c->n;
+    fa.nparts = grid;
+    fa.delta_mode = (kind == kPassDelta) ? 1 : 0;
+    fa.have_grad = grad ? 1 : 0;
+    fa.alpha = alpha;
+    fa.coff2 = 2. * beta * alpha;
+    const int fgrid = grad ? (int)ceil_div(c->d, plr::kFinCols) : 1;
+    hipLaunchKernelGGL(plr::finish_pass, dim3(fgrid),
+                       dim3(plr::kFinCols * plr::kFinSlices), 0, c->stream, fa);
+    PLR_HIP(c, hipGetLastError());
+    PLR_HIP(c, hipMemcpyAsync(c->h_out, c->d_out, (size_t)(c->d + 1) * sizeof(double),
+                              hipMemcpyDeviceToHost, c->stream));
+  }
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  float ms = 0.f;
+  PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
+  c->last_ms = ms;
+  c->sum_ms += ms;
+  c->launches += 1;
+  return PLR_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int plr_create(plr_ctx** out, int device_id) {
+  if (!out) {
+    g_create_error = "out must not be NULL";
+    return PLR_ERR_INVALID;
+  }
+  *out = nullptr;
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count < 1) {
+    (void)hipGetLastError();
+    g_create_error = std::string("no HIP device available: ") + hipGetErrorString(e);
+    return PLR_ERR_HIP;
+  }
+  if (device_id < 0 || device_id >= count) {
+    g_create_error = "device_id out of range";
+    return PLR_ERR_INVALID;
+  }
+  plr_ctx* c = new plr_ctx();
+  c->device = device_id;
+  hipDeviceProp_t prop;
+  if ((e = hipSetDevice(device_id)) != hipSuccess ||
+      (e = hipGetDeviceProperties(&prop, device_id)) != hipSuccess ||
+      (e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking)) != hipSuccess ||
+      (e = hipEventCreate(&c->ev0)) != hipSuccess ||
+      (e = hipEventCreate(&c->ev1)) != hipSuccess) {
+    g_create_error = std::string("context set-up failed: ") + hipGetErrorString(e);
+    (void)hipGetLastError();
+    plr_destroy(c);
+    return PLR_ERR_HIP;
+  }
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    g_create_error = std::string("device is ") + prop.gcnArchName +
+                     "; this library carries gfx950 code only";
+    plr_destroy(c);
+    return PLR_ERR_UNSUPPORTED;
+  }
+  c->num_cu = prop.multiProcessorCount;
+  *out = c;
+  return PLR_OK;
+}
+
+void plr_destroy(plr_ctx* c) {
+  if (!c) return;
+  free_shape(c);
+  if (c->ev0) (void)hipEventDestroy(c->ev0);
+  if (c->ev1) (void)hipEventDestroy(c->ev1);
+  if (c->stream) (void)hipStreamDestroy(c->stream);
+  delete c;
+}
+
+int plr_alloc_data(plr_ctx* c, int64_t n, int64_t d) {
+  if (!c) return PLR_ERR_INVALID;
+  return alloc_shape(c, n, d);
+}
+
+int plr_set_data_chunk(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
+                       int64_t ldx, const double* y) {
+  if (!c) return PLR_ERR_INVALID;
+  if (!c->have_data) return fail(c, PLR_ERR_NODATA, "call plr_alloc_data first");
+  return upload_rows(c, row0, nrows, X, ldx, y);
+}
+
+int plr_set_data(plr_ctx* c, const double* X, int64_t n, int64_t d, int64_t ldx,
+                 const double* y) {
+  if (!c) return PLR_ERR_INVALID;
+  if (n > 0 && (!X || !y)) return fail(c, PLR_ERR_INVALID, "X and y must not be NULL");
+  if (ldx < d) return fail(c, PLR_ERR_INVALID, "ldx must be >= d");
+  int rc = alloc_shape(c, n, d);
+  if (rc != PLR_OK) return rc;
+  return upload_rows(c, 0, n, X, ldx, y);
+}
+
+int plr_loss_grad(plr_ctx* c, const double* theta, double* gsum, double* loss_sum,
+                  int64_t* n_out, unsigned flags) {
+  if (!c) return PLR_ERR_INVALID;
+  int rc = run_pass(c, kPassGrad, theta, flags, 0., 0.);
+  if (rc != PLR_OK) return rc;
+  if (gsum) memcpy(gsum, c->h_out, (size_t)c->d * sizeof(double));
+  if (loss_sum) *loss_sum = c->h_out[c->d];
+  if (n_out) *n_out = c->n;
+  return PLR_OK;
+}
+
+int plr_dgd_delta(plr_ctx* c, const double* theta, double alpha, double beta,
+                  double* delta, double* loss_sum) {
+  if (!c) return PLR_ERR_INVALID;
+  if (!delta) return fail(c, PLR_ERR_INVALID, "delta must not be NULL");
+  int rc = run_pass(c, kPassDelta, theta,
+                    loss_sum ? plr::kLossReference : plr::kLossNone, alpha, beta);
+  if (rc != PLR_OK) return rc;
+  memcpy(delta, c->h_out, (size_t)c->d * sizeof(double));
+  if (loss_sum) *loss_sum = c->h_out[c->d];
+  return PLR_OK;
+}
+
+int plr_calc_loss(plr_ctx* c, const double* theta, double* loss_sum, int64_t* n_out,
+                  unsigned flags) {
+  if (!c) return PLR_ERR_INVALID;
+  if (flags == PLR_LOSS_NONE) return fail(c, PLR_ERR_INVALID, "plr_calc_loss needs a loss formula");
+  int rc = run_pass(c, kPassLoss, theta, flags, 0., 0.);
+  if (rc != PLR_OK) return rc;
+  if (loss_sum) *loss_sum = c->h_out[c->d];
+  if (n_out) *n_out = c->n;
+  return PLR_OK;
+}
+
+int plr_predict(plr_ctx* c, const double* theta, double* h_out) {
+  if (!c) return PLR_ERR_INVALID;
+  if (!h_out && c->n > 0) return fail(c, PLR_ERR_INVALID, "h_out must not be NULL");
+  int rc = run_pass(c, kPassPredict, theta, plr::kLossNone, 0., 0.);
+  if (rc != PLR_OK) return rc;
+  if (c->n > 0)
+    PLR_HIP(c, hipMemcpy(h_out, c->d_h, (size_t)c->n * sizeof(double), hipMemcpyDeviceToHost));
+  return PLR_OK;
+}
+
+int plr_get_shape(const plr_ctx* c, int64_t* n, int64_t* d) {
+  if (!c) return PLR_ERR_INVALID;
+  if (n) *n = c->n;
+  if (d) *d = c->d;
+  return PLR_OK;
+}
+
+int plr_get_timing(const plr_ctx* c, double* last_ms, double* sum_ms, int64_t* launches) {
+  if (!c) return PLR_ERR_INVALID;
+  if (last_ms) *last_ms = c->last_ms;
+  if (sum_ms) *sum_ms = c->sum_ms;
+  if (launches) *launches = c->launches;
+  return PLR_OK;
+}
+
+int plr_reset_timing(plr_ctx* c) {
+  if (!c) return PLR_ERR_INVALID;
+  c->last_ms = c->sum_ms = 0.;
+  c->launches = 0;
+  return PLR_OK;
+}
+
+const char* plr_kernel_info(const plr_ctx* c) { return c ? c->info.c_str() : ""; }
+
+const char* plr_last_error(const plr_ctx* c) {
+  return c ? c->err.c_str() : g_create_error.c_str();
+}
+
+const char* plr_version(void) { return "plr 0.1 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,397 @@
+// Device kernels for the logistic-regression shard pass on gfx950 (CDNA4).
+//
+// One fused, HBM-bound streaming pass.  X (n x d fp64, row-major, even pitch)
+// is read exactly once; everything derived from a row -- the dot product
+// x.theta, the sigmoid, the residual, the loss term and the rank-1 update of
+// the gradient -- happens on the registers the row was loaded into.
+//
+// Work decomposition
+//   * A wavefront (64 lanes) owns a slab of up to NCH*128 columns.  Within a
+//     128-column chunk lane l owns the adjacent pair (2l, 2l+1), so one
+//     global_load_dwordx4 per lane moves a contiguous 1 KiB per wave.
+//   * Rows are taken in tiles of R consecutive rows; all R*NCH loads of a
+//     tile are issued before the first use.  theta and the gradient
+//     accumulators for the slab live in registers for the kernel's lifetime.
+//   * The R per-lane partial dots are reduced across the 64 lanes by a
+//     transposing butterfly: log2(R) halving steps leave each lane with one
+//     row's partial, log2(64/R) plain butterfly steps finish it.  So the
+//     exp/log of a row is evaluated once per tile by the lane that holds
+//     it, not 64 times, and R-1+log2(64/R) lane exchanges replace 6R.
+//   * d > 1024: WCOL waves of a workgroup split the columns; their partial
+//     dots meet in LDS (double-buffered, one barrier per tile) and are summed
+//     in wave order.
+//   * Rows are spread over the grid tile-interleaved (tile t goes to row
+//     group t mod G), so at any moment the grid streams one contiguous window
+//     of X.
+// Determinism: no atomics; every sum has a fixed shape that depends only on
+// (n, d, grid), so results are bitwise reproducible.
+//
+// Replaces, for a resident shard, the loops of the reference's
+// alg/classification/logistic_regression/lr.cpp:69-72,132-138,322-330,361-363
+// and include/utils/ext_utility.hpp:171-174.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+namespace plr {
+
+typedef double v2d __attribute__((ext_vector_type(2)));
+
+// X is streamed once and never re-read: load it with the non-temporal hint.
+#ifndef PLR_NONTEMPORAL
+#define PLR_NONTEMPORAL 1
+#endif
+__device__ __forceinline__ v2d load_x(const v2d* p) {
+#if PLR_NONTEMPORAL
+  return __builtin_nontemporal_load(p);
+#else
+  return *p;
+#endif
+}
+
+constexpr int kWave = 64;
+constexpr int kChunkCols = 2 * kWave;  // columns per chunk (double2 per lane)
+
+enum : unsigned {
+  kLossReference = 0u,
+  kLossStable = 1u,
+  kLossNone = 2u,
+};
+
+struct PassArgs {
+  const double* X;       // n x pitch
+  const double* y;       // n
+  const double* theta;   // padded with zeros to wcol*nch_rt*128 entries
+  double* part_g;        // [grid][pitch]  per-workgroup partial gradients
+  double* part_loss;     // [grid]
+  double* h_out;         // n, or nullptr (predict)
+  int64_t n;
+  int64_t pitch;         // doubles per row in X, even, >= d
+  int64_t ntiles;        // ceil(n / R)
+  int nch_rt;            // chunks per wave actually used (<= NCH)
+  unsigned loss_mode;
+};
+
+// Row held by `lane` after the transposing reduction over R rows.
+template <int R>
+__device__ __forceinline__ int row_of_lane(int lane) {
+  int rho = 0;
+#pragma unroll
+  for (int s = 0; (1 << s) < R; ++s)
+    if (lane & (1 << s)) rho += R >> (s + 1);
+  return rho;
+}
+
+// Lowest lane that holds row r (inverse of row_of_lane on lanes [0, R)).
+template <int R>
+__host__ __device__ constexpr int lane_of_row(int r) {
+  int lane = 0;
+  for (int s = 0; (1 << s) < R; ++s)
+    if (r & (R >> (s + 1))) lane |= (1 << s);
+  return lane;
+}
+
+// p[r] = this lane's partial dot of row r.  Returns the full 64-lane sum of
+// row row_of_lane<R>(lane); identical bits in every lane holding that row.
+template <int R>
+__device__ __forceinline__ double reduce_rows(double (&p)[R], int lane) {
+#pragma unroll
+  for (int s = 0, cnt = R / 2; cnt >= 1; ++s, cnt >>= 1) {
+    const int m = 1 << s;
+    const bool up = (lane & m) != 0;
+#pragma unroll
+    for (int k = 0; k < cnt; ++k) {
+      const double send = up ? p[k] : p[k + cnt];
+      const double keep = up ? p[k + cnt] : p[k];
+      p[k] = keep + __shfl_xor(send, m, kWave);
+    }
+  }
+  double z = p[0];
+#pragma unroll
+  for (int m = R; m < kWave; m <<= 1) z += __shfl_xor(z, m, kWave);
+  return z;
+}
+
+__device__ __forceinline__ double bcast_lane(double v, int src_lane) {
+  // src_lane is a compile-time constant at every call site: two v_readlane.
+  int lo = __double2loint(v), hi = __double2hiint(v);
+  lo = __builtin_amdgcn_readlane(lo, src_lane);
+  hi = __builtin_amdgcn_readlane(hi, src_lane);
+  return __hiloint2double(hi, lo);
+}
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int m = 1; m < kWave; m <<= 1) v += __shfl_xor(v, m, kWave);
+  return v;
+}
+
+// One tile of R rows: loads, dots, lane reduction, sigmoid/residual/loss,
+// rank-1 update.  FULL = every row of the tile exists (no row predication).
+// ALLCH = the wave uses all NCH chunks (no per-chunk predication).
+template <int NCH, int R, int WCOL, bool GRAD, bool FULL, bool ALLCH>
+__device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_base,
+                                          int64_t row0, uint32_t lane_off, int lane,
+                                          int wc, int my_nch, int ragged_c,
+                                          bool lane_in_ragged, int my_row,
+                                          const v2d (&th)[NCH], v2d (&acc)[NCH],
+                                          double& loss_acc, double* zbuf) {
+  // ---- issue every load of the tile (uniform base + 32-bit lane offset) ----
+  v2d x[R][NCH];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const char* rowp = reinterpret_cast<const char*>(tile_base + (int64_t)r * a.pitch);
+    const bool rv = FULL || (row0 + r) < a.n;  // uniform
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      x[r][c] = v2d{0., 0.};
+      if (rv && (ALLCH || c < my_nch))  // uniform
+        x[r][c] = load_x(reinterpret_cast<const v2d*>(
+            rowp + lane_off + (uint32_t)(c * kChunkCols * sizeof(double))));
+    }
+  }
+  const int64_t myrow_g = row0 + my_row;
+  const bool my_valid = FULL || myrow_g < a.n;
+  double yv = 0.;
+  if (my_valid && a.y) yv = a.y[myrow_g];
+
+  // lanes past the end of the row in the ragged last chunk hold the next
+  // row's (or slack) bytes: zero them so they cannot poison the dot product
+  if (ragged_c >= 0) {
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+      if (c == ragged_c) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) x[r][c] = lane_in_ragged ? x[r][c] : v2d{0., 0.};
+      }
+  }
+
+  // ---- per-lane partial dots ----
+  double p[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    double s0 = 0., s1 = 0.;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      s0 = fma(x[r][c].x, th[c].x, s0);
+      s1 = fma(x[r][c].y, th[c].y, s1);
+    }
+    p[r] = s0 + s1;
+  }
+  double z = reduce_rows<R>(p, lane);
+
+  if (WCOL > 1) {
+    if (lane < R) zbuf[wc * R + my_row] = z;
+    __syncthreads();
+    double s = 0.;
+#pragma unroll
+    for (int w = 0; w < WCOL; ++w) s += zbuf[w * R + my_row];
+    z = s;
+  }
+
+  // ---- sigmoid, residual, loss for the row this lane holds ----
+  const double e = exp(-z);
+  const double h = 1. / (1. + e);
+  const double res = my_valid ? (h - yv) : 0.;
+  if (a.h_out && my_valid && lane < R && wc == 0) a.h_out[myrow_g] = h;
+  if (a.loss_mode != kLossNone) {
+    double l;
+    if (a.loss_mode == kLossReference) {
+      l = (yv == 1.) ? -log(h) : -log(1. - h);
+    } else {
+      const double sgn = (yv == 1.) ? -z : z;  // loss = log(1 + exp(sgn))
+      l = log1p(exp(-fabs(sgn))) + fmax(sgn, 0.);
+    }
+    if (my_valid && lane < R && wc == 0) loss_acc += l;
+  }
+
+  // ---- rank-1 update of the gradient slab from the same registers ----
+  if (GRAD) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const double rr = bcast_lane(res, lane_of_row<R>(r));
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        acc[c].x = fma(rr, x[r][c].x, acc[c].x);
+        acc[c].y = fma(rr, x[r][c].y, acc[c].y);
+      }
+    }
+  }
+}
+
+// NCH  : 128-column chunks per wave (compile-time bound; nch_rt used)
+// R    : rows per tile (power of two, <= 64)
+// WCOL : waves of a workgroup side by side over the columns
+// WROW : independent row groups per workgroup (must be 1 when WCOL > 1)
+// MINW : waves per SIMD the register allocation must leave room for
+// GRAD : accumulate the gradient (false: loss / predict only)
+template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD>
+__global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a) {
+  static_assert(WCOL == 1 || WROW == 1, "column-split workgroups own one row group");
+  static_assert((R & (R - 1)) == 0 && R <= kWave, "R must be a power of two");
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform
+  const int wc = (WCOL > 1) ? wave : 0;
+  const int wr = (WCOL > 1) ? 0 : wave;
+
+  const int64_t chunks = (a.pitch + kChunkCols - 1) / kChunkCols;
+  const int64_t slab_c0 = (int64_t)wc * a.nch_rt;          // first chunk of this wave
+  int64_t left = chunks - slab_c0;
+  const int my_nch = (int)(left < 0 ? 0 : (left > a.nch_rt ? a.nch_rt : left));
+  const int64_t slab_col0 = slab_c0 * kChunkCols;
+  const int64_t col0 = slab_col0 + 2 * lane;
+  const uint32_t lane_off = (uint32_t)(2 * lane * sizeof(double));
+  // the chunk that straddles the end of the row, if this wave owns it
+  const int tail_cols = (int)(a.pitch % kChunkCols);
+  const int ragged_c = (tail_cols != 0 && slab_c0 + my_nch == chunks && my_nch > 0)
+                           ? my_nch - 1 : -1;
+  const bool lane_in_ragged = 2 * lane < tail_cols;
+
+  // theta slab -> registers (theta is zero-padded on the device)
+  v2d th[NCH], acc[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    th[c] = v2d{0., 0.};
+    acc[c] = v2d{0., 0.};
+    if (c < a.nch_rt)
+      th[c] = *reinterpret_cast<const v2d*>(a.theta + col0 + (int64_t)c * kChunkCols);
+  }
+  double loss_acc = 0.;
+
+  __shared__ double zx[(WCOL > 1) ? 2 * WCOL * R : 1];
+
+  const int my_row = row_of_lane<R>(lane & (R - 1));
+  const int64_t group = (int64_t)blockIdx.x * WROW + wr;
+  const int64_t ngroups = (int64_t)gridDim.x * WROW;
+  const int64_t nfull = a.n / R;  // tiles with all R rows present
+
+  auto run_tiles = [&](auto allch) {
+    constexpr bool ALLCH = decltype(allch)::value;
+    int parity = 0;
+    for (int64_t tile = group; tile < a.ntiles; tile += ngroups, parity ^= 1) {
+      const int64_t row0 = tile * R;
+      const double* tile_base = a.X + row0 * a.pitch + slab_col0;
+      double* zbuf = zx + ((WCOL > 1) ? parity * (WCOL * R) : 0);
+      if (tile < nfull)
+        tile_step<NCH, R, WCOL, GRAD, true, ALLCH>(a, tile_base, row0, lane_off, lane, wc,
+                                                   my_nch, ragged_c, lane_in_ragged, my_row,
+                                                   th, acc, loss_acc, zbuf);
+      else
+        tile_step<NCH, R, WCOL, GRAD, false, ALLCH>(a, tile_base, row0, lane_off, lane, wc,
+                                                    my_nch, ragged_c, lane_in_ragged, my_row,
+                                                    th, acc, loss_acc, zbuf);
+    }
+  };
+  if (my_nch == NCH)
+    run_tiles(std::true_type{});
+  else
+    run_tiles(std::false_type{});
+
+  // ---- combine the workgroup's partials in a fixed order ----
+  if (GRAD) {
+    double* out = a.part_g + (int64_t)blockIdx.x * a.pitch;
+    if (WROW == 1) {
+#pragma unroll
+      for (int c = 0; c < NCH; ++c)
+        if (c < my_nch && (c != ragged_c || lane_in_ragged))
+          *reinterpret_cast<v2d*>(out + col0 + (int64_t)c * kChunkCols) = acc[c];
+    } else {
+      __shared__ v2d gx[(WROW > 1) ? (WROW - 1) * kWave : 1];
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        if (c < my_nch) {  // uniform over the workgroup (WCOL == 1 here)
+          if (wr > 0) gx[(wr - 1) * kWave + lane] = acc[c];
+          __syncthreads();
+          if (wr == 0) {
+            v2d s = acc[c];
+#pragma unroll
+            for (int w = 1; w < WROW; ++w) {
+              const v2d o = gx[(w - 1) * kWave + lane];
+              s.x += o.x;
+              s.y += o.y;
+            }
+            if (c != ragged_c || lane_in_ragged)
+              *reinterpret_cast<v2d*>(out + col0 + (int64_t)c * kChunkCols) = s;
+          }
+          __syncthreads();
+        }
+      }
+    }
+  }
+  {
+    __shared__ double lx[WCOL * WROW];
+    const double wl = wave_sum(loss_acc);
+    if (lane == 0) lx[wave] = wl;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      double s = 0.;
+#pragma unroll
+      for (int w = 0; w < WCOL * WROW; ++w) s += lx[w];
+      a.part_loss[blockIdx.x] = s;
+    }
+  }
+}
+
+struct FinishArgs {
+  const double* part_g;   // [nparts][pitch]
+  const double* part_loss;  // [nparts]
+  const double* theta;
+  double* out;            // d doubles (gsum or delta), then out[d] = loss_sum
+  int64_t pitch;
+  int64_t d;
+  int64_t n;
+  int nparts;
+  int delta_mode;         // 0: out = gsum; 1: out = -alpha*gsum - coff2*n*theta
+  int have_grad;
+  double alpha;
+  double coff2;
+};
+
+constexpr int kFinCols = 64;
+constexpr int kFinSlices = 16;
+
+// Sums the per-workgroup partials: thread (col, slice) adds parts slice,
+// slice+16, ... in order; the 16 slice sums meet in LDS and are added in
+// slice order.  Block 0 also folds the loss partials the same way.
+__global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a) {
+  __shared__ double sm[kFinSlices][kFinCols];
+  const int cx = threadIdx.x % kFinCols;
+  const int sl = threadIdx.x / kFinCols;
+  const int64_t col = (int64_t)blockIdx.x * kFinCols + cx;
+  if (a.have_grad) {
+    double s = 0.;
+    if (col < a.d)
+      for (int p = sl; p < a.nparts; p += kFinSlices)
+        s += a.part_g[(int64_t)p * a.pitch + col];
+    sm[sl][cx] = s;
+    __syncthreads();
+    if (sl == 0 && col < a.d) {
+      double g = sm[0][cx];
+#pragma unroll
+      for (int k = 1; k < kFinSlices; ++k) g += sm[k][cx];
+      if (a.delta_mode)
+        g = -a.alpha * g - (a.coff2 * (double)a.n) * a.theta[col];
+      a.out[col] = g;
+    }
+    __syncthreads();
+  }
+  if (blockIdx.x == 0) {
+    double s = 0.;
+    for (int p = threadIdx.x; p < a.nparts; p += kFinCols * kFinSlices)
+      s += a.part_loss[p];
+    sm[sl][cx] = s;
+    __syncthreads();
+    if (threadIdx.x < kFinCols) {
+      double t = sm[0][cx];
+#pragma unroll
+      for (int k = 1; k < kFinSlices; ++k) t += sm[k][cx];
+      t = wave_sum(t);
+      if (threadIdx.x == 0) a.out[a.d] = t;
+    }
+  }
+}
+
+}  // namespace plr

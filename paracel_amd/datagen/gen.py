@@ -1,0 +1,153 @@
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(os.path.dirname(_HERE), "libplr_gen.so")
+
+NORMAL, UNIFORM = 0, 1
+STREAM_THETA, STREAM_THETA_STAR = 5, 6
+
+
+class GenSpec(C.Structure):
+    _fields_ = [("seed", C.c_uint64), ("kind", C.c_int32), ("outlier_mod", C.c_int32),
+                ("scale", C.c_double), ("zero_prob", C.c_double), ("outlier_scale", C.c_double)]
+
+
+_lib = None
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            raise ImportError("%s is missing: run __graft_entry__.build()" % _LIB)
+        lib = C.CDLL(_LIB)
+        dp = C.POINTER(C.c_double)
+        lib.plr_gen_X.argtypes = [C.POINTER(GenSpec), C.c_int64, C.c_int64, C.c_int64, C.c_int64, dp, C.c_int]
+        lib.plr_gen_X.restype = None
+        lib.plr_gen_vec.argtypes = [C.c_uint64, C.c_uint64, C.c_int, C.c_double, C.c_double, C.c_int64, dp]
+        lib.plr_gen_vec.restype = None
+        lib.plr_gen_labels.argtypes = [C.POINTER(GenSpec), C.c_int64, C.c_int64, C.c_int64, C.c_int64, dp, dp, dp, C.c_int]
+        lib.plr_gen_labels.restype = None
+        lib.plr_gen_u01.argtypes = [C.c_uint64] * 4
+        lib.plr_gen_u01.restype = C.c_double
+        lib.plr_gen_normal.argtypes = [C.c_uint64] * 4
+        lib.plr_gen_normal.restype = C.c_double
+        _lib = lib
+    return _lib
+
+
+def _dp(a):
+    return a.ctypes.data_as(C.POINTER(C.c_double))
+
+
+def default_threads():
+    return max(1, min(16, os.cpu_count() or 1))
+
+
+def gen_X(spec, row0, nrows, d, threads=None, out=None):
+    X = out if out is not None else np.empty((nrows, d), dtype=np.float64)
+    assert X.flags.c_contiguous and X.shape == (nrows, d)
+    _load().plr_gen_X(C.byref(spec), row0, nrows, d, d, _dp(X), threads or default_threads())
+    return X
+
+
+def gen_vec(seed, stream, n, kind=NORMAL, scale=1.0, nonzero_frac=1.0):
+    out = np.empty(n, dtype=np.float64)
+    _load().plr_gen_vec(seed, stream, kind, scale, nonzero_frac, n, _dp(out))
+    return out
+
+
+def gen_labels(spec, row0, X, theta_star, threads=None):
+    n, d = X.shape
+    y = np.empty(n, dtype=np.float64)
+    ts = np.ascontiguousarray(theta_star, dtype=np.float64)
+    _load().plr_gen_labels(C.byref(spec), row0, n, d, d, _dp(X), _dp(ts), _dp(y),
+                           threads or default_threads())
+    return y
+
+
+def u01(seed, stream, i, j):
+    return _load().plr_gen_u01(seed, stream, i, j)
+
+
+def normal(seed, stream, i, j):
+    return _load().plr_gen_normal(seed, stream, i, j)
+
+
+class Config:
+    """One benchmark configuration: shape, distributions, hyper-parameters.
+
+    alpha/beta are the reference's knobs (lr.cpp:119,134): the un-normalised
+    update applies the L2 term once per sample, so plain gradient descent with
+    step lr on mean log-loss + (lam/2)|theta|^2 is alpha = lr/n, beta = lam/2.
+    """
+
+    def __init__(self, name, n, d, seed, kind, scale, lam, lr=0.1, zero_prob=0.0,
+                 outlier_mod=0, outlier_scale=1.0, theta_scale=1.0, theta_nonzero=1.0,
+                 theta0_zero=False):
+        self.name, self.n, self.d, self.seed = name, n, d, seed
+        self.spec = GenSpec(seed, kind, outlier_mod, scale, zero_prob, outlier_scale)
+        self.lam, self.lr = lam, lr
+        self.theta_scale, self.theta_nonzero = theta_scale, theta_nonzero
+        self.theta0_zero = theta0_zero
+
+    @property
+    def alpha(self):
+        return self.lr / self.n
+
+    @property
+    def beta(self):
+        return self.lam / 2.0
+
+    def scaled(self, n):
+        """Same distributions and seed on the first n rows (alpha keeps the full n)."""
+        c = Config.__new__(Config)
+        c.__dict__.update(self.__dict__)
+        c.n = n
+        return c
+
+    def theta_star(self):
+        return gen_vec(self.seed, STREAM_THETA_STAR, self.d, NORMAL, self.theta_scale,
+                       self.theta_nonzero)
+
+    def theta(self):
+        """theta the timed gradient step is evaluated at."""
+        if self.theta0_zero:
+            return np.zeros(self.d)
+        return self.theta_star()
+
+    def rows(self, row0, nrows, threads=None):
+        X = gen_X(self.spec, row0, nrows, self.d, threads)
+        y = gen_labels(self.spec, row0, X, self.theta_star(), threads)
+        return X, y
+
+    def algorithmic_bytes(self):
+        """X once + y + theta in + gradient out + loss."""
+        return 8 * self.n * self.d + 8 * self.n + 16 * self.d + 8
+
+
+def configs():
+    d2 = 1000
+    return {
+        # dense, CPU-runnable: X~N(0,1), theta*~N(0,1), theta0=0, lam=0.01, lr=0.1
+        "c1_dense_100k_x_100": Config("c1_dense_100k_x_100", 100_000, 100, 0x5EED0001, NORMAL, 1.0,
+                                      lam=0.01, theta0_zero=True),
+        # headline: X~N(0,1/d), theta~N(0,1), y~Bernoulli(sigmoid(X theta))
+        "c2_headline_1m_x_1000": Config("c2_headline_1m_x_1000", 1_000_000, d2, 0x5EED0002, NORMAL,
+                                        1.0 / np.sqrt(d2), lam=0.01),
+        # tall-skinny: U[-1,1], 1% of rows x100, theta*~N(0, sigma=0.1)
+        "c3_tall_10m_x_256": Config("c3_tall_10m_x_256", 10_000_000, 256, 0x5EED0003, UNIFORM, 1.0,
+                                    lam=0.001, outlier_mod=100, outlier_scale=100.0,
+                                    theta_scale=0.1),
+        # wide: 90% exact zeros, theta* nonzero on 5% of coordinates
+        "c4_wide_200k_x_16384": Config("c4_wide_200k_x_16384", 200_000, 16384, 0x5EED0004, NORMAL,
+                                       1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
+        "c4b_wide_200k_x_16385": Config("c4b_wide_200k_x_16385", 200_000, 16385, 0x5EED0004, NORMAL,
+                                        1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
+        # end-to-end through the host parameter server
+        "c5_e2e_2m_x_512": Config("c5_e2e_2m_x_512", 2_000_000, 512, 0x5EED0005, NORMAL,
+                                  1.0 / np.sqrt(512), lam=0.01, theta0_zero=True),
+    }

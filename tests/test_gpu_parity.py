@@ -1,0 +1,267 @@
+"""GPU parity: the HIP shard pass, called through the C ABI, against the CPU
+oracle on identical seeded inputs.
+
+Tolerances (fp64): relative L2 error <= 1e-10 per gradient / delta, <= 1e-8 on
+theta after 100 iterations; loss sums relative <= 1e-10 where no row is
+saturated (|z| moderate), stated per test otherwise.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GRAD_TOL = 1e-10
+LOSS_TOL = 1e-10
+
+
+def rel(a, b):
+    nb = np.linalg.norm(b)
+    return np.linalg.norm(a - b) / (nb if nb > 0 else 1.0)
+
+
+def make(gen, n, d, seed=0xABCD, scale=None, theta_scale=1.0):
+    spec = gen.GenSpec(seed, gen.NORMAL, 0, scale if scale else 1.0 / np.sqrt(d), 0.0, 1.0)
+    X = gen.gen_X(spec, 0, n, d)
+    ts = gen.gen_vec(seed, gen.STREAM_THETA_STAR, d, gen.NORMAL, theta_scale)
+    y = gen.gen_labels(spec, 0, X, ts) if n else np.zeros(0)
+    th = gen.gen_vec(seed, gen.STREAM_THETA, d, gen.NORMAL, theta_scale)
+    return X, y, th
+
+
+# every kernel variant (d <= 128, 256, 512, 1024, 2048, 4096, 8192, 16384,
+# 20480), widths that are not multiples of the 128-column chunk or of 2, and
+# row counts around the tile sizes
+SHAPES = [
+    (1, 1), (5, 2), (7, 3), (64, 17), (300, 64), (1000, 100), (257, 127), (1030, 128),
+    (515, 129), (1000, 255), (4099, 256), (333, 257), (1001, 512), (2051, 1000),
+    (700, 1024), (300, 1025), (260, 2047), (130, 4097), (70, 8193), (40, 16384),
+    (37, 16385), (21, 20480),
+]
+
+
+@pytest.mark.parametrize("n,d", SHAPES)
+def test_loss_grad_matches_oracle(plr, oracle, gen, n, d):
+    print("case n=%d d=%d" % (n, d), flush=True)
+    X, y, th = make(gen, n, d)
+    plr.set_data(X, y)
+    print(plr.kernel_info(), flush=True)
+    g, loss, n_out = plr.loss_grad(th)
+    assert n_out == n
+    g_ref = oracle.gsum(X, y, th)
+    assert rel(g, g_ref) <= GRAD_TOL
+    # long-double arbiter agrees too
+    assert rel(g, oracle.gsum(X, y, th, hp=True)) <= GRAD_TOL
+    loss_ref = oracle.calc_loss_sum(X, y, th)
+    assert abs(loss - loss_ref) <= LOSS_TOL * abs(loss_ref)
+
+
+@pytest.mark.parametrize("n,d", [(1000, 100), (2051, 1000), (333, 257), (70, 8193), (37, 16385)])
+def test_dgd_delta_matches_oracle(plr, oracle, gen, n, d):
+    X, y, th = make(gen, n, d)
+    plr.set_data(X, y)
+    alpha, beta = 0.1 / n, 0.005
+    delta, loss = plr.dgd_delta(th, alpha, beta)
+    d_ref = oracle.dgd_delta(X, y, th, alpha, beta)
+    assert rel(delta, d_ref) <= GRAD_TOL
+    assert rel(delta, oracle.dgd_delta_hp(X, y, th, alpha, beta)) <= GRAD_TOL
+    # a shuffled traversal (the reference shuffles with a time seed) only moves rounding
+    order = np.random.default_rng(1).permutation(n)
+    assert rel(delta, oracle.dgd_delta(X, y, th, alpha, beta, order=order)) <= GRAD_TOL
+    assert abs(loss - oracle.calc_loss_sum(X, y, th)) <= LOSS_TOL * abs(loss)
+    # the reference's own knobs (README: alpha=0.001, beta=0.01)
+    delta2, _ = plr.dgd_delta(th, 0.001, 0.01, want_loss=False)
+    assert rel(delta2, oracle.dgd_delta(X, y, th, 0.001, 0.01)) <= GRAD_TOL
+
+
+@pytest.mark.parametrize("n,d", [(999, 100), (2051, 1000), (130, 4097)])
+def test_calc_loss_and_predict(plr, oracle, gen, n, d):
+    X, y, th = make(gen, n, d)
+    plr.set_data(X, y)
+    loss, n_out = plr.calc_loss(th)
+    assert n_out == n
+    ref = oracle.calc_loss_sum(X, y, th)
+    assert abs(loss - ref) <= LOSS_TOL * abs(ref)
+    h = plr.predict(th)
+    h_ref = oracle.predict(X, th)
+    assert np.max(np.abs(h - h_ref)) <= 1e-14
+    # fused pass and loss-only pass agree with each other
+    _, loss2, _ = plr.loss_grad(th)
+    assert abs(loss2 - loss) <= 1e-12 * abs(loss)
+
+
+def test_theta_zero_closed_forms(plr, gen):
+    # theta = 0 => h = 1/2 exactly: gsum = X^T (1/2 - y) (a plain GEMV), loss = n ln 2
+    X, y, _ = make(gen, 3001, 300)
+    plr.set_data(X, y)
+    g, loss, n = plr.loss_grad(np.zeros(300))
+    assert rel(g, X.T @ (0.5 - y)) <= 1e-13
+    assert abs(loss - n * np.log(2.0)) <= 1e-12 * n
+    for flags in (0, 1):
+        l2, _ = plr.calc_loss(np.zeros(300), flags)
+        assert abs(l2 - n * np.log(2.0)) <= 1e-12 * n
+
+
+def test_x_zero_gives_pure_l2_delta(plr, gen):
+    # X = 0 => delta = -2 alpha beta n theta exactly (up to one rounding)
+    n, d = 777, 130
+    X = np.zeros((n, d))
+    y = (np.arange(n) % 2).astype(float)
+    th = gen.gen_vec(3, gen.STREAM_THETA, d)
+    plr.set_data(X, y)
+    delta, _ = plr.dgd_delta(th, 1e-3, 0.25)
+    np.testing.assert_allclose(delta, -2 * 1e-3 * 0.25 * n * th, rtol=4e-16, atol=0)
+
+
+def test_one_hot_rows_count_columns(plr):
+    # one-hot rows with theta = 0: gsum[j] = sum over rows hitting j of (1/2 - y)
+    n, d = 1000, 200
+    rng = np.random.default_rng(5)
+    cols = rng.integers(0, d, n)
+    X = np.zeros((n, d))
+    X[np.arange(n), cols] = 1.0
+    y = (rng.random(n) < 0.3).astype(float)
+    plr.set_data(X, y)
+    g, _, _ = plr.loss_grad(np.zeros(d))
+    want = np.zeros(d)
+    np.add.at(want, cols, 0.5 - y)
+    np.testing.assert_array_equal(g, want)  # halves add exactly
+
+
+def test_shard_additivity(plr, gen):
+    # gsum(S1 u S2) = gsum(S1) + gsum(S2): the multi-worker invariant of update.cpp:26-32
+    X, y, th = make(gen, 5000, 700)
+    plr.set_data(X, y)
+    g, loss, _ = plr.loss_grad(th)
+    plr.set_data(X[:1777], y[:1777])
+    g1, l1, _ = plr.loss_grad(th)
+    plr.set_data(X[1777:], y[1777:])
+    g2, l2, _ = plr.loss_grad(th)
+    assert rel(g1 + g2, g) <= 1e-13
+    assert abs(l1 + l2 - loss) <= 1e-13 * abs(loss)
+
+
+def test_bitwise_reproducible(plr, gen):
+    X, y, th = make(gen, 9000, 1000)
+    plr.set_data(X, y)
+    g1, l1, _ = plr.loss_grad(th)
+    g2, l2, _ = plr.loss_grad(th)
+    np.testing.assert_array_equal(g1, g2)
+    assert l1 == l2
+
+
+def test_chunked_upload_equals_whole(plr, gen):
+    X, y, th = make(gen, 3000, 513)
+    plr.set_data(X, y)
+    g, loss, _ = plr.loss_grad(th)
+    plr.alloc_data(3000, 513)
+    for lo, hi in ((2000, 3000), (0, 700), (700, 2000)):
+        plr.set_data_chunk(lo, X[lo:hi], y[lo:hi])
+    g2, loss2, _ = plr.loss_grad(th)
+    np.testing.assert_array_equal(g, g2)
+    assert loss == loss2
+
+
+def test_pitched_input(plr, oracle, gen):
+    X, y, th = make(gen, 500, 333)
+    wide = np.full((500, 400), np.nan)
+    wide[:, :333] = X
+    plr.set_data(wide[:, :333], y)  # ldx = 400 > d, NaNs outside must not be read
+    g, _, _ = plr.loss_grad(th)
+    assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
+
+
+def test_saturated_rows_stable_vs_reference_loss(plr, oracle, gen):
+    # rows scaled x100 saturate the sigmoid: the reference formula returns
+    # +inf once exp(-z) < 2^-53 (lr.cpp:328 with h == 1.0); the stable form
+    # stays finite and matches the long-double value
+    n, d = 2000, 256
+    spec = gen.GenSpec(77, gen.UNIFORM, 100, 1.0, 0.0, 100.0)
+    X = gen.gen_X(spec, 0, n, d)
+    ts = gen.gen_vec(77, gen.STREAM_THETA_STAR, d, gen.NORMAL, 0.1)
+    y = gen.gen_labels(spec, 0, X, ts)
+    th = 3.0 * ts
+    # flip a label on a saturated row so the naive formula overflows
+    z = X @ th
+    i = int(np.argmax(z))
+    assert z[i] > 40
+    y[i] = 0.0
+    plr.set_data(X, y)
+    _, loss_ref_formula, _ = plr.loss_grad(th, 0)
+    assert np.isinf(loss_ref_formula) and np.isinf(oracle.calc_loss_sum(X, y, th))
+    g, loss_stable, _ = plr.loss_grad(th, 1)
+    want = oracle.stable_loss_sum_hp(X, y, th)
+    assert np.isfinite(loss_stable)
+    assert abs(loss_stable - want) <= 1e-12 * abs(want)
+    # the gradient is insensitive to saturation
+    assert rel(g, oracle.gsum(X, y, th, hp=True)) <= GRAD_TOL
+
+
+def test_stable_loss_equals_reference_loss_when_unsaturated(plr, gen):
+    X, y, th = make(gen, 4000, 100)
+    plr.set_data(X, y)
+    a, _ = plr.calc_loss(th, 0)
+    b, _ = plr.calc_loss(th, 1)
+    assert abs(a - b) <= 1e-13 * abs(a)
+
+
+def test_labels_other_than_one_are_class_zero(plr, oracle, gen):
+    # lr.cpp:325 compares labels[i] == 1. exactly; anything else takes the -log(1-h) branch
+    X, y, th = make(gen, 500, 60)
+    y[::7] = 0.5
+    y[::11] = -1.0
+    plr.set_data(X, y)
+    g, loss, _ = plr.loss_grad(th)
+    assert abs(loss - oracle.calc_loss_sum(X, y, th)) <= LOSS_TOL * abs(loss)
+    assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
+
+
+def test_empty_shard(plr):
+    plr.set_data(np.zeros((0, 10)), np.zeros(0))
+    g, loss, n = plr.loss_grad(np.ones(10))
+    assert n == 0 and loss == 0.0
+    np.testing.assert_array_equal(g, np.zeros(10))
+    delta, _ = plr.dgd_delta(np.ones(10), 0.1, 0.1)
+    np.testing.assert_array_equal(np.abs(delta), np.zeros(10))
+    assert plr.predict(np.ones(10)).size == 0
+
+
+def test_errors(plr):
+    from paracel_amd import PlrError
+
+    with pytest.raises(PlrError) as e:
+        plr.loss_grad(np.zeros(0))
+    assert e.value.code == -4  # PLR_ERR_NODATA
+    with pytest.raises(PlrError) as e:
+        plr.alloc_data(10, 20481)
+    assert e.value.code == -5  # PLR_ERR_UNSUPPORTED
+    with pytest.raises(PlrError) as e:
+        plr.alloc_data(10, 0)
+    assert e.value.code == -1
+    plr.set_data(np.ones((4, 3)), np.ones(4))
+    with pytest.raises(ValueError):
+        plr.loss_grad(np.zeros(5))
+    with pytest.raises(PlrError) as e:
+        plr.set_data_chunk(3, np.ones((2, 3)), np.ones(2))
+    assert e.value.code == -1
+
+
+def test_config1_trajectory_100_iterations(plr, oracle, gen):
+    # dense n=100000 d=100, theta0=0, lr=0.1, lam=0.01 => alpha=lr/n, beta=lam/2;
+    # 100 full-batch rounds of read theta -> delta -> theta += delta
+    # (lr.cpp:124-146 with update.cpp:26-32).  theta rel error <= 1e-8.
+    cfg = gen.configs()["c1_dense_100k_x_100"]
+    X, y = cfg.rows(0, cfg.n)
+    plr.set_data(X, y)
+    theta = np.zeros(cfg.d)
+    worst = 0.0
+    for it in range(100):
+        delta, _ = plr.dgd_delta(theta, cfg.alpha, cfg.beta, want_loss=False)
+        if it in (0, 50, 99):
+            worst = max(worst, rel(delta, oracle.dgd_delta(X, y, theta, cfg.alpha, cfg.beta)))
+        theta = theta + delta
+    theta_ref = oracle.train_dgd(X, y, np.zeros(cfg.d), cfg.alpha, cfg.beta, 100)
+    print("per-step delta rel-L2 worst %.3e, theta rel %.3e" % (worst, rel(theta, theta_ref)))
+    assert worst <= GRAD_TOL
+    assert rel(theta, theta_ref) <= 1e-8
+    loss, n = plr.calc_loss(theta)
+    assert abs(loss / n - oracle.calc_loss(X, y, theta_ref)) <= 1e-9
