@@ -1,0 +1,185 @@
+#!/usr/bin/env python3
+"""Benchmark of the worker-side logistic-regression gradient step on one MI355X.
+
+A step is one fused loss+gradient pass (plr_loss_grad through the C ABI) over a
+synthetic shard that is already resident in HBM: theta goes in from the host,
+the gradient sum and the loss come back to the host.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps 50] [--warmup 5] [--workload NAME]
+                    [--no-cpu-baseline] [--rows N]
+
+roofline.achieved = algorithmic bytes per step (X once + y + theta + gradient +
+loss = 8nd + 8n + 16d + 8) / average duration of the streaming kernel, measured
+with HIP events recorded on the library's own stream around that launch.
+cpu_baseline times the CPU oracle's restatement of the reference traversal
+(lr.cpp:132-138, reference data layout) on the host cores of this box, on a
+bounded row sample, scaled linearly in n to the full shard.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
+
+# HBM bytes per launch of the streaming kernel from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs, scaled by what the same counters read for a copy kernel of
+# known size; None until measured for that workload.
+MEASURED_TRAFFIC_BYTES = {
+}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=int(os.environ.get("WORLD_SIZE", "1")))
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2_headline_1m_x_1000")
+    ap.add_argument("--rows", type=int, default=0, help="override n (debugging)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-rows", type=int, default=0)
+    return ap.parse_args()
+
+
+def upload(ctx, cfg, chunk_rows=131072, keep_rows=0):
+    """Generate the shard on the host in row chunks and stream it to HBM.
+    Returns the first keep_rows rows (for the CPU baseline sample)."""
+    import numpy as np
+
+    ctx.alloc_data(cfg.n, cfg.d)
+    keepX, keepy = [], []
+    kept = 0
+    buf = np.empty((min(chunk_rows, cfg.n), cfg.d))  # reused: first touch of fresh pages is slow
+    for lo in range(0, cfg.n, chunk_rows):
+        m = min(chunk_rows, cfg.n - lo)
+        X, y = cfg.rows(lo, m, out=buf[:m])
+        ctx.set_data_chunk(lo, X, y)
+        if kept < keep_rows:
+            t = min(m, keep_rows - kept)
+            keepX.append(X[:t].copy())
+            keepy.append(y[:t].copy())
+            kept += t
+    if keep_rows:
+        return np.concatenate(keepX), np.concatenate(keepy)
+    return None, None
+
+
+def cpu_baseline(cfg, Xs, ys, theta):
+    """Reference traversal on the host cores: 1 core (tool/lr_serial, prun.py -w 1)
+    and P local workers (mpirun -n P bin/lr), on the row sample, scaled to n."""
+    from oracle import oracle
+
+    m = Xs.shape[0]
+    cores = max(1, min(16, os.cpu_count() or 1))
+    t1, _, tl1, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=1, reps=2)
+    tp, _, tlp, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=cores, reps=5)
+    scale = cfg.n / float(m)
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name"):
+                    model = ln.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {
+        "value": 1.0 / (tp * scale),
+        "unit": "steps/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": "first %d of %d rows (d=%d), gradient traversal lr.cpp:132-138 in the "
+                  "reference's vector<vector<double>> layout, g++ -O3, %d threads as local "
+                  "workers; time scaled linearly in n" % (m, cfg.n, cfg.d, cores),
+        "value_1core": 1.0 / (t1 * scale),
+        "loss_pass_seconds_1core_scaled": tl1 * scale,
+        "loss_pass_seconds_pcore_scaled": tlp * scale,
+        "cpu_model": model,
+    }
+
+
+def main():
+    a = parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU's shard: this build has no multi-GPU path "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np  # noqa: F401
+
+    from paracel_amd import Plr
+    from paracel_amd.datagen import gen
+
+    cfgs = gen.configs()
+    if a.workload not in cfgs:
+        print("unknown workload %s; known: %s" % (a.workload, ", ".join(cfgs)), file=sys.stderr)
+        sys.exit(2)
+    cfg = cfgs[a.workload]
+    if a.rows:
+        cfg = cfg.scaled(a.rows)
+    theta = cfg.theta()
+
+    # ~2 GB sample for the CPU leg (bounded: a few seconds per traversal on one core)
+    sample_rows = 0
+    if not a.no_cpu_baseline:
+        sample_rows = a.cpu_sample_rows or max(1, min(cfg.n, int(2.0e9 // (8 * cfg.d))))
+
+    ctx = Plr(0)
+    t0 = time.time()
+    Xs, ys = upload(ctx, cfg, keep_rows=sample_rows)
+    t_up = time.time() - t0
+    print("# shard %d x %d generated and uploaded in %.1f s; %s" %
+          (cfg.n, cfg.d, t_up, ctx.kernel_info()), file=sys.stderr, flush=True)
+
+    for _ in range(a.warmup):
+        ctx.loss_grad(theta)
+    ctx.reset_timing()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        g, loss, n = ctx.loss_grad(theta)   # synchronous: returns after the stream drained
+    elapsed = time.perf_counter() - t0
+    _, kern_ms_sum, launches = ctx.timing()
+    assert launches == a.steps and n == cfg.n
+    kern_ms = kern_ms_sum / launches
+
+    bytes_step = cfg.algorithmic_bytes()
+    achieved = bytes_step / (kern_ms * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name)
+    out = {
+        "metric": "lr_gradient_steps_per_sec",
+        "value": a.steps / elapsed,
+        "unit": "steps/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": 1e3 * elapsed / a.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f64",
+        "data": "synthetic",
+        "config": {"workload": cfg.name, "n": cfg.n, "d": cfg.d,
+                   "step": "plr_loss_grad: theta host->device, fused loss+gradient pass, "
+                           "gsum+loss device->host",
+                   "lambda": cfg.lam, "alpha": cfg.alpha, "beta": cfg.beta,
+                   "kernel": ctx.kernel_info()},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel_ms": kern_ms, "algorithmic_bytes": bytes_step,
+                     "whole_step_gbs": bytes_step / (elapsed / a.steps) / 1e9},
+        "cpu_baseline": None,
+        "loss_mean": loss / n,
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, Xs, ys, theta)
+    ctx.close()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -21,23 +21,32 @@ typedef void (*pass_fn)(PassArgs);
 
 struct Variant {
   int nch, R, wcol, wrow;
-  pass_fn grad, nograd;
+  // [grad][allch]
+  pass_fn fn[2][2];
 };
 
-#define PLR_VARIANT(NCH, R, WCOL, WROW, MINW)                          \
-  {NCH, R, WCOL, WROW, plr::shard_pass<NCH, R, WCOL, WROW, MINW, true>, \
-   plr::shard_pass<NCH, R, WCOL, WROW, MINW, false>}
+#define PLR_VARIANT(NCH, R, WCOL, WROW, MINW)                            \
+  {NCH, R, WCOL, WROW,                                                   \
+   {{plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, false>,            \
+     plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, true>},            \
+    {plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, false>,             \
+     plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, true>}}}
 
-// Ordered by the number of 128-column chunks they cover (wcol * nch).
+// Ordered by the number of 128-column chunks they cover (wcol * nch).  Tile
+// shapes and register budgets (MINW = waves per SIMD the allocation leaves
+// room for) come from sweeps on MI355X: one or two resident waves per SIMD,
+// each with 16-32 KiB of loads in flight, stream fastest; any variant that
+// spills registers loses a third of the bandwidth or more.
 const Variant kVariants[] = {
-    PLR_VARIANT(1, 16, 1, 4, 4),   // d <= 128
-    PLR_VARIANT(2, 16, 1, 4, 2),   // d <= 256
-    PLR_VARIANT(4, 8, 1, 4, 2),    // d <= 512
-    PLR_VARIANT(8, 4, 1, 4, 2),    // d <= 1024
-    PLR_VARIANT(8, 4, 2, 1, 2),    // d <= 2048
-    PLR_VARIANT(8, 4, 4, 1, 2),    // d <= 4096
-    PLR_VARIANT(8, 4, 8, 1, 2),    // d <= 8192
+    PLR_VARIANT(1, 16, 1, 4, 2),   // d <= 128
+    PLR_VARIANT(2, 32, 1, 4, 1),   // d <= 256
+    PLR_VARIANT(4, 8, 1, 4, 1),    // d <= 512
+    PLR_VARIANT(8, 4, 1, 4, 1),    // d <= 1024
+    PLR_VARIANT(4, 4, 4, 1, 2),    // d <= 2048
+    PLR_VARIANT(4, 4, 8, 1, 2),    // d <= 4096
+    PLR_VARIANT(8, 2, 8, 1, 2),    // d <= 8192
     PLR_VARIANT(16, 1, 8, 1, 2),   // d <= 16384
+    PLR_VARIANT(17, 1, 8, 1, 2),   // d <= 17408
     PLR_VARIANT(20, 1, 8, 1, 2),   // d <= 20480
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -63,6 +72,7 @@ struct plr_ctx {
   const Variant* var = nullptr;
   int nch_rt = 0;
   int grid = 0, grid_nograd = 0;
+  bool allch = false;
   int64_t theta_len = 0;
   double* d_theta = nullptr;    // theta_len doubles, zero padded
   double* d_part_g = nullptr;   // grid x pitch
@@ -138,15 +148,16 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   c->var = v;
   c->pitch = pitch;
   c->nch_rt = (int)ceil_div(chunks, v->wcol);
+  c->allch = (chunks == (int64_t)v->nch * v->wcol);
   c->theta_len = (int64_t)v->wcol * c->nch_rt * plr::kChunkCols;
   const int threads = plr::kWave * v->wcol * v->wrow;
   const int64_t ntiles = ceil_div(n, v->R);
   const int64_t want = ceil_div(ntiles, v->wrow);
   int occ = 0, occ_ng = 0;
   PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                 &occ, reinterpret_cast<const void*>(v->grad), threads, 0));
+                 &occ, reinterpret_cast<const void*>(v->fn[1][c->allch]), threads, 0));
   PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                 &occ_ng, reinterpret_cast<const void*>(v->nograd), threads, 0));
+                 &occ_ng, reinterpret_cast<const void*>(v->fn[0][c->allch]), threads, 0));
   if (occ < 1 || occ_ng < 1)
     return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
   int64_t g = (int64_t)c->num_cu * occ, g2 = (int64_t)c->num_cu * occ_ng;
@@ -158,9 +169,9 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   c->grid_nograd = (int)g2;
   char b[256];
   snprintf(b, sizeof b,
-           "shard_pass<NCH=%d,R=%d,WCOL=%d,WROW=%d> nch_rt=%d pitch=%lld grid=%d x %d "
+           "shard_pass<NCH=%d,R=%d,WCOL=%d,WROW=%d,ALLCH=%d> nch_rt=%d pitch=%lld grid=%d x %d "
            "threads (occupancy %d blocks/CU, %d CUs)",
-           v->nch, v->R, v->wcol, v->wrow, c->nch_rt, (long long)pitch, c->grid,
+           v->nch, v->R, v->wcol, v->wrow, (int)c->allch, c->nch_rt, (long long)pitch, c->grid,
            threads, occ, c->num_cu);
   c->info = b;
   return PLR_OK;
@@ -252,7 +263,7 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
   pa.loss_mode = (kind == kPassPredict) ? (unsigned)plr::kLossNone : loss_mode;
 
   PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
-  hipLaunchKernelGGL(grad ? v->grad : v->nograd, dim3(grid), dim3(threads), 0,
+  hipLaunchKernelGGL(v->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
                      c->stream, pa);
   PLR_HIP(c, hipGetLastError());
   PLR_HIP(c, hipEventRecord(c->ev1, c->stream));

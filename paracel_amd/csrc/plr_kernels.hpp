@@ -96,22 +96,44 @@ __host__ __device__ constexpr int lane_of_row(int r) {
 
 // p[r] = this lane's partial dot of row r.  Returns the full 64-lane sum of
 // row row_of_lane<R>(lane); identical bits in every lane holding that row.
+constexpr int ilog2(int v) { return v <= 1 ? 0 : 1 + ilog2(v >> 1); }
+
+// The partials travel in an ext-vector (pure SSA values): with a plain array
+// the compiler folds the lane-dependent selects into dynamically indexed
+// loads and parks the array in scratch memory.
 template <int R>
-__device__ __forceinline__ double reduce_rows(double (&p)[R], int lane) {
+struct RowVec {
+  typedef double type __attribute__((ext_vector_type(R)));
+};
+template <>
+struct RowVec<1> {
+  typedef double type;
+};
+
+template <int R>
+__device__ __forceinline__ double reduce_rows(typename RowVec<R>::type p, int lane) {
+  constexpr int kSteps = ilog2(R);
+  double z;
+  if constexpr (R == 1) {
+    z = p;
+  } else {
 #pragma unroll
-  for (int s = 0, cnt = R / 2; cnt >= 1; ++s, cnt >>= 1) {
-    const int m = 1 << s;
-    const bool up = (lane & m) != 0;
+    for (int s = 0; s < kSteps; ++s) {
+      const int cnt = R >> (s + 1);
+      const int m = 1 << s;
+      const bool up = (lane & m) != 0;
 #pragma unroll
-    for (int k = 0; k < cnt; ++k) {
-      const double send = up ? p[k] : p[k + cnt];
-      const double keep = up ? p[k + cnt] : p[k];
-      p[k] = keep + __shfl_xor(send, m, kWave);
+      for (int k = 0; k < cnt; ++k) {
+        const double lo = p[k], hi = p[k + cnt];
+        const double send = up ? lo : hi;
+        const double keep = up ? hi : lo;
+        p[k] = keep + __shfl_xor(send, m, kWave);
+      }
     }
+    z = p[0];
   }
-  double z = p[0];
 #pragma unroll
-  for (int m = R; m < kWave; m <<= 1) z += __shfl_xor(z, m, kWave);
+  for (int s = kSteps; s < 6; ++s) z += __shfl_xor(z, 1 << s, kWave);
   return z;
 }
 
@@ -170,7 +192,7 @@ __device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_
   }
 
   // ---- per-lane partial dots ----
-  double p[R];
+  typename RowVec<R>::type p;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     double s0 = 0., s1 = 0.;
@@ -179,7 +201,10 @@ __device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_
       s0 = fma(x[r][c].x, th[c].x, s0);
       s1 = fma(x[r][c].y, th[c].y, s1);
     }
-    p[r] = s0 + s1;
+    if constexpr (R == 1)
+      p = s0 + s1;
+    else
+      p[r] = s0 + s1;
   }
   double z = reduce_rows<R>(p, lane);
 
@@ -200,7 +225,7 @@ __device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_
   if (a.loss_mode != kLossNone) {
     double l;
     if (a.loss_mode == kLossReference) {
-      l = (yv == 1.) ? -log(h) : -log(1. - h);
+      l = -log((yv == 1.) ? h : 1. - h);
     } else {
       const double sgn = (yv == 1.) ? -z : z;  // loss = log(1 + exp(sgn))
       l = log1p(exp(-fabs(sgn))) + fmax(sgn, 0.);
@@ -228,7 +253,9 @@ __device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_
 // WROW : independent row groups per workgroup (must be 1 when WCOL > 1)
 // MINW : waves per SIMD the register allocation must leave room for
 // GRAD : accumulate the gradient (false: loss / predict only)
-template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD>
+// ALLCH: the row is exactly WCOL*NCH chunks wide (the last one may be ragged),
+//        so no wave has an unused chunk slot and no load is predicated
+template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD, bool ALLCH>
 __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a) {
   static_assert(WCOL == 1 || WROW == 1, "column-split workgroups own one row group");
   static_assert((R & (R - 1)) == 0 && R <= kWave, "R must be a power of two");
@@ -240,7 +267,7 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   const int64_t chunks = (a.pitch + kChunkCols - 1) / kChunkCols;
   const int64_t slab_c0 = (int64_t)wc * a.nch_rt;          // first chunk of this wave
   int64_t left = chunks - slab_c0;
-  const int my_nch = (int)(left < 0 ? 0 : (left > a.nch_rt ? a.nch_rt : left));
+  const int my_nch = ALLCH ? NCH : (int)(left < 0 ? 0 : (left > a.nch_rt ? a.nch_rt : left));
   const int64_t slab_col0 = slab_c0 * kChunkCols;
   const int64_t col0 = slab_col0 + 2 * lane;
   const uint32_t lane_off = (uint32_t)(2 * lane * sizeof(double));
@@ -256,7 +283,7 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   for (int c = 0; c < NCH; ++c) {
     th[c] = v2d{0., 0.};
     acc[c] = v2d{0., 0.};
-    if (c < a.nch_rt)
+    if (ALLCH || c < a.nch_rt)
       th[c] = *reinterpret_cast<const v2d*>(a.theta + col0 + (int64_t)c * kChunkCols);
   }
   double loss_acc = 0.;
@@ -268,27 +295,21 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   const int64_t ngroups = (int64_t)gridDim.x * WROW;
   const int64_t nfull = a.n / R;  // tiles with all R rows present
 
-  auto run_tiles = [&](auto allch) {
-    constexpr bool ALLCH = decltype(allch)::value;
-    int parity = 0;
-    for (int64_t tile = group; tile < a.ntiles; tile += ngroups, parity ^= 1) {
-      const int64_t row0 = tile * R;
-      const double* tile_base = a.X + row0 * a.pitch + slab_col0;
-      double* zbuf = zx + ((WCOL > 1) ? parity * (WCOL * R) : 0);
-      if (tile < nfull)
-        tile_step<NCH, R, WCOL, GRAD, true, ALLCH>(a, tile_base, row0, lane_off, lane, wc,
-                                                   my_nch, ragged_c, lane_in_ragged, my_row,
-                                                   th, acc, loss_acc, zbuf);
-      else
-        tile_step<NCH, R, WCOL, GRAD, false, ALLCH>(a, tile_base, row0, lane_off, lane, wc,
-                                                    my_nch, ragged_c, lane_in_ragged, my_row,
-                                                    th, acc, loss_acc, zbuf);
-    }
-  };
-  if (my_nch == NCH)
-    run_tiles(std::true_type{});
-  else
-    run_tiles(std::false_type{});
+  // full tiles, then the one partial tile of the shard (if this row group
+  // is the one it falls to)
+  int parity = 0;
+  int64_t tile = group;
+#pragma clang loop unroll(disable)
+  for (; tile < nfull; tile += ngroups, parity ^= 1)
+    tile_step<NCH, R, WCOL, GRAD, true, ALLCH>(
+        a, a.X + tile * R * a.pitch + slab_col0, tile * R, lane_off, lane, wc, my_nch,
+        ragged_c, lane_in_ragged, my_row, th, acc, loss_acc,
+        zx + ((WCOL > 1) ? parity * (WCOL * R) : 0));
+  if (tile < a.ntiles)
+    tile_step<NCH, R, WCOL, GRAD, false, ALLCH>(
+        a, a.X + tile * R * a.pitch + slab_col0, tile * R, lane_off, lane, wc, my_nch,
+        ragged_c, lane_in_ragged, my_row, th, acc, loss_acc,
+        zx + ((WCOL > 1) ? parity * (WCOL * R) : 0));
 
   // ---- combine the workgroup's partials in a fixed order ----
   if (GRAD) {

@@ -119,8 +119,10 @@ class Config:
             return np.zeros(self.d)
         return self.theta_star()
 
-    def rows(self, row0, nrows, threads=None):
-        X = gen_X(self.spec, row0, nrows, self.d, threads)
+    def rows(self, row0, nrows, threads=None, out=None):
+        """Rows [row0, row0+nrows) of the shard and their labels.  `out` (a
+        C-contiguous nrows x d array) is filled in place when given."""
+        X = gen_X(self.spec, row0, nrows, self.d, threads, out=out)
         y = gen_labels(self.spec, row0, X, self.theta_star(), threads)
         return X, y
 
