@@ -31,6 +31,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # WRITE_SIZE runs, scaled by what the same counters read for a copy kernel of
 # known size; None until measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
+    # FETCH_SIZE 3932597.4 x 2.000 KiB + WRITE_SIZE 2008.0 x 1.000 KiB per dispatch
+    "c2_headline_1m_x_1000": 8056015667,
 }
 
 

@@ -43,5 +43,13 @@ def build_libplr_gen():
     return out
 
 
+def build_copy_probe():
+    """Plain device copy of known size (counter calibration) -> paracel_amd/copy_probe"""
+    out = os.path.join(_HERE, "copy_probe")
+    flags = [f for f in HIPCC_FLAGS if f not in ("-fPIC", "-shared")]
+    _run([hipcc()] + flags + ["-o", out, os.path.join(_HERE, "csrc", "copy_probe.hip")])
+    return out
+
+
 def build_all():
-    return [build_libplr(), build_libplr_gen()]
+    return [build_libplr(), build_libplr_gen(), build_copy_probe()]
