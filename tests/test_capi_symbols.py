@@ -1,0 +1,43 @@
+"""The C-ABI library loads and exports exactly what include/plr.h declares
+(no compute calls: this runs without a GPU)."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "plr.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(plr_[a-z_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    from paracel_amd import capi
+
+    assert declared_symbols() == sorted(name for name, _, _ in capi.SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol():
+    from paracel_amd import capi
+
+    lib = ctypes.CDLL(capi.lib_path())
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+    loaded = capi.load_library()
+    assert loaded.plr_version().decode().startswith("plr ")
+    assert loaded.plr_last_error(None) is not None
+
+
+def test_product_does_not_touch_the_oracle():
+    # the oracle is test infrastructure: nothing under paracel_amd/ or include/ may
+    # import, link or load it
+    bad = []
+    for base in ("paracel_amd", "include"):
+        for dp, _, files in os.walk(os.path.join(ROOT, base)):
+            for f in files:
+                if f.endswith((".py", ".hip", ".hpp", ".h", ".c", ".cpp")):
+                    if "oracle" in open(os.path.join(dp, f), errors="ignore").read():
+                        bad.append(os.path.join(dp, f))
+    assert not bad, bad

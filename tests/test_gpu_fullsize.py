@@ -1,0 +1,80 @@
+"""Full-size shards of the benchmark configurations, checked through
+size-independent properties: the shard is streamed to HBM chunk by chunk and,
+per chunk, a library-routine reference (numpy BLAS GEMV + scipy expit /
+logaddexp, fp64) of the chunk's gradient and loss is accumulated on the host --
+shard additivity then fixes the full-size answer.  The CPU oracle itself is
+used on a leading slab only (it is a scalar loop).
+
+Tolerance: relative L2 <= 1e-10 on the gradient, relative 1e-10 on the stable
+loss, 1e-9 on the reference-formula loss (it amplifies the last-bit difference
+between device and host exp by 1/(1-h)).
+"""
+import numpy as np
+import pytest
+from scipy.special import expit
+
+pytestmark = pytest.mark.gpu
+
+
+def rel(a, b):
+    return np.linalg.norm(a - b) / np.linalg.norm(b)
+
+
+def stream_and_reference(plr, cfg, theta, slab_rows=0):
+    d = cfg.d
+    chunk = max(1, int(1.0e9 // (8 * d)))
+    plr.alloc_data(cfg.n, d)
+    buf = np.empty((min(chunk, cfg.n), d))
+    g = np.zeros(d)
+    g0 = np.zeros(d)
+    loss = 0.0
+    slabX = slaby = None
+    for lo in range(0, cfg.n, chunk):
+        m = min(chunk, cfg.n - lo)
+        X, y = cfg.rows(lo, m, out=buf[:m])
+        plr.set_data_chunk(lo, X, y)
+        z = X @ theta
+        g += X.T @ (expit(z) - y)
+        g0 += X.T @ (0.5 - y)
+        loss += np.sum(np.logaddexp(0.0, np.where(y == 1.0, -z, z)))
+        if lo == 0 and slab_rows:
+            slabX, slaby = X[:slab_rows].copy(), y[:slab_rows].copy()
+    return g, g0, loss, slabX, slaby
+
+
+FULL = ["c2_headline_1m_x_1000", "c3_tall_10m_x_256", "c4_wide_200k_x_16384",
+        "c4b_wide_200k_x_16385", "c5_e2e_2m_x_512"]
+
+
+@pytest.mark.parametrize("name", FULL)
+def test_full_size_shard(plr, oracle, gen, name):
+    cfg = gen.configs()[name]
+    theta = cfg.theta_star()
+    print("case %s n=%d d=%d" % (name, cfg.n, cfg.d), flush=True)
+    slab = max(64, int(4.0e6 // cfg.d))
+    g_ref, g0_ref, loss_ref, Xs, ys = stream_and_reference(plr, cfg, theta, slab)
+    print(plr.kernel_info(), flush=True)
+
+    g, loss_naive, n = plr.loss_grad(theta, 0)
+    assert n == cfg.n
+    assert rel(g, g_ref) <= 1e-10
+    assert abs(loss_naive - loss_ref) <= 1e-9 * loss_ref
+    g2, loss_stable, _ = plr.loss_grad(theta, 1)
+    np.testing.assert_array_equal(g, g2)            # bitwise reproducible, loss mode aside
+    assert abs(loss_stable - loss_ref) <= 1e-10 * loss_ref
+
+    # theta = 0: gsum = X^T (1/2 - y) (plain GEMV), loss = n ln 2
+    gz, lz, _ = plr.loss_grad(np.zeros(cfg.d), 0)
+    assert rel(gz, g0_ref) <= 1e-12
+    assert abs(lz - cfg.n * np.log(2.0)) <= 1e-12 * cfg.n
+
+    # delta in the reference's signs and scaling: -alpha gsum - 2 alpha beta n theta
+    delta, _ = plr.dgd_delta(theta, cfg.alpha, cfg.beta, want_loss=False)
+    assert rel(delta, -cfg.alpha * g_ref - 2 * cfg.alpha * cfg.beta * cfg.n * theta) <= 1e-10
+
+    # the CPU oracle on a leading slab, same device code path (re-uploaded as its own shard)
+    plr.set_data(Xs, ys)
+    gs, ls, _ = plr.loss_grad(theta, 0)
+    assert rel(gs, oracle.gsum(Xs, ys, theta)) <= 1e-10
+    want = oracle.calc_loss_sum(Xs, ys, theta)
+    assert abs(ls - want) <= 1e-9 * want
