@@ -220,9 +220,13 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
   if (row0 < 0 || nrows < 0 || row0 + nrows > c->n)
     return fail(c, PLR_ERR_INVALID, "row range outside the reserved shard");
   PLR_HIP(c, hipSetDevice(c->device));
-  PLR_HIP(c, hipMemcpy2D(c->dX + row0 * c->pitch, (size_t)c->pitch * sizeof(double), X,
-                         (size_t)ldx * sizeof(double), (size_t)c->d * sizeof(double),
-                         (size_t)nrows, hipMemcpyHostToDevice));
+  if (ldx == c->pitch)  // same pitch on both sides: one linear copy
+    PLR_HIP(c, hipMemcpy(c->dX + row0 * c->pitch, X,
+                         (size_t)nrows * c->pitch * sizeof(double), hipMemcpyHostToDevice));
+  else
+    PLR_HIP(c, hipMemcpy2D(c->dX + row0 * c->pitch, (size_t)c->pitch * sizeof(double), X,
+                           (size_t)ldx * sizeof(double), (size_t)c->d * sizeof(double),
+                           (size_t)nrows, hipMemcpyHostToDevice));
   PLR_HIP(c, hipMemcpy(c->dy + row0, y, (size_t)nrows * sizeof(double),
                        hipMemcpyHostToDevice));
   return PLR_OK;
