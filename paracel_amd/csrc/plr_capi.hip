@@ -21,16 +21,17 @@ typedef void (*pass_fn)(PassArgs);
 
 struct Variant {
   int nch, R, wcol, wrow;
+  bool thl;
   // [grad][allch]
   pass_fn fn[2][2];
 };
 
-#define PLR_VARIANT(NCH, R, WCOL, WROW, MINW)                            \
-  {NCH, R, WCOL, WROW,                                                   \
-   {{plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, false>,            \
-     plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, true>},            \
-    {plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, false>,             \
-     plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, true>}}}
+#define PLR_VARIANT(NCH, R, WCOL, WROW, MINW, THL)                         \
+  {NCH, R, WCOL, WROW, THL,                                                \
+   {{plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, false, THL>,         \
+     plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, true, THL>},         \
+    {plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, false, THL>,          \
+     plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, true, THL>}}}
 
 // Ordered by the number of 128-column chunks they cover (wcol * nch).  Tile
 // shapes and register budgets (MINW = waves per SIMD the allocation leaves
@@ -38,19 +39,19 @@ struct Variant {
 // each with 16-32 KiB of loads in flight, stream fastest; any variant that
 // spills registers loses a third of the bandwidth or more.
 const Variant kVariants[] = {
-    PLR_VARIANT(1, 16, 1, 4, 2),   // d <= 128
-    PLR_VARIANT(2, 32, 1, 4, 1),   // d <= 256
-    PLR_VARIANT(4, 8, 1, 4, 1),    // d <= 512
-    PLR_VARIANT(8, 4, 1, 4, 1),    // d <= 1024
-    PLR_VARIANT(4, 4, 4, 1, 2),    // d <= 2048
-    PLR_VARIANT(4, 4, 8, 1, 2),    // d <= 4096
-    PLR_VARIANT(8, 2, 8, 1, 2),    // d <= 8192
-    PLR_VARIANT(16, 1, 8, 1, 2),   // d <= 16384
-    PLR_VARIANT(17, 1, 8, 1, 2),   // d <= 17408
-    PLR_VARIANT(20, 1, 8, 1, 2),   // d <= 20480
+    PLR_VARIANT(1, 16, 1, 4, 2, false),   // d <= 128
+    PLR_VARIANT(2, 32, 1, 4, 1, false),   // d <= 256
+    PLR_VARIANT(4, 8, 1, 4, 1, false),    // d <= 512
+    PLR_VARIANT(8, 4, 1, 4, 1, false),    // d <= 1024
+    PLR_VARIANT(2, 8, 8, 1, 2, false),    // d <= 2048
+    PLR_VARIANT(4, 4, 8, 1, 2, false),    // d <= 4096
+    PLR_VARIANT(8, 4, 8, 1, 2, true),     // d <= 8192
+    PLR_VARIANT(16, 1, 8, 1, 2, true),    // d <= 16384
+    PLR_VARIANT(17, 1, 8, 1, 2, true),    // d <= 17408
+    PLR_VARIANT(19, 1, 8, 1, 2, true),    // d <= 19456 (152 KiB of theta in LDS)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
-constexpr int64_t kMaxCols = 20480;
+constexpr int64_t kMaxCols = 19456;
 
 std::string g_create_error;
 
@@ -136,7 +137,9 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
     return fail(c, PLR_ERR_UNSUPPORTED,
                 "d = " + std::to_string(d) + " exceeds the widest kernel variant (" +
                     std::to_string(kMaxCols) + " columns)");
-  const int64_t pitch = (d + 1) & ~int64_t(1);
+  // even pitch so that every row start is 16-byte aligned; wide rows are
+  // aligned to 128 B (<= 0.7 % more bytes, +3 % bandwidth when d is odd)
+  const int64_t pitch = (d >= 2048) ? ((d + 15) & ~int64_t(15)) : ((d + 1) & ~int64_t(1));
   const int64_t chunks = ceil_div(pitch, plr::kChunkCols);
   const Variant* v = nullptr;
   for (int i = 0; i < kNumVariants; ++i)

@@ -151,18 +151,23 @@ __device__ __forceinline__ double wave_sum(double v) {
   return v;
 }
 
-// One tile of R rows: loads, dots, lane reduction, sigmoid/residual/loss,
-// rank-1 update.  FULL = every row of the tile exists (no row predication).
-// ALLCH = the wave uses all NCH chunks (no per-chunk predication).
-template <int NCH, int R, int WCOL, bool GRAD, bool FULL, bool ALLCH>
-__device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_base,
-                                          int64_t row0, uint32_t lane_off, int lane,
-                                          int wc, int my_nch, int ragged_c,
-                                          bool lane_in_ragged, int my_row,
-                                          const v2d (&th)[NCH], v2d (&acc)[NCH],
-                                          double& loss_acc, double* zbuf) {
-  // ---- issue every load of the tile (uniform base + 32-bit lane offset) ----
-  v2d x[R][NCH];
+// Per-wave constants of one pass.
+struct WaveCtx {
+  int lane;
+  int wc;             // column slab of this wave within the workgroup
+  int my_nch;         // chunks this wave really owns
+  int ragged_c;       // its chunk that straddles the row end, or -1
+  bool lane_in_ragged;
+  int my_row;         // row of the tile whose dot product ends up in this lane
+  uint32_t lane_off;  // byte offset of this lane inside a chunk
+};
+
+// Issue every load of one tile of R rows (uniform base + 32-bit lane offset).
+// FULL = every row of the tile exists; ALLCH = the wave uses all NCH chunks.
+template <int NCH, int R, bool FULL, bool ALLCH>
+__device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
+                                          const double* tile_base, int64_t row0,
+                                          v2d (&x)[R][NCH], double& yv) {
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const char* rowp = reinterpret_cast<const char*>(tile_base + (int64_t)r * a.pitch);
@@ -170,50 +175,70 @@ __device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       x[r][c] = v2d{0., 0.};
-      if (rv && (ALLCH || c < my_nch))  // uniform
+      if (rv && (ALLCH || c < w.my_nch))  // uniform
         x[r][c] = load_x(reinterpret_cast<const v2d*>(
-            rowp + lane_off + (uint32_t)(c * kChunkCols * sizeof(double))));
+            rowp + w.lane_off + (uint32_t)(c * kChunkCols * sizeof(double))));
     }
   }
-  const int64_t myrow_g = row0 + my_row;
+  yv = 0.;
+  if ((FULL || row0 + w.my_row < a.n) && a.y) yv = a.y[row0 + w.my_row];
+}
+
+// Everything that happens on a loaded tile: dots, lane reduction,
+// sigmoid/residual/loss, rank-1 update of the gradient slab.
+// THL: theta is read from the wave's LDS slab (thl) instead of registers.
+template <int NCH, int R, int WCOL, bool GRAD, bool FULL, bool THL>
+__device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w,
+                                             int64_t row0, v2d (&x)[R][NCH], double yv,
+                                             const v2d (&th)[NCH], const v2d* thl,
+                                             v2d (&acc)[NCH], double& loss_acc,
+                                             double* zbuf) {
+  const int lane = w.lane;
+  const int64_t myrow_g = row0 + w.my_row;
   const bool my_valid = FULL || myrow_g < a.n;
-  double yv = 0.;
-  if (my_valid && a.y) yv = a.y[myrow_g];
 
   // lanes past the end of the row in the ragged last chunk hold the next
   // row's (or slack) bytes: zero them so they cannot poison the dot product
-  if (ragged_c >= 0) {
+  if (w.ragged_c >= 0) {
 #pragma unroll
     for (int c = 0; c < NCH; ++c)
-      if (c == ragged_c) {
+      if (c == w.ragged_c) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) x[r][c] = lane_in_ragged ? x[r][c] : v2d{0., 0.};
+        for (int r = 0; r < R; ++r) x[r][c] = w.lane_in_ragged ? x[r][c] : v2d{0., 0.};
       }
   }
 
   // ---- per-lane partial dots ----
   typename RowVec<R>::type p;
+  {
+    double s0[R], s1[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    double s0 = 0., s1 = 0.;
+    for (int r = 0; r < R; ++r) s0[r] = s1[r] = 0.;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
-      s0 = fma(x[r][c].x, th[c].x, s0);
-      s1 = fma(x[r][c].y, th[c].y, s1);
+      const v2d t = THL ? thl[c * kWave] : th[c];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        s0[r] = fma(x[r][c].x, t.x, s0[r]);
+        s1[r] = fma(x[r][c].y, t.y, s1[r]);
+      }
     }
-    if constexpr (R == 1)
-      p = s0 + s1;
-    else
-      p[r] = s0 + s1;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if constexpr (R == 1)
+        p = s0[r] + s1[r];
+      else
+        p[r] = s0[r] + s1[r];
+    }
   }
   double z = reduce_rows<R>(p, lane);
 
   if (WCOL > 1) {
-    if (lane < R) zbuf[wc * R + my_row] = z;
+    if (lane < R) zbuf[w.wc * R + w.my_row] = z;
     __syncthreads();
     double s = 0.;
 #pragma unroll
-    for (int w = 0; w < WCOL; ++w) s += zbuf[w * R + my_row];
+    for (int k = 0; k < WCOL; ++k) s += zbuf[k * R + w.my_row];
     z = s;
   }
 
@@ -221,7 +246,7 @@ __device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_
   const double e = exp(-z);
   const double h = 1. / (1. + e);
   const double res = my_valid ? (h - yv) : 0.;
-  if (a.h_out && my_valid && lane < R && wc == 0) a.h_out[myrow_g] = h;
+  if (a.h_out && my_valid && lane < R && w.wc == 0) a.h_out[myrow_g] = h;
   if (a.loss_mode != kLossNone) {
     double l;
     if (a.loss_mode == kLossReference) {
@@ -230,7 +255,7 @@ __device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_
       const double sgn = (yv == 1.) ? -z : z;  // loss = log(1 + exp(sgn))
       l = log1p(exp(-fabs(sgn))) + fmax(sgn, 0.);
     }
-    if (my_valid && lane < R && wc == 0) loss_acc += l;
+    if (my_valid && lane < R && w.wc == 0) loss_acc += l;
   }
 
   // ---- rank-1 update of the gradient slab from the same registers ----
@@ -255,7 +280,9 @@ __device__ __forceinline__ void tile_step(const PassArgs& a, const double* tile_
 // GRAD : accumulate the gradient (false: loss / predict only)
 // ALLCH: the row is exactly WCOL*NCH chunks wide (the last one may be ragged),
 //        so no wave has an unused chunk slot and no load is predicated
-template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD, bool ALLCH>
+// THL  : theta lives in LDS (one slab per wave) instead of registers -- for
+//        wide rows, where theta + accumulators + tile would not fit
+template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD, bool ALLCH, bool THL>
 __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a) {
   static_assert(WCOL == 1 || WROW == 1, "column-split workgroups own one row group");
   static_assert((R & (R - 1)) == 0 && R <= kWave, "R must be a power of two");
@@ -270,46 +297,64 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   const int my_nch = ALLCH ? NCH : (int)(left < 0 ? 0 : (left > a.nch_rt ? a.nch_rt : left));
   const int64_t slab_col0 = slab_c0 * kChunkCols;
   const int64_t col0 = slab_col0 + 2 * lane;
-  const uint32_t lane_off = (uint32_t)(2 * lane * sizeof(double));
   // the chunk that straddles the end of the row, if this wave owns it
   const int tail_cols = (int)(a.pitch % kChunkCols);
   const int ragged_c = (tail_cols != 0 && slab_c0 + my_nch == chunks && my_nch > 0)
                            ? my_nch - 1 : -1;
   const bool lane_in_ragged = 2 * lane < tail_cols;
+  WaveCtx w;
+  w.lane = lane;
+  w.wc = wc;
+  w.my_nch = my_nch;
+  w.ragged_c = ragged_c;
+  w.lane_in_ragged = lane_in_ragged;
+  w.my_row = row_of_lane<R>(lane & (R - 1));
+  w.lane_off = (uint32_t)(2 * lane * sizeof(double));
 
-  // theta slab -> registers (theta is zero-padded on the device)
-  v2d th[NCH], acc[NCH];
+  // theta slab -> registers, or -> this wave's private LDS slab (theta is
+  // zero-padded on the device)
+  __shared__ v2d th_lds[THL ? WCOL * WROW * NCH * kWave : 1];
+  v2d* thl = th_lds + (THL ? (wave * NCH * kWave + lane) : 0);
+  v2d thr[NCH], acc[NCH];  // thr is dead (and eliminated) when THL
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
-    th[c] = v2d{0., 0.};
+    v2d t = v2d{0., 0.};
     acc[c] = v2d{0., 0.};
     if (ALLCH || c < a.nch_rt)
-      th[c] = *reinterpret_cast<const v2d*>(a.theta + col0 + (int64_t)c * kChunkCols);
+      t = *reinterpret_cast<const v2d*>(a.theta + col0 + (int64_t)c * kChunkCols);
+    if (THL) thl[c * kWave] = t;
+    thr[c] = t;
   }
   double loss_acc = 0.;
 
   __shared__ double zx[(WCOL > 1) ? 2 * WCOL * R : 1];
 
-  const int my_row = row_of_lane<R>(lane & (R - 1));
   const int64_t group = (int64_t)blockIdx.x * WROW + wr;
   const int64_t ngroups = (int64_t)gridDim.x * WROW;
   const int64_t nfull = a.n / R;  // tiles with all R rows present
+  const int64_t tile_stride = (int64_t)R * a.pitch;
+  const double* xbase = a.X + slab_col0;
+  constexpr int kZ = (WCOL > 1) ? WCOL * R : 0;
 
   // full tiles, then the one partial tile of the shard (if this row group
   // is the one it falls to)
-  int parity = 0;
   int64_t tile = group;
+  int par = 0;  // which half of zx the next tile uses (alternates per tile)
 #pragma clang loop unroll(disable)
-  for (; tile < nfull; tile += ngroups, parity ^= 1)
-    tile_step<NCH, R, WCOL, GRAD, true, ALLCH>(
-        a, a.X + tile * R * a.pitch + slab_col0, tile * R, lane_off, lane, wc, my_nch,
-        ragged_c, lane_in_ragged, my_row, th, acc, loss_acc,
-        zx + ((WCOL > 1) ? parity * (WCOL * R) : 0));
-  if (tile < a.ntiles)
-    tile_step<NCH, R, WCOL, GRAD, false, ALLCH>(
-        a, a.X + tile * R * a.pitch + slab_col0, tile * R, lane_off, lane, wc, my_nch,
-        ragged_c, lane_in_ragged, my_row, th, acc, loss_acc,
-        zx + ((WCOL > 1) ? parity * (WCOL * R) : 0));
+  for (; tile < nfull; tile += ngroups, par ^= 1) {
+    v2d x[R][NCH];
+    double yv;
+    load_tile<NCH, R, true, ALLCH>(a, w, xbase + tile * tile_stride, tile * R, x, yv);
+    compute_tile<NCH, R, WCOL, GRAD, true, THL>(a, w, tile * R, x, yv, thr, thl, acc,
+                                                loss_acc, zx + par * kZ);
+  }
+  if (tile < a.ntiles) {
+    v2d x[R][NCH];
+    double yv;
+    load_tile<NCH, R, false, ALLCH>(a, w, xbase + tile * tile_stride, tile * R, x, yv);
+    compute_tile<NCH, R, WCOL, GRAD, false, THL>(a, w, tile * R, x, yv, thr, thl, acc,
+                                                 loss_acc, zx + par * kZ);
+  }
 
   // ---- combine the workgroup's partials in a fixed order ----
   if (GRAD) {

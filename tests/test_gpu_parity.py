@@ -29,13 +29,13 @@ def make(gen, n, d, seed=0xABCD, scale=None, theta_scale=1.0):
 
 
 # every kernel variant (d <= 128, 256, 512, 1024, 2048, 4096, 8192, 16384,
-# 20480), widths that are not multiples of the 128-column chunk or of 2, and
+# 19456), widths that are not multiples of the 128-column chunk or of 2, and
 # row counts around the tile sizes
 SHAPES = [
     (1, 1), (5, 2), (7, 3), (64, 17), (300, 64), (1000, 100), (257, 127), (1030, 128),
     (515, 129), (1000, 255), (4099, 256), (333, 257), (1001, 512), (2051, 1000),
     (700, 1024), (300, 1025), (260, 2047), (130, 4097), (70, 8193), (40, 16384),
-    (37, 16385), (21, 20480),
+    (37, 16385), (21, 19456),
 ]
 
 
@@ -232,7 +232,7 @@ def test_errors(plr):
         plr.loss_grad(np.zeros(0))
     assert e.value.code == -4  # PLR_ERR_NODATA
     with pytest.raises(PlrError) as e:
-        plr.alloc_data(10, 20481)
+        plr.alloc_data(10, 19457)
     assert e.value.code == -5  # PLR_ERR_UNSUPPORTED
     with pytest.raises(PlrError) as e:
         plr.alloc_data(10, 0)
