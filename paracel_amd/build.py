@@ -51,5 +51,12 @@ def build_copy_probe():
     return out
 
 
+def build_worker():
+    """Host side of the worker path (g++): parameter-server process, reducer
+    plugin, GPU LR worker -> paracel_amd/{plr_ps_server,liblr_update.so,plr_lr_worker}"""
+    _run(["make", "-B", "-C", os.path.join(_HERE, "worker")])
+    return [os.path.join(_HERE, f) for f in ("plr_ps_server", "liblr_update.so", "plr_lr_worker")]
+
+
 def build_all():
-    return [build_libplr(), build_libplr_gen(), build_copy_probe()]
+    return [build_libplr(), build_libplr_gen(), build_copy_probe()] + build_worker()

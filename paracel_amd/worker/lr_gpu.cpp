@@ -1,0 +1,195 @@
+#include "lr_gpu.hpp"
+
+#include <stdlib.h>
+
+#include <chrono>
+#include <iostream>
+#include <stdexcept>
+
+namespace plr_ps {
+
+logistic_regression_gpu::logistic_regression_gpu(
+    const std::string& hosts_dct_str, const std::string& _input, const std::string& output,
+    const std::string& update_file_name, const std::string& update_func_name,
+    const std::string& method, int _rounds, double _alpha, double _beta, bool _debug,
+    int device_id)
+    : paralg(hosts_dct_str, output, _rounds),
+      input(_input),
+      update_file(update_file_name),
+      update_func(update_func_name),
+      learning_method(method),
+      worker_id((int)get_worker_id()),
+      rounds(_rounds),
+      alpha(_alpha),
+      beta(_beta),
+      debug(_debug) {
+  check(plr_create(&gpu, device_id), "plr_create");
+}
+
+logistic_regression_gpu::~logistic_regression_gpu() { plr_destroy(gpu); }
+
+void logistic_regression_gpu::check(int rc, const char* what) {
+  if (rc != PLR_OK)
+    throw std::runtime_error(std::string(what) + ": " + plr_last_error(gpu));
+}
+
+void logistic_regression_gpu::local_parser(const std::vector<std::string>& linelst, char sep) {
+  flat.clear();
+  labels.clear();
+  n_local = 0;
+  data_dim = 0;
+  std::vector<double> row;
+  for (const std::string& line : linelst) {
+    row.clear();
+    row.push_back(1.);  // bias column
+    size_t st = 0;
+    std::vector<double> fields;
+    for (;;) {  // str_split: empty fields are dropped (ext_utility.hpp:38-50)
+      const size_t en = line.find(sep, st);
+      const std::string tok = line.substr(st, en == std::string::npos ? en : en - st);
+      if (!tok.empty()) fields.push_back(std::stod(tok));
+      if (en == std::string::npos) break;
+      st = en + 1;
+    }
+    if (fields.empty()) throw std::invalid_argument("empty sample line");
+    for (size_t i = 0; i + 1 < fields.size(); ++i) row.push_back(fields[i]);
+    if (data_dim == 0) data_dim = (int64_t)row.size();
+    if ((int64_t)row.size() != data_dim) throw std::invalid_argument("ragged sample line");
+    flat.insert(flat.end(), row.begin(), row.end());
+    labels.push_back(fields.back());
+    ++n_local;
+  }
+  if (kdim == 0 && data_dim > 0) kdim = (int)data_dim - 1;
+}
+
+void logistic_regression_gpu::set_samples(const double* X, int64_t n, int64_t d, int64_t ldx,
+                                          const double* y) {
+  n_local = n;
+  data_dim = d;
+  check(plr_set_data(gpu, X, n, d, ldx, y), "plr_set_data");
+  flat.clear();
+  labels.clear();
+}
+
+void logistic_regression_gpu::upload() {
+  check(plr_set_data(gpu, flat.data(), n_local, data_dim, data_dim, labels.data()),
+        "plr_set_data");
+  std::vector<double>().swap(flat);
+  std::vector<double>().swap(labels);
+}
+
+void logistic_regression_gpu::dgd_learning() {
+  if (theta0.empty()) {  // random_double_list(data_dim): U(0,1) from libc random()
+    for (int64_t i = 0; i < data_dim; ++i) {
+      double v = random() / static_cast<double>(RAND_MAX);
+      while (v == 0 || v == 1.) v = random() / static_cast<double>(RAND_MAX);
+      theta0.push_back(v);
+    }
+  }
+  if ((int64_t)theta0.size() != data_dim) throw std::invalid_argument("theta0 has the wrong length");
+  theta = theta0;
+  paracel_write("theta", theta);  // first push
+  paracel_register_bupdate(update_file, update_func);
+  std::vector<double> delta(data_dim);
+  const auto t0 = std::chrono::steady_clock::now();
+  for (int rd = 0; rd < rounds; ++rd) {
+    theta = paracel_read<std::vector<double> >("theta");
+    // lr.cpp:125-142 in one fused pass over the resident shard; with debug the
+    // round's loss at the theta just read is recorded (the reference records
+    // it after every sample, an O(n^2 d) loop)
+    double loss_sum = 0.;
+    check(plr_dgd_delta(gpu, theta.data(), alpha, beta, delta.data(),
+                        debug ? &loss_sum : nullptr),
+          "plr_dgd_delta");
+    if (debug) loss_error.push_back(n_local ? loss_sum / (double)n_local : 0.);
+    paracel_sync();
+    paracel_bupdate("theta", delta);
+    paracel_sync();
+    if (debug || rounds <= 10)
+      std::cout << "worker" << get_worker_id() << " finished round: " << rd << std::endl;
+  }
+  round_sec += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  theta = paracel_read<std::vector<double> >("theta");  // last pull
+}
+
+void logistic_regression_gpu::solve() {
+  if (!input.empty()) {
+    auto lines = paracel_load(input);
+    local_parser(lines);
+    upload();
+  }
+  paracel_sync();
+  if (learning_method == "dgd") {
+    dgd_learning();
+  } else {
+    // ipm/downpour/agd update theta inside the row loop (lr.cpp:179-182,...):
+    // a serial dependence between rows, not a batch gradient
+    std::cerr << "method do not support" << std::endl;
+  }
+  paracel_sync();
+}
+
+double logistic_regression_gpu::calc_loss() {
+  double loss = 0.;
+  int64_t cnt = 0;
+  check(plr_calc_loss(gpu, theta.data(), &loss, &cnt, PLR_LOSS_REFERENCE), "plr_calc_loss");
+  allreduce(loss);  // lr.cpp:331-334
+  int sz = (int)cnt;
+  allreduce(sz);
+  return loss / static_cast<double>(sz);
+}
+
+void logistic_regression_gpu::dump_result() {
+  if (worker_id == 0) {
+    paracel_dump_vector(theta, "lr_theta_", "|");
+    if (debug) paracel_dump_vector(loss_error, "lr_loss_error_", "\n");
+  }
+  if (!pred_h.empty()) paracel_dump_vector(pred_h, "pred_v_", "\n");
+}
+
+void logistic_regression_gpu::test(const std::string& test_fn) {
+  auto lines = paracel_load(test_fn);
+  local_parser(lines);
+  upload();
+  std::cout << "loss in test dataset is: " << calc_loss() << std::endl;
+  paracel_sync();
+}
+
+void logistic_regression_gpu::predict(const std::string& pred_fn) {
+  // lr.cpp:95-107: "f1,...,fk,..." -> [1.0, f1..fk]; no label
+  auto lines = paracel_load(pred_fn);
+  flat.clear();
+  labels.clear();
+  n_local = 0;
+  for (const std::string& line : lines) {
+    flat.push_back(1.);
+    size_t st = 0;
+    int got = 0;
+    while (got < kdim) {
+      const size_t en = line.find(',', st);
+      const std::string tok = line.substr(st, en == std::string::npos ? en : en - st);
+      if (!tok.empty()) {
+        flat.push_back(std::stod(tok));
+        ++got;
+      }
+      if (en == std::string::npos) break;
+      st = en + 1;
+    }
+    if (got != kdim) throw std::invalid_argument("predict line has too few fields");
+    labels.push_back(0.);
+    ++n_local;
+  }
+  data_dim = kdim + 1;
+  upload();
+  pred_h.assign(n_local, 0.);
+  check(plr_predict(gpu, theta.data(), pred_h.data()), "plr_predict");
+  paracel_sync();
+}
+
+double logistic_regression_gpu::gpu_kernel_ms() const {
+  double sum = 0.;
+  plr_get_timing(gpu, nullptr, &sum, nullptr);
+  return sum;
+}
+
+}  // namespace plr_ps

@@ -1,0 +1,230 @@
+// The slice of Paracel's worker API (class paralg, reference include/ps.hpp)
+// that the logistic-regression worker uses, with the same method names,
+// argument meaning and error behaviour, on top of a client that speaks the
+// reference's ZeroMQ/msgpack protocol (include/client.hpp).  One worker
+// process, one thread; REQ sockets are created lazily per op family and
+// strictly alternate send/recv like kvclt's (client.hpp:541-561).
+//
+// Worker-to-worker collectives are MPI in the reference (ps.hpp:890-899);
+// this build runs one worker per GPU box, so paracel_sync() is a no-op and
+// the all-reduces over workers are identities.  A multi-worker build links
+// the reference's own Comm instead.
+#pragma once
+
+#include <stdio.h>
+#include <sys/stat.h>
+#include <zmq.h>
+
+#include <fstream>
+#include <iostream>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "msgpack_lite.hpp"
+
+namespace plr_ps {
+
+// kvclt: include/client.hpp.  ports: [0] pull/contains/remove, [1] push,
+// [2] update, [3] bupdate/register_bupdate, [4] ssp ints.
+class kvclt {
+ public:
+  kvclt(const std::string& host, const std::vector<std::string>& ports, void* zctx)
+      : host_(host), ports_(ports), zctx_(zctx) {
+    for (auto& s : socks_) s = nullptr;
+  }
+  ~kvclt() {
+    for (auto s : socks_)
+      if (s) zmq_close(s);
+  }
+
+  template <class V>
+  bool pull(const std::string& key, V& val) {
+    return req(0, paste({pack<std::string>("pull"), pack(key)}), val);
+  }
+  template <class V>
+  bool push(const std::string& key, const V& val) {
+    bool stat = false;
+    const bool r = req(1, paste({pack<std::string>("push"), pack(key), pack(val)}), stat);
+    return r && stat;
+  }
+  bool register_bupdate(const std::string& file, const std::string& func) {
+    bool stat = false;
+    const bool r = req(3, paste({pack<std::string>("register_bupdate"), pack(file), pack(func)}),
+                       stat);
+    return r && stat;
+  }
+  template <class V>
+  V bupdate(const std::string& key, const V& delta, bool& r) {
+    V val;
+    r = req(3, paste({pack<std::string>("bupdate"), pack(key), pack(delta)}), val);
+    return val;
+  }
+  bool push_int(const std::string& key, int v) {
+    bool stat = true;
+    const bool r = req(4, paste({pack<std::string>("push_int"), pack(key), pack(v)}), stat);
+    return r && stat;
+  }
+  bool contains(const std::string& key) {
+    bool v = false;
+    req(0, paste({pack<std::string>("contains"), pack(key)}), v);
+    return v;
+  }
+
+ private:
+  template <class V>
+  bool req(int port_idx, const std::string& scrip, V& val) {
+    void*& s = socks_[port_idx];
+    if (!s) {
+      s = zmq_socket(zctx_, ZMQ_REQ);
+      const std::string ep = "tcp://" + host_ + ":" + ports_.at(port_idx);
+      if (zmq_connect(s, ep.c_str()) != 0)
+        throw std::runtime_error("connect " + ep + ": " + zmq_strerror(zmq_errno()));
+    }
+    if (zmq_send(s, scrip.data(), scrip.size(), 0) < 0)
+      throw std::runtime_error(std::string("zmq_send: ") + zmq_strerror(zmq_errno()));
+    zmq_msg_t m;
+    zmq_msg_init(&m);
+    if (zmq_msg_recv(&m, s, 0) < 0) {
+      zmq_msg_close(&m);
+      throw std::runtime_error(std::string("zmq_recv: ") + zmq_strerror(zmq_errno()));
+    }
+    std::string data((const char*)zmq_msg_data(&m), zmq_msg_size(&m));
+    zmq_msg_close(&m);
+    if (data.empty()) throw std::runtime_error("paracel internal error!");  // client.hpp:551
+    if (data == "nokey") return false;
+    val = unpack<V>(data);
+    return true;
+  }
+
+  std::string host_;
+  std::vector<std::string> ports_;
+  void* zctx_;
+  void* socks_[5];
+};
+
+class paralg {
+ public:
+  // hosts_dct_str: "host:p0,p1,p2,p3,p4" per server joined by _PARACEL_
+  // (server.hpp:417-435, utils.hpp:80-92).  The LR model lives under one key
+  // ("theta"), i.e. on one server (lr.cpp:16-21), so the ring degenerates to
+  // server 0 unless more are given; keys are then placed by std::hash modulo.
+  paralg(const std::string& hosts_dct_str, const std::string& _output = "", int _rounds = 1,
+         int worker_id = 0, int worker_sz = 1)
+      : output(_output), rounds(_rounds), rank_(worker_id), nworker_(worker_sz) {
+    zctx_ = zmq_ctx_new();
+    for (const std::string& one : split_fields(hosts_dct_str)) {
+      const size_t c = one.find(':');
+      if (c == std::string::npos) throw std::invalid_argument("bad server info: " + one);
+      std::vector<std::string> ports;
+      size_t st = c + 1;
+      for (;;) {
+        const size_t en = one.find(',', st);
+        ports.push_back(one.substr(st, en == std::string::npos ? en : en - st));
+        if (en == std::string::npos) break;
+        st = en + 1;
+      }
+      if (ports.size() != 5) throw std::invalid_argument("server info needs 5 ports: " + one);
+      kvm_.emplace_back(new kvclt(one.substr(0, c), ports, zctx_));
+    }
+    if (kvm_.empty()) throw std::invalid_argument("no server given");
+    if (!output.empty()) mkdir(output.c_str(), 0755);
+    if (rank_ == 0) kvm_[0]->push_int("worker_sz", nworker_);  // ps.hpp:119-123
+    paracel_sync();
+  }
+  virtual ~paralg() {
+    kvm_.clear();
+    if (zctx_) zmq_ctx_term(zctx_);
+  }
+
+  // ps.hpp:192-197 -> loader::fixload (load/loader.hpp:81-96): this worker's
+  // byte range of the file, line-aligned by the rule of
+  // load/partition.hpp:57-86,121-139: np equal byte ranges, the last one
+  // running to the end; a range owns the lines that START inside it.
+  std::vector<std::string> paracel_load(const std::string& fn) {
+    std::ifstream f(fn, std::ios::ate);
+    if (!f) throw std::runtime_error("cannot open " + fn);
+    const long sz = f.tellg();
+    const long bk = sz / nworker_;
+    const long st = (long)rank_ * bk;
+    const long en = (rank_ == nworker_ - 1) ? sz : (long)(rank_ + 1) * bk;
+    std::vector<std::string> lines;
+    long offset = st;
+    f.seekg(0);
+    if (offset) {
+      f.seekg(offset - 1);
+      std::string l;
+      std::getline(f, l);
+      offset += (long)l.size();
+    }
+    while (offset < en) {
+      std::string l;
+      if (!std::getline(f, l)) break;
+      offset += (long)l.size() + 1;
+      lines.push_back(l);
+    }
+    std::cout << "lines got: " << lines.size() << std::endl;  // loader.hpp:93
+    return lines;
+  }
+
+  // ps.hpp:437-462: blocking pull; a missing key is an error
+  template <class V>
+  V paracel_read(const std::string& key) {
+    V val;
+    if (!srv(key).pull(key, val)) {
+      std::cerr << "key does not exist" << std::endl;  // ERROR_ABORT only prints
+      return V();
+    }
+    return val;
+  }
+  // ps.hpp:648-657
+  template <class V>
+  bool paracel_write(const std::string& key, const V& val) {
+    return srv(key).push(key, val);
+  }
+  // ps.hpp:372-380: every server loads the reducer
+  bool paracel_register_bupdate(const std::string& file, const std::string& func) {
+    bool r = true;
+    for (auto& k : kvm_) r = r && k->register_bupdate(file, func);
+    return r;
+  }
+  // ps.hpp:753-770: blocking; the reply (the new value) is unpacked and dropped
+  template <class V>
+  bool paracel_bupdate(const std::string& key, const V& delta) {
+    bool r = false;
+    (void)srv(key).bupdate(key, delta, r);
+    return r;
+  }
+  void paracel_sync() {}                       // ps.hpp:890-892 (MPI_Barrier; 1 worker)
+  size_t get_worker_id() const { return rank_; }
+  size_t get_worker_size() const { return nworker_; }
+  template <class T>
+  void allreduce(T&) const {}                  // comm.hpp:629-636 MPI_SUM over 1 worker
+
+  // ps.hpp:983-1017 / :1308: "<output><prefix><rank>", std::to_string
+  // (6 decimals) joined by sep
+  void paracel_dump_vector(const std::vector<double>& v, const std::string& prefix,
+                           const std::string& sep) {
+    std::ofstream os(todir(output) + prefix + std::to_string(rank_), std::ios_base::app);
+    for (size_t i = 0; i + 1 < v.size(); ++i) os << std::to_string(v[i]) << sep;
+    if (!v.empty()) os << std::to_string(v.back()) << '\n';
+  }
+
+ protected:
+  std::string output;
+  int rounds;
+
+ private:
+  static std::string todir(const std::string& d) {
+    return (d.empty() || d.back() == '/') ? d : d + "/";
+  }
+  kvclt& srv(const std::string& key) {
+    return *kvm_[kvm_.size() == 1 ? 0 : std::hash<std::string>()(key) % kvm_.size()];
+  }
+  int rank_, nworker_;
+  void* zctx_ = nullptr;
+  std::vector<std::unique_ptr<kvclt> > kvm_;
+};
+
+}  // namespace plr_ps

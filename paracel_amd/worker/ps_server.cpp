@@ -1,0 +1,187 @@
+// A small parameter-server process that speaks Paracel's wire protocol for
+// the operations on the logistic-regression path, so that the worker's
+// paracel_read / paracel_write / paracel_register_bupdate / paracel_bupdate
+// cross a real ZeroMQ REQ/REP boundary with a dlopen'ed reducer.
+//
+// What it mirrors (reference include/server.hpp): five REP sockets, one
+// thread each (:405-459); four run the op dispatcher thrd_exec (:170-402),
+// the fifth the integer table thrd_exec_ssp (:114-167); values are stored as
+// the packed bytes the client sent (:312-317); bupdate = get -> reducer ->
+// set under one global mutex and replies with the new value (:88-100,
+// :331-349); a missing key is answered with the raw bytes "nokey" (:237-247);
+// the reducer registered on a socket is that socket's thread's state (:173).
+// The reference's servers report their ports to a collector process; this one
+// prints "host:p0,p1,p2,p3,p4" (the format of utils.hpp:80-92) on stdout.
+//
+// Usage: plr_ps_server [--host 127.0.0.1]      (runs until killed, like the
+// reference's start_server, which prun.py ends with killpg)
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <zmq.h>
+
+#include <mutex>
+#include <string>
+#include <thread>
+#include <unordered_map>
+#include <vector>
+
+#include "ps_plugin.hpp"
+
+using namespace plr_ps;
+
+static std::unordered_map<std::string, std::string> tbl_store;  // kv_def.hpp:23
+static std::unordered_map<std::string, int> ssp_tbl;            // kv_def.hpp:24
+static std::mutex store_mutex;                                   // server.hpp:36
+
+static bool recv_all(void* sock, std::string& out) {
+  zmq_msg_t m;
+  zmq_msg_init(&m);
+  const int rc = zmq_msg_recv(&m, sock, 0);
+  if (rc < 0) {
+    zmq_msg_close(&m);
+    return false;
+  }
+  out.assign((const char*)zmq_msg_data(&m), zmq_msg_size(&m));
+  zmq_msg_close(&m);
+  return true;
+}
+
+static void reply(void* sock, const std::string& s) { zmq_send(sock, s.data(), s.size(), 0); }
+
+static void op_thread(void* sock) {
+  update_result update_f;
+  std::string scrip;
+  while (recv_all(sock, scrip)) {
+    std::vector<std::string> msg = split_fields(scrip);
+    std::string op;
+    try {
+      op = unpack<std::string>(msg.at(0));
+      if (op == "contains") {
+        std::lock_guard<std::mutex> g(store_mutex);
+        reply(sock, pack<bool>(tbl_store.count(unpack<std::string>(msg.at(1))) != 0));
+      } else if (op == "pull") {
+        std::string val;
+        bool exist;
+        {
+          std::lock_guard<std::mutex> g(store_mutex);
+          auto it = tbl_store.find(unpack<std::string>(msg.at(1)));
+          exist = it != tbl_store.end();
+          if (exist) val = it->second;
+        }
+        reply(sock, exist ? val : std::string("nokey"));
+      } else if (op == "register_bupdate" || op == "register_update") {
+        std::string err;
+        if (!load_update_plugin(unpack<std::string>(msg.at(1)), unpack<std::string>(msg.at(2)),
+                                update_f, err)) {
+          fprintf(stderr, "%s\n", err.c_str());  // the reference aborts here
+          abort();
+        }
+        reply(sock, pack<bool>(true));
+      } else if (op == "push") {
+        std::lock_guard<std::mutex> g(store_mutex);
+        tbl_store[unpack<std::string>(msg.at(1))] = msg.at(2);  // stored verbatim
+        reply(sock, pack<bool>(true));
+      } else if (op == "update" || op == "bupdate") {
+        if (msg.size() == 5) {
+          std::string err;
+          if (!load_update_plugin(unpack<std::string>(msg[3]), unpack<std::string>(msg[4]),
+                                  update_f, err)) {
+            fprintf(stderr, "%s\n", err.c_str());
+            abort();
+          }
+        }
+        if (!update_f) {
+          fprintf(stderr, "bupdate before register_bupdate on this port\n");
+          abort();
+        }
+        std::string result;
+        {
+          std::lock_guard<std::mutex> g(store_mutex);
+          const std::string key = unpack<std::string>(msg.at(1));
+          auto it = tbl_store.find(key);
+          if (it == tbl_store.end()) {
+            tbl_store[key] = msg.at(2);  // first update of a missing key = set
+            result = msg[2];
+          } else {
+            it->second = update_f(it->second, msg.at(2));
+            result = it->second;
+          }
+        }
+        reply(sock, result);
+      } else if (op == "remove") {
+        std::lock_guard<std::mutex> g(store_mutex);
+        reply(sock, pack<bool>(tbl_store.erase(unpack<std::string>(msg.at(1))) != 0));
+      } else if (op == "clear") {
+        std::lock_guard<std::mutex> g(store_mutex);
+        tbl_store.clear();
+        reply(sock, pack<bool>(true));
+      } else {
+        fprintf(stderr, "plr_ps_server: unsupported op '%s'\n", op.c_str());
+        reply(sock, pack<bool>(false));
+      }
+    } catch (const std::exception& e) {
+      fprintf(stderr, "plr_ps_server: bad request (%s)\n", e.what());
+      reply(sock, pack<bool>(false));
+    }
+  }
+}
+
+static void ssp_thread(void* sock) {
+  std::string scrip;
+  while (recv_all(sock, scrip)) {
+    std::vector<std::string> msg = split_fields(scrip);
+    try {
+      const std::string op = unpack<std::string>(msg.at(0));
+      if (op == "push_int") {
+        std::lock_guard<std::mutex> g(store_mutex);
+        ssp_tbl[unpack<std::string>(msg.at(1))] = unpack<int>(msg.at(2));
+        reply(sock, pack<bool>(true));
+      } else if (op == "pull_int") {
+        std::lock_guard<std::mutex> g(store_mutex);
+        auto it = ssp_tbl.find(unpack<std::string>(msg.at(1)));
+        if (it == ssp_tbl.end()) reply(sock, "nokey");
+        else reply(sock, pack<int>(it->second));
+      } else if (op == "incr_int") {
+        std::lock_guard<std::mutex> g(store_mutex);
+        ssp_tbl[unpack<std::string>(msg.at(1))] += unpack<int>(msg.at(2));
+        reply(sock, pack<bool>(true));
+      } else {
+        reply(sock, pack<bool>(false));
+      }
+    } catch (const std::exception& e) {
+      reply(sock, pack<bool>(false));
+    }
+  }
+}
+
+int main(int argc, char** argv) {
+  std::string host = "127.0.0.1";
+  for (int i = 1; i + 1 < argc; ++i)
+    if (!strcmp(argv[i], "--host")) host = argv[i + 1];
+  void* ctx = zmq_ctx_new();
+  const int kThreads = 5;  // paracel_types.hpp:45 threads_num
+  void* socks[kThreads];
+  std::string info = host + ":";
+  for (int i = 0; i < kThreads; ++i) {
+    socks[i] = zmq_socket(ctx, ZMQ_REP);
+    const std::string ep = "tcp://" + host + ":*";
+    if (zmq_bind(socks[i], ep.c_str()) != 0) {
+      fprintf(stderr, "plr_ps_server: bind %s failed: %s\n", ep.c_str(), zmq_strerror(zmq_errno()));
+      return 1;
+    }
+    char bound[256];
+    size_t len = sizeof bound;
+    zmq_getsockopt(socks[i], ZMQ_LAST_ENDPOINT, bound, &len);
+    const char* colon = strrchr(bound, ':');
+    info += (i ? "," : "");
+    info += (colon ? colon + 1 : "0");
+  }
+  printf("%s\n", info.c_str());
+  fflush(stdout);
+  std::vector<std::thread> th;
+  for (int i = 0; i < 4; ++i) th.emplace_back(op_thread, socks[i]);
+  th.emplace_back(ssp_thread, socks[4]);
+  for (auto& t : th) t.join();
+  return 0;
+}

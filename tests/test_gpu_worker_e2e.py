@@ -1,0 +1,93 @@
+"""End to end through the host parameter server: the C++ worker
+(paracel_amd/worker, same call order as the reference's dgd_learning) reads
+theta over ZeroMQ, computes delta on the GPU through the C ABI and pushes it
+with paracel_bupdate into a server process whose reducer is the dlopen'ed
+lr_theta_update plugin.  The final theta is compared with the CPU oracle's
+training loop (tool/lr_serial.cpp:95-110 restated) on the same seeded data:
+relative error <= 1e-8 after 100 iterations.
+"""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "paracel_amd")
+
+
+def rel(a, b):
+    return np.linalg.norm(a - b) / np.linalg.norm(b)
+
+
+@pytest.fixture()
+def server_info():
+    for f in ("plr_ps_server", "plr_lr_worker", "liblr_update.so"):
+        assert os.path.exists(os.path.join(PKG, f)), "%s is not built" % f
+    p = subprocess.Popen([os.path.join(PKG, "plr_ps_server")], stdout=subprocess.PIPE, text=True)
+    info = p.stdout.readline().strip()
+    yield info
+    p.kill()
+    p.wait()
+
+
+def test_synthetic_100_rounds_match_oracle(server_info, oracle, gen, tmp_path):
+    n, d, rounds = 20000, 512, 100
+    cfg = gen.configs()["c5_e2e_2m_x_512"].scaled(n)
+    alpha, beta = cfg.lr / n, cfg.lam / 2
+    out = tmp_path / "theta.bin"
+    cmd = [os.path.join(PKG, "plr_lr_worker"), "--server_info", server_info,
+           "--synthetic", "%x,%d,%d,%.17g" % (cfg.seed, n, d, cfg.spec.scale),
+           "--rounds", str(rounds), "--alpha", "%.17g" % alpha, "--beta", "%.17g" % beta,
+           "--theta0", "zero", "--update_file", os.path.join(PKG, "liblr_update.so"),
+           "--theta_out", str(out)]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr
+    rep = json.loads(r.stdout.strip().splitlines()[-1])
+    print(rep)
+    theta = np.fromfile(out)
+    X, y = cfg.rows(0, n)
+    theta_ref = oracle.train_dgd(X, y, np.zeros(d), alpha, beta, rounds)
+    assert theta.shape == (d,)
+    assert rel(theta, theta_ref) <= 1e-8
+    assert abs(rep["final_loss"] - oracle.calc_loss(X, y, theta_ref)) <= 1e-10
+    assert rep["rounds"] == rounds and rep["iters_per_sec"] > 0
+
+
+def test_csv_driver_follows_the_reference_call_order(server_info, oracle, tmp_path):
+    # training file "f1,...,fk,label" (lr.cpp:74-75), cfg keys of lr_driver.cpp:45-59
+    rng = np.random.default_rng(3)
+    n, k = 400, 6
+    F = np.round(rng.normal(size=(n, k)), 4)
+    lab = (rng.random(n) < 0.5).astype(int)
+    train = tmp_path / "train.csv"
+    with open(train, "w") as f:
+        for i in range(n):
+            f.write(",".join("%.4f" % v for v in F[i]) + ",%d\n" % lab[i])
+    outdir = tmp_path / "out"
+    cfgf = tmp_path / "cfg.json"
+    cfgf.write_text(json.dumps({
+        "training_input": str(train), "test_input": str(train), "predict_input": str(train),
+        "output": str(outdir) + "/", "update_file": os.path.join(PKG, "liblr_update.so"),
+        "update_func": "lr_theta_update", "method": "dgd", "rounds": 20,
+        "alpha": 0.001, "beta": 0.01, "debug": True}, indent=2))
+    r = subprocess.run([os.path.join(PKG, "plr_lr_worker"), "--server_info", server_info,
+                        "--cfg_file", str(cfgf), "--theta0", "zero"],
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr
+    X = np.hstack([np.ones((n, 1)), F])          # bias column first (lr.cpp:83)
+    y = lab.astype(float)
+    theta_ref = oracle.train_dgd(X, y, np.zeros(k + 1), 0.001, 0.01, 20)
+    # lr_theta_<rank>: std::to_string (6 decimals) joined by '|' (lr.cpp:340, ps.hpp:1308)
+    dumped = np.array([float(t) for t in (outdir / "lr_theta_0").read_text().strip().split("|")])
+    np.testing.assert_allclose(dumped, theta_ref, atol=5.1e-7, rtol=0)
+    loss_line = [ln for ln in r.stdout.splitlines() if ln.startswith("final loss:")][0]
+    assert abs(float(loss_line.split(":")[1]) - oracle.calc_loss(X, y, theta_ref)) <= 1e-10
+    assert "loss in test dataset is:" in r.stdout
+    pred = np.array([float(t) for t in (outdir / "pred_v_0").read_text().split()])
+    np.testing.assert_allclose(pred, oracle.predict(X, theta_ref), atol=5.1e-7, rtol=0)
+    # debug: one loss per round, at the theta read at the start of that round
+    curve = np.array([float(t) for t in (outdir / "lr_loss_error_0").read_text().split()])
+    assert curve.shape == (20,) and abs(curve[0] - np.log(2)) < 1e-6 and curve[-1] < curve[0]
