@@ -45,6 +45,9 @@ def parse_args():
     ap.add_argument("--rows", type=int, default=0, help="override n (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-rows", type=int, default=0)
+    ap.add_argument("--e2e", action="store_true",
+                    help="end-to-end rounds through the host parameter server (C++ worker + "
+                         "plr_ps_server over ZeroMQ) instead of the bare gradient step")
     return ap.parse_args()
 
 
@@ -105,6 +108,70 @@ def cpu_baseline(cfg, Xs, ys, theta):
     }
 
 
+def run_e2e(a, cfg):
+    """steps rounds of read theta -> GPU delta -> bupdate against a real server
+    process; final theta against the CPU oracle's multi-worker training."""
+    import subprocess
+    import tempfile
+
+    import numpy as np
+
+    pkg = os.path.join(ROOT, "paracel_amd")
+    srv = subprocess.Popen([os.path.join(pkg, "plr_ps_server")], stdout=subprocess.PIPE, text=True)
+    try:
+        info = srv.stdout.readline().strip()
+        with tempfile.TemporaryDirectory() as td:
+            tout = os.path.join(td, "theta.bin")
+            cmd = [os.path.join(pkg, "plr_lr_worker"), "--server_info", info,
+                   "--synthetic", "%x,%d,%d,%.17g" % (cfg.seed, cfg.n, cfg.d, cfg.spec.scale),
+                   "--rounds", str(a.steps), "--alpha", "%.17g" % cfg.alpha,
+                   "--beta", "%.17g" % cfg.beta, "--theta0", "zero",
+                   "--update_file", os.path.join(pkg, "liblr_update.so"), "--theta_out", tout]
+            r = subprocess.run(cmd, capture_output=True, text=True)
+            if r.returncode != 0:
+                raise RuntimeError("worker failed: " + r.stderr)
+            rep = json.loads(r.stdout.strip().splitlines()[-1])
+            theta_gpu = np.fromfile(tout)
+    finally:
+        srv.kill()
+        srv.wait()
+    out = {
+        "metric": "lr_e2e_iters_per_sec", "value": rep["iters_per_sec"], "unit": "iters/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": 0,
+        "ms_per_step": 1e3 / rep["iters_per_sec"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": cfg.name + " via parameter server", "n": cfg.n, "d": cfg.d,
+                   "step": "paracel_read theta -> plr_dgd_delta -> paracel_bupdate delta "
+                           "(ZeroMQ REQ/REP, msgpack, dlopen'ed lr_theta_update)",
+                   "alpha": cfg.alpha, "beta": cfg.beta},
+        "gpu_only_iters_per_sec": rep["gpu_only_iters_per_sec"],
+        "gpu_kernel_ms_per_iter": rep["gpu_kernel_ms_per_iter"],
+        "final_loss": rep["final_loss"],
+        "theta_rel_err_vs_cpu": None,
+    }
+    if not a.no_cpu_baseline:
+        from oracle import oracle
+
+        cores = max(1, min(16, os.cpu_count() or 1))
+        X = np.empty((cfg.n, cfg.d))
+        y = np.empty(cfg.n)
+        step = 262144
+        for lo in range(0, cfg.n, step):
+            m = min(step, cfg.n - lo)
+            _, y[lo:lo + m] = cfg.rows(lo, m, out=X[lo:lo + m])
+        t0 = time.time()
+        theta_cpu = oracle.train_dgd_workers(X, y, np.zeros(cfg.d), cfg.alpha, cfg.beta,
+                                             a.steps, cores)
+        sec = time.time() - t0
+        out["theta_rel_err_vs_cpu"] = float(np.linalg.norm(theta_gpu - theta_cpu) /
+                                            np.linalg.norm(theta_cpu))
+        out["cpu_baseline"] = {"value": a.steps / sec, "unit": "iters/s", "cores": cores,
+                               "kind": "port",
+                               "sample": "all %d rounds on the full shard, %d local workers "
+                                         "(threads), in-process server add" % (a.steps, cores)}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     a = parse_args()
     if a.gpus != 1:
@@ -124,6 +191,9 @@ def main():
     cfg = cfgs[a.workload]
     if a.rows:
         cfg = cfg.scaled(a.rows)
+    if a.e2e:
+        run_e2e(a, cfg)
+        return
     theta = cfg.theta()
 
     # ~2 GB sample for the CPU leg (bounded: a few seconds per traversal on one core)

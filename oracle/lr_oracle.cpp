@@ -127,6 +127,26 @@ void oracle_train_dgd(const double* X, int64_t n, int64_t d, int64_t ldx,
   }
 }
 
+void oracle_train_dgd_workers(const double* X, int64_t n, int64_t d, int64_t ldx,
+                              const double* y, double* theta, double alpha,
+                              double beta, int rounds, int workers) {
+  if (workers < 1) workers = 1;
+  vector<vector<double> > delta(workers, vector<double>(d));
+  for (int rd = 0; rd < rounds; ++rd) {
+    vector<std::thread> th;
+    for (int w = 0; w < workers; ++w) {
+      const int64_t lo = n * w / workers, hi = n * (w + 1) / workers;
+      th.emplace_back([=, &delta]() {
+        oracle_dgd_delta(X + lo * ldx, hi - lo, d, ldx, y + lo, theta, alpha, beta,
+                         nullptr, delta[w].data());
+      });
+    }
+    for (auto& t : th) t.join();
+    for (int w = 0; w < workers; ++w)
+      for (int64_t i = 0; i < d; ++i) theta[i] = theta[i] + delta[w][i];
+  }
+}
+
 int64_t oracle_local_parser(const char* text, int64_t nlines, char sep,
                             double* X_out, double* y_out,
                             int64_t k_expected) {

@@ -81,6 +81,15 @@ void oracle_train_dgd(const double* X, int64_t n, int64_t d, int64_t ldx,
                       const double* y, double* theta,
                       double alpha, double beta, int rounds);
 
+/* The same rounds with P local workers (mpirun -n P bin/lr, prun.py:78-79):
+ * rows split into P contiguous shards, each worker traverses its shard
+ * (lr.cpp:132-138) in its own thread, then the server folds the worker deltas
+ * into theta one at a time in worker order (update.cpp:26-32 applied P times
+ * per round).  P = 1 is oracle_train_dgd. */
+void oracle_train_dgd_workers(const double* X, int64_t n, int64_t d, int64_t ldx,
+                              const double* y, double* theta, double alpha,
+                              double beta, int rounds, int workers);
+
 /* lr.cpp:76-93: parse CSV lines "f1,...,fk,label" into rows [1.0,f1..fk]
  * and labels.  `text` holds `nlines` '\n'-separated lines.  X_out must hold
  * nlines*(k+1) doubles, y_out nlines.  Returns k+1 (row width D), or -1 on a

@@ -41,6 +41,8 @@ def load():
             getattr(L, f).argtypes = shp + [_dp, _dp, _dp]
         L.oracle_train_dgd.restype = None
         L.oracle_train_dgd.argtypes = shp + [_dp, _dp, C.c_double, C.c_double, C.c_int]
+        L.oracle_train_dgd_workers.restype = None
+        L.oracle_train_dgd_workers.argtypes = shp + [_dp, _dp, C.c_double, C.c_double, C.c_int, C.c_int]
         L.oracle_dgd_delta_hp.restype = None
         L.oracle_dgd_delta_hp.argtypes = shp + [_dp, _dp, C.c_double, C.c_double, _dp]
         L.oracle_local_parser.restype = C.c_int64
@@ -149,6 +151,14 @@ def train_dgd(X, y, theta0, alpha, beta, rounds):
     y = _c(y)
     theta = np.array(theta0, dtype=np.float64, copy=True)
     load().oracle_train_dgd(_p(X), n, d, d, _p(y), _p(theta), alpha, beta, rounds)
+    return theta
+
+
+def train_dgd_workers(X, y, theta0, alpha, beta, rounds, workers):
+    X, n, d = _shape(X)
+    y = _c(y)
+    theta = np.array(theta0, dtype=np.float64, copy=True)
+    load().oracle_train_dgd_workers(_p(X), n, d, d, _p(y), _p(theta), alpha, beta, rounds, workers)
     return theta
 
 

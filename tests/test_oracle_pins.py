@@ -204,6 +204,16 @@ def test_training_reaches_the_regularised_optimum(oracle):
     np.testing.assert_array_equal(t1, oracle.theta_update(th, oracle.dgd_delta(X, y, th, lr / n, lam / 2)))
 
 
+def test_multi_worker_training_matches_single_worker(oracle):
+    # P workers + server-side folding only regroups the sums (shard additivity)
+    X, y, _ = rand_case(3000, 12, 9)
+    n = X.shape[0]
+    t1 = oracle.train_dgd(X, y, np.zeros(12), 0.5 / n, 0.01, 30)
+    assert np.array_equal(t1, oracle.train_dgd_workers(X, y, np.zeros(12), 0.5 / n, 0.01, 30, 1))
+    t4 = oracle.train_dgd_workers(X, y, np.zeros(12), 0.5 / n, 0.01, 30, 4)
+    assert rel(t4, t1) <= 1e-13
+
+
 def test_local_parser(oracle):
     # lr.cpp:76-93: "f1,...,fk,label" -> [1.0, f1..fk], label; empty fields are dropped
     X, y = oracle.local_parser("0.5,2,1\n-1e-3,4.25,0\n")
