@@ -219,6 +219,7 @@ def main():
     assert launches == a.steps and n == cfg.n
     kern_ms = kern_ms_sum / launches
 
+    read_ceiling = ctx.probe_read_bandwidth(10)
     bytes_step = cfg.algorithmic_bytes()
     achieved = bytes_step / (kern_ms * 1e-3) / 1e9
     traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name)
@@ -243,7 +244,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel_ms": kern_ms, "algorithmic_bytes": bytes_step,
-                     "whole_step_gbs": bytes_step / (elapsed / a.steps) / 1e9},
+                     "whole_step_gbs": bytes_step / (elapsed / a.steps) / 1e9,
+                     "read_ceiling_gbs": read_ceiling,
+                     "frac_of_read_ceiling": achieved / read_ceiling},
         "cpu_baseline": None,
         "loss_mean": loss / n,
     }

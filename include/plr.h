@@ -99,6 +99,13 @@ int plr_get_timing(const plr_ctx* ctx, double* last_ms, double* sum_ms,
                    int64_t* launches);
 int plr_reset_timing(plr_ctx* ctx);
 
+/* Read ceiling of this device, measured on the resident shard: a kernel that
+ * only streams X (same access pattern as the fused pass, no arithmetic) is
+ * launched `reps` times; reports GB/s.  No counterpart in the reference; used
+ * by benchmarks to state the fused pass as a fraction of what a pure read
+ * sustains. */
+int plr_probe_read_bandwidth(plr_ctx* ctx, int reps, double* gb_per_s);
+
 /* Human-readable description of the kernel variant chosen for the resident
  * shape (tile shape, grid), for logs.  Context-owned, never freed. */
 const char* plr_kernel_info(const plr_ctx* ctx);

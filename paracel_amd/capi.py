@@ -32,6 +32,7 @@ SYMBOLS = [
     ("plr_get_shape", C.c_int, [_ctx, _i64p, _i64p]),
     ("plr_get_timing", C.c_int, [_ctx, _dp, _dp, _i64p]),
     ("plr_reset_timing", C.c_int, [_ctx]),
+    ("plr_probe_read_bandwidth", C.c_int, [_ctx, C.c_int, _dp]),
     ("plr_kernel_info", C.c_char_p, [_ctx]),
     ("plr_last_error", C.c_char_p, [_ctx]),
     ("plr_version", C.c_char_p, []),
@@ -181,6 +182,12 @@ class Plr:
 
     def reset_timing(self):
         self._check(self._lib.plr_reset_timing(self._h))
+
+    def probe_read_bandwidth(self, reps=10):
+        """GB/s a pure streaming read of the resident shard sustains."""
+        gbs = C.c_double()
+        self._check(self._lib.plr_probe_read_bandwidth(self._h, reps, C.byref(gbs)))
+        return gbs.value
 
     def kernel_info(self):
         return self._lib.plr_kernel_info(self._h).decode()

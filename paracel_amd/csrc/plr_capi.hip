@@ -78,10 +78,10 @@ struct plr_ctx {
   double* d_theta = nullptr;    // theta_len doubles, zero padded
   double* d_part_g = nullptr;   // grid x pitch
   double* d_part_loss = nullptr;  // max(grid, grid_nograd)
-  double* d_out = nullptr;      // d + 1
   double* d_h = nullptr;        // n (predict), lazily allocated
   double* h_theta = nullptr;    // pinned, theta_len
-  double* h_out = nullptr;      // pinned, d + 1
+  double* h_out = nullptr;      // pinned + device-mapped, d + 1: finish_pass writes it
+  double* h_out_dev = nullptr;  // the device's address of h_out
 
   double last_ms = 0., sum_ms = 0.;
   int64_t launches = 0;
@@ -117,12 +117,11 @@ void free_shape(plr_ctx* c) {
   if (c->d_theta) (void)hipFree(c->d_theta);
   if (c->d_part_g) (void)hipFree(c->d_part_g);
   if (c->d_part_loss) (void)hipFree(c->d_part_loss);
-  if (c->d_out) (void)hipFree(c->d_out);
   if (c->d_h) (void)hipFree(c->d_h);
   if (c->h_theta) (void)hipHostFree(c->h_theta);
   if (c->h_out) (void)hipHostFree(c->h_out);
-  c->dX = c->dy = c->d_theta = c->d_part_g = c->d_part_loss = c->d_out =
-      c->d_h = c->h_theta = c->h_out = nullptr;
+  c->dX = c->dy = c->d_theta = c->d_part_g = c->d_part_loss = c->d_h =
+      c->h_theta = c->h_out = c->h_out_dev = nullptr;
   c->n = c->d = c->pitch = 0;
   c->have_data = false;
   c->var = nullptr;
@@ -201,9 +200,12 @@ int alloc_shape(plr_ctx* c, int64_t n, int64_t d) {
   PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)c->theta_len * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_g, (size_t)c->grid * c->pitch * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_loss, (size_t)gmax * sizeof(double)));
-  PLR_HIP(c, hipMalloc(&c->d_out, (size_t)(d + 1) * sizeof(double)));
   PLR_HIP(c, hipHostMalloc(&c->h_theta, (size_t)c->theta_len * sizeof(double), hipHostMallocDefault));
-  PLR_HIP(c, hipHostMalloc(&c->h_out, (size_t)(d + 1) * sizeof(double), hipHostMallocDefault));
+  // results land in host memory straight from the finishing kernel (no
+  // device-to-host copy in the step): pinned, mapped, coherent
+  PLR_HIP(c, hipHostMalloc(&c->h_out, (size_t)(d + 1) * sizeof(double),
+                           hipHostMallocMapped | hipHostMallocCoherent));
+  PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_out_dev), c->h_out, 0));
   memset(c->h_theta, 0, (size_t)c->theta_len * sizeof(double));
   PLR_HIP(c, hipMemsetAsync(c->d_theta, 0, (size_t)c->theta_len * sizeof(double), c->stream));
   if (n > 0 && c->pitch != d)  // the pad column must read as zero
@@ -280,7 +282,7 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
     fa.part_g = c->d_part_g;
     fa.part_loss = c->d_part_loss;
     fa.theta = c->d_theta;
-    fa.out = c->d_out;
+    fa.out = c->h_out_dev;
     fa.pitch = c->pitch;
     fa.d = c->d;
     fa.n = c->n;
@@ -293,10 +295,15 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
     hipLaunchKernelGGL(plr::finish_pass, dim3(fgrid),
                        dim3(plr::kFinCols * plr::kFinSlices), 0, c->stream, fa);
     PLR_HIP(c, hipGetLastError());
-    PLR_HIP(c, hipMemcpyAsync(c->h_out, c->d_out, (size_t)(c->d + 1) * sizeof(double),
-                              hipMemcpyDeviceToHost, c->stream));
   }
-  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  // Poll the stream instead of sleeping on it: a blocking wait adds an
+  // interrupt wake-up to every step, and a step is only ~1 ms long.
+  for (;;) {
+    const hipError_t q = hipStreamQuery(c->stream);
+    if (q == hipSuccess) break;
+    if (q != hipErrorNotReady) PLR_HIP(c, q);
+    __builtin_ia32_pause();
+  }
   float ms = 0.f;
   PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
   c->last_ms = ms;
@@ -422,6 +429,31 @@ int plr_predict(plr_ctx* c, const double* theta, double* h_out) {
   if (rc != PLR_OK) return rc;
   if (c->n > 0)
     PLR_HIP(c, hipMemcpy(h_out, c->d_h, (size_t)c->n * sizeof(double), hipMemcpyDeviceToHost));
+  return PLR_OK;
+}
+
+int plr_probe_read_bandwidth(plr_ctx* c, int reps, double* gb_per_s) {
+  if (!c) return PLR_ERR_INVALID;
+  if (!gb_per_s || reps < 1) return fail(c, PLR_ERR_INVALID, "need reps >= 1 and an output");
+  if (!c->have_data || c->n == 0) return fail(c, PLR_ERR_NODATA, "no shard resident");
+  PLR_HIP(c, hipSetDevice(c->device));
+  const size_t bytes = (size_t)c->n * c->pitch * sizeof(double);
+  const int64_t ntiles = (int64_t)(bytes / 8192);
+  if (ntiles < 1) return fail(c, PLR_ERR_INVALID, "shard smaller than one 8 KiB tile");
+  const int grid = c->num_cu;
+  for (int i = 0; i < 2; ++i)
+    hipLaunchKernelGGL(plr::read_probe, dim3(grid), dim3(256), 0, c->stream,
+                       reinterpret_cast<const plr::v2d*>(c->dX), ntiles, c->d_part_loss);
+  PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
+  for (int i = 0; i < reps; ++i)
+    hipLaunchKernelGGL(plr::read_probe, dim3(grid), dim3(256), 0, c->stream,
+                       reinterpret_cast<const plr::v2d*>(c->dX), ntiles, c->d_part_loss);
+  PLR_HIP(c, hipGetLastError());
+  PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  float ms = 0.f;
+  PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
+  *gb_per_s = (double)ntiles * 8192.0 * reps / (ms * 1e-3) / 1e9;
   return PLR_OK;
 }
 
