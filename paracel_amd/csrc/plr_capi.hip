@@ -41,7 +41,7 @@ struct Variant {
 const Variant kVariants[] = {
     PLR_VARIANT(1, 16, 1, 4, 2, false),   // d <= 128
     PLR_VARIANT(2, 32, 1, 4, 1, false),   // d <= 256
-    PLR_VARIANT(4, 8, 1, 4, 1, false),    // d <= 512
+    PLR_VARIANT(4, 16, 1, 2, 1, false),   // d <= 512
     PLR_VARIANT(8, 4, 1, 4, 1, false),    // d <= 1024
     PLR_VARIANT(2, 8, 8, 1, 2, false),    // d <= 2048
     PLR_VARIANT(4, 4, 8, 1, 2, false),    // d <= 4096
