@@ -53,9 +53,11 @@ def build_copy_probe():
 
 def build_worker():
     """Host side of the worker path (g++): parameter-server process, reducer
-    plugin, GPU LR worker -> paracel_amd/{plr_ps_server,liblr_update.so,plr_lr_worker}"""
+    plugin, GPU LR worker, shard tool ->
+    paracel_amd/{plr_ps_server,liblr_update.so,plr_lr_worker,plr_shard_tool}"""
     _run(["make", "-B", "-C", os.path.join(_HERE, "worker")])
-    return [os.path.join(_HERE, f) for f in ("plr_ps_server", "liblr_update.so", "plr_lr_worker")]
+    return [os.path.join(_HERE, f) for f in ("plr_ps_server", "liblr_update.so", "plr_lr_worker",
+                                             "plr_shard_tool")]
 
 
 def build_all():

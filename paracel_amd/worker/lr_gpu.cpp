@@ -34,32 +34,35 @@ void logistic_regression_gpu::check(int rc, const char* what) {
 }
 
 void logistic_regression_gpu::local_parser(const std::vector<std::string>& linelst, char sep) {
-  flat.clear();
-  labels.clear();
-  n_local = 0;
-  data_dim = 0;
-  std::vector<double> row;
-  for (const std::string& line : linelst) {
-    row.clear();
-    row.push_back(1.);  // bias column
-    size_t st = 0;
-    std::vector<double> fields;
-    for (;;) {  // str_split: empty fields are dropped (ext_utility.hpp:38-50)
-      const size_t en = line.find(sep, st);
-      const std::string tok = line.substr(st, en == std::string::npos ? en : en - st);
-      if (!tok.empty()) fields.push_back(std::stod(tok));
-      if (en == std::string::npos) break;
-      st = en + 1;
-    }
-    if (fields.empty()) throw std::invalid_argument("empty sample line");
-    for (size_t i = 0; i + 1 < fields.size(); ++i) row.push_back(fields[i]);
-    if (data_dim == 0) data_dim = (int64_t)row.size();
-    if ((int64_t)row.size() != data_dim) throw std::invalid_argument("ragged sample line");
-    flat.insert(flat.end(), row.begin(), row.end());
-    labels.push_back(fields.back());
-    ++n_local;
-  }
+  ParsedShard s = parse_lines(linelst, sep);
+  n_local = s.n;
+  data_dim = s.d;
+  flat.swap(s.X);
+  labels.swap(s.y);
   if (kdim == 0 && data_dim > 0) kdim = (int)data_dim - 1;
+}
+
+// paracel_load + local_parser, through the binary shard cache when it is fresh
+void logistic_regression_gpu::load_and_parse(const std::string& fn) {
+  ParsedShard s;
+  const int rank = (int)get_worker_id(), np = (int)get_worker_size();
+  if (read_cache(fn, rank, np, s)) {
+    std::cout << "shard cache hit: " << s.n << " x " << s.d << std::endl;
+    n_local = s.n;
+    data_dim = s.d;
+    flat.swap(s.X);
+    labels.swap(s.y);
+    if (kdim == 0 && data_dim > 0) kdim = (int)data_dim - 1;
+    return;
+  }
+  local_parser(paracel_load(fn));
+  s.n = n_local;
+  s.d = data_dim;
+  s.X.swap(flat);
+  s.y.swap(labels);
+  if (!write_cache(fn, rank, np, s)) std::cout << "shard cache not written" << std::endl;
+  flat.swap(s.X);
+  labels.swap(s.y);
 }
 
 void logistic_regression_gpu::set_samples(const double* X, int64_t n, int64_t d, int64_t ldx,
@@ -114,8 +117,7 @@ void logistic_regression_gpu::dgd_learning() {
 
 void logistic_regression_gpu::solve() {
   if (!input.empty()) {
-    auto lines = paracel_load(input);
-    local_parser(lines);
+    load_and_parse(input);
     upload();
   }
   paracel_sync();
@@ -148,8 +150,7 @@ void logistic_regression_gpu::dump_result() {
 }
 
 void logistic_regression_gpu::test(const std::string& test_fn) {
-  auto lines = paracel_load(test_fn);
-  local_parser(lines);
+  load_and_parse(test_fn);
   upload();
   std::cout << "loss in test dataset is: " << calc_loss() << std::endl;
   paracel_sync();

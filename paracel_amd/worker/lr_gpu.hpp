@@ -48,6 +48,7 @@ class logistic_regression_gpu : public paralg {
   double round_seconds() const { return round_sec; }  // wall time inside the rounds loop
 
  private:
+  void load_and_parse(const std::string& fn);  // paracel_load + local_parser, cached
   void upload();                // flat rows -> HBM, then the host copy is dropped
   void check(int rc, const char* what);
 

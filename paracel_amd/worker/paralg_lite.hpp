@@ -23,6 +23,7 @@
 #include <vector>
 
 #include "msgpack_lite.hpp"
+#include "shard_io.hpp"
 
 namespace plr_ps {
 
@@ -139,31 +140,9 @@ class paralg {
   }
 
   // ps.hpp:192-197 -> loader::fixload (load/loader.hpp:81-96): this worker's
-  // byte range of the file, line-aligned by the rule of
-  // load/partition.hpp:57-86,121-139: np equal byte ranges, the last one
-  // running to the end; a range owns the lines that START inside it.
+  // byte range of the file, line-aligned (rule in shard_io.hpp)
   std::vector<std::string> paracel_load(const std::string& fn) {
-    std::ifstream f(fn, std::ios::ate);
-    if (!f) throw std::runtime_error("cannot open " + fn);
-    const long sz = f.tellg();
-    const long bk = sz / nworker_;
-    const long st = (long)rank_ * bk;
-    const long en = (rank_ == nworker_ - 1) ? sz : (long)(rank_ + 1) * bk;
-    std::vector<std::string> lines;
-    long offset = st;
-    f.seekg(0);
-    if (offset) {
-      f.seekg(offset - 1);
-      std::string l;
-      std::getline(f, l);
-      offset += (long)l.size();
-    }
-    while (offset < en) {
-      std::string l;
-      if (!std::getline(f, l)) break;
-      offset += (long)l.size() + 1;
-      lines.push_back(l);
-    }
+    std::vector<std::string> lines = load_lines(fn, rank_, nworker_);
     std::cout << "lines got: " << lines.size() << std::endl;  // loader.hpp:93
     return lines;
   }

@@ -1,0 +1,189 @@
+// Host-side producer of the shard the GPU keeps: file -> this worker's lines
+// -> numeric rows, plus a binary cache of the parsed shard so that the text
+// is parsed once (std::stod over ~20 GB of text per 8 GB of doubles is the
+// real end-to-end cost of a file-fed run).
+//
+//   load_lines : the reference's "linesplit" rule -- np equal byte ranges,
+//                the last one running to the end; a range owns the lines that
+//                START inside it (include/load/partition.hpp:57-86,121-139,
+//                reached from paralg::paracel_load, include/ps.hpp:178-197).
+//   parse_lines: logistic_regression::local_parser (lr.cpp:76-93):
+//                "f1,...,fk,label" -> [1.0, f1..fk] and the label; empty
+//                fields are dropped as str_split does
+//                (include/utils/ext_utility.hpp:38-50); std::stod semantics.
+//                Lines are parsed by several threads; the result does not
+//                depend on the thread count.
+//   *_cache    : "<input>.plrshard.<rank>of<np>": header + X (row-major,
+//                n x d doubles, bias column included) + y.  Rejected unless
+//                magic, version, input size and input mtime all match.
+#pragma once
+
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+#include <sys/stat.h>
+
+#include <fstream>
+#include <stdexcept>
+#include <string>
+#include <thread>
+#include <vector>
+
+namespace plr_ps {
+
+inline std::vector<std::string> load_lines(const std::string& fn, int rank, int np) {
+  std::ifstream f(fn, std::ios::ate);
+  if (!f) throw std::runtime_error("cannot open " + fn);
+  const long sz = f.tellg();
+  const long bk = sz / np;
+  const long st = (long)rank * bk;
+  const long en = (rank == np - 1) ? sz : (long)(rank + 1) * bk;
+  std::vector<std::string> lines;
+  long offset = st;
+  f.seekg(0);
+  if (offset) {
+    // step back one byte and finish the line in progress: if that byte is the
+    // newline itself, the next line starts exactly at `st` and is ours
+    f.seekg(offset - 1);
+    std::string l;
+    std::getline(f, l);
+    offset += (long)l.size();
+  }
+  while (offset < en) {
+    std::string l;
+    if (!std::getline(f, l)) break;
+    offset += (long)l.size() + 1;
+    lines.push_back(l);
+  }
+  return lines;
+}
+
+struct ParsedShard {
+  int64_t n = 0, d = 0;          // d counts the bias column
+  std::vector<double> X, y;      // X: n x d row-major
+};
+
+inline void parse_one_line(const std::string& line, char sep, std::vector<double>& fields) {
+  fields.clear();
+  size_t st = 0;
+  for (;;) {
+    const size_t en = line.find(sep, st);
+    const size_t len = (en == std::string::npos ? line.size() : en) - st;
+    if (len) fields.push_back(std::stod(line.substr(st, len)));  // throws like the reference
+    if (en == std::string::npos) break;
+    st = en + 1;
+  }
+}
+
+inline ParsedShard parse_lines(const std::vector<std::string>& lines, char sep = ',',
+                               int threads = 16) {
+  ParsedShard s;
+  s.n = (int64_t)lines.size();
+  if (s.n == 0) return s;
+  std::vector<double> first;
+  parse_one_line(lines[0], sep, first);
+  if (first.empty()) throw std::invalid_argument("empty sample line");
+  s.d = (int64_t)first.size();  // k features + label  ->  bias + k features
+  s.X.resize((size_t)s.n * s.d);
+  s.y.resize(s.n);
+  if (threads < 1) threads = 1;
+  if ((int64_t)threads > s.n) threads = (int)s.n;
+  std::vector<std::string> errors(threads);
+  auto work = [&](int t) {
+    std::vector<double> fields;
+    const int64_t lo = s.n * t / threads, hi = s.n * (t + 1) / threads;
+    try {
+      for (int64_t i = lo; i < hi; ++i) {
+        parse_one_line(lines[i], sep, fields);
+        if ((int64_t)fields.size() != s.d)
+          throw std::invalid_argument("ragged sample line " + std::to_string(i));
+        double* row = s.X.data() + i * s.d;
+        row[0] = 1.;
+        for (int64_t j = 0; j + 1 < s.d; ++j) row[j + 1] = fields[j];
+        s.y[i] = fields.back();
+      }
+    } catch (const std::exception& e) {
+      errors[t] = e.what();
+    }
+  };
+  std::vector<std::thread> th;
+  for (int t = 1; t < threads; ++t) th.emplace_back(work, t);
+  work(0);
+  for (auto& x : th) x.join();
+  for (const std::string& e : errors)
+    if (!e.empty()) throw std::invalid_argument(e);
+  return s;
+}
+
+struct ShardCacheHeader {
+  char magic[8];        // "PLRSHARD"
+  uint32_t version;     // 1
+  uint32_t reserved;
+  int64_t n, d;
+  int64_t src_size;     // bytes of the text file the shard was parsed from
+  int64_t src_mtime_ns;
+};
+
+inline std::string cache_path(const std::string& input, int rank, int np) {
+  return input + ".plrshard." + std::to_string(rank) + "of" + std::to_string(np);
+}
+
+inline bool source_stamp(const std::string& input, int64_t& size, int64_t& mtime_ns) {
+  struct stat st;
+  if (stat(input.c_str(), &st) != 0) return false;
+  size = (int64_t)st.st_size;
+  mtime_ns = (int64_t)st.st_mtim.tv_sec * 1000000000LL + st.st_mtim.tv_nsec;
+  return true;
+}
+
+inline bool write_cache(const std::string& input, int rank, int np, const ParsedShard& s) {
+  ShardCacheHeader h;
+  memset(&h, 0, sizeof h);
+  memcpy(h.magic, "PLRSHARD", 8);
+  h.version = 1;
+  h.n = s.n;
+  h.d = s.d;
+  if (!source_stamp(input, h.src_size, h.src_mtime_ns)) return false;
+  const std::string path = cache_path(input, rank, np), tmp = path + ".tmp";
+  FILE* f = fopen(tmp.c_str(), "wb");
+  if (!f) return false;  // read-only input directory: run without a cache
+  bool ok = fwrite(&h, sizeof h, 1, f) == 1;
+  ok = ok && (s.X.empty() || fwrite(s.X.data(), sizeof(double), s.X.size(), f) == s.X.size());
+  ok = ok && (s.y.empty() || fwrite(s.y.data(), sizeof(double), s.y.size(), f) == s.y.size());
+  ok = (fclose(f) == 0) && ok;
+  if (ok) ok = rename(tmp.c_str(), path.c_str()) == 0;
+  if (!ok) remove(tmp.c_str());
+  return ok;
+}
+
+// Reads the header only and validates it against the source file.
+inline bool open_cache(const std::string& input, int rank, int np, ShardCacheHeader& h,
+                       FILE*& f) {
+  f = fopen(cache_path(input, rank, np).c_str(), "rb");
+  if (!f) return false;
+  int64_t size = 0, mtime = 0;
+  const bool ok = fread(&h, sizeof h, 1, f) == 1 && memcmp(h.magic, "PLRSHARD", 8) == 0 &&
+                  h.version == 1 && h.n >= 0 && h.d >= 1 && source_stamp(input, size, mtime) &&
+                  size == h.src_size && mtime == h.src_mtime_ns;
+  if (!ok) {
+    fclose(f);
+    f = nullptr;
+  }
+  return ok;
+}
+
+inline bool read_cache(const std::string& input, int rank, int np, ParsedShard& s) {
+  ShardCacheHeader h;
+  FILE* f = nullptr;
+  if (!open_cache(input, rank, np, h, f)) return false;
+  s.n = h.n;
+  s.d = h.d;
+  s.X.resize((size_t)h.n * h.d);
+  s.y.resize(h.n);
+  bool ok = s.X.empty() || fread(s.X.data(), sizeof(double), s.X.size(), f) == s.X.size();
+  ok = ok && (s.y.empty() || fread(s.y.data(), sizeof(double), s.y.size(), f) == s.y.size());
+  fclose(f);
+  return ok;
+}
+
+}  // namespace plr_ps

@@ -91,3 +91,16 @@ def test_csv_driver_follows_the_reference_call_order(server_info, oracle, tmp_pa
     # debug: one loss per round, at the theta read at the start of that round
     curve = np.array([float(t) for t in (outdir / "lr_loss_error_0").read_text().split()])
     assert curve.shape == (20,) and abs(curve[0] - np.log(2)) < 1e-6 and curve[-1] < curve[0]
+
+    # second run: the text is not parsed again (binary shard cache), same result
+    assert "shard cache hit" not in r.stdout
+    outdir2 = tmp_path / "out2"
+    cfg2 = json.loads(cfgf.read_text())
+    cfg2["output"] = str(outdir2) + "/"
+    cfgf.write_text(json.dumps(cfg2))
+    r2 = subprocess.run([os.path.join(PKG, "plr_lr_worker"), "--server_info", server_info,
+                         "--cfg_file", str(cfgf), "--theta0", "zero"],
+                        capture_output=True, text=True, timeout=110)
+    assert r2.returncode == 0, r2.stderr
+    assert "shard cache hit: 400 x 7" in r2.stdout
+    assert (outdir2 / "lr_theta_0").read_text() == (outdir / "lr_theta_0").read_text()

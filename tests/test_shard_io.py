@@ -1,0 +1,102 @@
+"""The host-side shard producer (paracel_amd/worker/shard_io.hpp) through its
+command-line tool: the reference's byte-range line partition
+(include/load/partition.hpp:57-86,121-139; the reference's own
+test/test_partition.cpp checks line continuity for np = 1..99), the CSV parser
+(lr.cpp:76-93) against the oracle's restatement, and the binary shard cache."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TOOL = os.path.join(ROOT, "paracel_amd", "plr_shard_tool")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _tool():
+    if not os.path.exists(TOOL):
+        subprocess.run(["make", "-C", os.path.join(ROOT, "paracel_amd", "worker"),
+                        os.path.join("..", "plr_shard_tool")], check=True)
+
+
+def run(*args):
+    return subprocess.run([TOOL] + [str(a) for a in args], capture_output=True, text=True)
+
+
+def make_csv(path, n, k, seed, ragged_len=True):
+    rng = np.random.default_rng(seed)
+    lines = []
+    for i in range(n):
+        kk = k
+        vals = rng.normal(size=kk)
+        # fields of varying printed width so that byte ranges cut lines at every position
+        fmt = ["%.1f", "%.6f", "%.12g", "%e"][i % 4] if ragged_len else "%.6f"
+        lines.append(",".join(fmt % v for v in vals) + ",%d" % (i % 2))
+    path.write_text("\n".join(lines) + "\n")
+    return lines
+
+
+@pytest.mark.parametrize("np_", [1, 2, 3, 4, 7, 16, 33, 99])
+def test_partition_covers_every_line_once(tmp_path, np_):
+    f = tmp_path / "a.csv"
+    lines = make_csv(f, 250, 5, 1)
+    got = []
+    for r in range(np_):
+        out = run("lines", f, r, np_)
+        assert out.returncode == 0, out.stderr
+        got.extend(out.stdout.splitlines())
+    assert got == lines                      # no line lost, duplicated or split; order kept
+
+
+def test_partition_when_a_boundary_hits_a_newline(tmp_path):
+    # 4 lines of 9 bytes + newline = 40 bytes; np=4 puts every boundary right after a newline
+    f = tmp_path / "b.csv"
+    lines = ["1.0,2.0,%d" % (i % 2) for i in range(4)]
+    f.write_text("\n".join(lines) + "\n")
+    for r in range(4):
+        assert run("lines", f, r, 4).stdout.splitlines() == [lines[r]]
+    # and np=8: every second range owns nothing
+    owned = [run("lines", f, r, 8).stdout.splitlines() for r in range(8)]
+    assert sum(owned, []) == lines
+
+
+def test_parser_matches_oracle_and_cache_roundtrip(tmp_path, oracle):
+    f = tmp_path / "c.csv"
+    lines = make_csv(f, 300, 7, 2)
+    out = run("parse", f, 0, 1)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.split() == ["300", "8"]            # bias column added: D = k + 1
+    raw = np.fromfile(str(f) + ".plrshard.0of1", dtype=np.uint8)
+    hdr = raw[:48]
+    assert bytes(hdr[:8]) == b"PLRSHARD"
+    n, d = np.frombuffer(hdr[16:32].tobytes(), dtype=np.int64)
+    body = np.frombuffer(raw[48:].tobytes(), dtype=np.float64)
+    X, y = body[: n * d].reshape(n, d), body[n * d:]
+    Xo, yo = oracle.local_parser(f.read_text())
+    np.testing.assert_array_equal(X, Xo)                 # bit-exact: same strtod
+    np.testing.assert_array_equal(y, yo)
+    assert np.all(X[:, 0] == 1.0)
+    assert run("info", f, 0, 1).stdout.split() == ["300", "8"]
+    # touching the source invalidates the cache
+    os.utime(f, ns=(1, 1))
+    assert run("info", f, 0, 1).returncode == 1
+    # per-rank shards concatenate to the whole
+    parts = []
+    for r in range(3):
+        assert run("parse", f, r, 3).returncode == 0
+        rr = np.fromfile(str(f) + ".plrshard.%dof3" % r, dtype=np.uint8)
+        nn, dd = np.frombuffer(rr[16:32].tobytes(), dtype=np.int64)
+        parts.append(np.frombuffer(rr[48:48 + 8 * nn * dd].tobytes(), dtype=np.float64).reshape(nn, dd))
+    np.testing.assert_array_equal(np.vstack(parts), Xo)
+
+
+def test_parser_errors(tmp_path):
+    f = tmp_path / "d.csv"
+    f.write_text("1,2,1\n1,1\n")
+    assert run("parse", f, 0, 1).returncode == 1        # ragged
+    f.write_text("1,abc,1\n")
+    assert run("parse", f, 0, 1).returncode == 1        # std::stod throws
+    f.write_text("3,,7,1\n")                            # empty field dropped (str_split)
+    assert run("parse", f, 0, 1).stdout.split() == ["1", "3"]
+    assert run("parse", tmp_path / "missing.csv", 0, 1).returncode == 1
