@@ -43,6 +43,10 @@ typedef enum {
 #define PLR_LOSS_STABLE 1u    /* log1p(exp(-|z|)) + max(-/+z, 0): same value,
                                  finite for any z                            */
 #define PLR_LOSS_NONE 2u      /* skip the loss (loss_sum receives 0)         */
+#define PLR_LOSS_SQUARED 3u   /* linear model instead of logistic: residual
+                                 x.theta - y, loss (x.theta - y)^2 -- the
+                                 ridge worker's calc_loss,
+                                 alg/regression/ridge/ridge.hpp:103-109       */
 
 /* Create a context on HIP device `device_id`.  Replaces nothing in the
  * reference (which has no device); it is the constructor-time set-up a
@@ -87,6 +91,10 @@ int plr_calc_loss(plr_ctx* ctx, const double* theta, double* loss_sum,
 
 /* lr.cpp:361-363: h_i for every resident row (n doubles out). */
 int plr_predict(plr_ctx* ctx, const double* theta, double* h_out);
+
+/* alg/regression/ridge/ridge.hpp:130-139: x_i.theta for every resident row
+ * (the linear model's prediction; n doubles out). */
+int plr_predict_linear(plr_ctx* ctx, const double* theta, double* z_out);
 
 /* Shape of the resident shard (0,0 before plr_set_data). */
 int plr_get_shape(const plr_ctx* ctx, int64_t* n, int64_t* d);

@@ -189,6 +189,31 @@ int64_t oracle_local_parser(const char* text, int64_t nlines, char sep,
   return D;
 }
 
+double oracle_ridge_loss_sum(const double* X, int64_t n, int64_t d, int64_t ldx,
+                             const double* y, const double* theta) {
+  double loss = 0.;
+  for (int64_t i = 0; i < n; ++i) {
+    double h = dot_seq(X + i * ldx, theta, d) - y[i];
+    loss += h * h;
+  }
+  return loss;
+}
+
+void oracle_predict_linear(const double* X, int64_t n, int64_t d, int64_t ldx,
+                           const double* theta, double* z_out) {
+  for (int64_t i = 0; i < n; ++i) z_out[i] = dot_seq(X + i * ldx, theta, d);
+}
+
+void oracle_lsq_gsum(const double* X, int64_t n, int64_t d, int64_t ldx,
+                     const double* y, const double* theta, double* gsum) {
+  for (int64_t j = 0; j < d; ++j) gsum[j] = 0.;
+  for (int64_t i = 0; i < n; ++i) {
+    const double* x = X + i * ldx;
+    double r = dot_seq(x, theta, d) - y[i];
+    for (int64_t j = 0; j < d; ++j) gsum[j] += r * x[j];
+  }
+}
+
 void oracle_gsum_hp(const double* X, int64_t n, int64_t d, int64_t ldx,
                     const double* y, const double* theta, double* gsum) {
   vector<long double> acc(d, 0.L);

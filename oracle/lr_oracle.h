@@ -97,6 +97,17 @@ void oracle_train_dgd_workers(const double* X, int64_t n, int64_t d, int64_t ldx
 int64_t oracle_local_parser(const char* text, int64_t nlines, char sep,
                             double* X_out, double* y_out, int64_t k_expected);
 
+/* alg/regression/ridge/ridge.hpp:103-109: sum over rows of (x.theta - y)^2,
+ * row order, from 0.0 (the local sum before the all-reduces of :110-113). */
+double oracle_ridge_loss_sum(const double* X, int64_t n, int64_t d, int64_t ldx,
+                             const double* y, const double* theta);
+/* ridge.hpp:130-139: x_i.theta per row. */
+void oracle_predict_linear(const double* X, int64_t n, int64_t d, int64_t ldx,
+                           const double* theta, double* z_out);
+/* least-squares counterpart of oracle_gsum: X^T (X theta - y), row by row. */
+void oracle_lsq_gsum(const double* X, int64_t n, int64_t d, int64_t ldx,
+                     const double* y, const double* theta, double* gsum);
+
 /* long-double arbiters: same formulas, every sum and exp/log in 80-bit. */
 void oracle_gsum_hp(const double* X, int64_t n, int64_t d, int64_t ldx,
                     const double* y, const double* theta, double* gsum);

@@ -29,14 +29,15 @@ def load():
         L.oracle_dgd_delta.restype = None
         L.oracle_dgd_delta.argtypes = shp + [_dp, _dp, C.c_double, C.c_double, _i64p, _dp]
         for f in ("oracle_calc_loss_sum", "oracle_calc_loss", "oracle_calc_loss_sum_hp",
-                  "oracle_stable_loss_sum_hp"):
+                  "oracle_stable_loss_sum_hp", "oracle_ridge_loss_sum"):
             getattr(L, f).restype = C.c_double
             getattr(L, f).argtypes = shp + [_dp, _dp]
         L.oracle_theta_update.restype = None
         L.oracle_theta_update.argtypes = [_dp, _dp, C.c_int64, _dp]
-        L.oracle_predict.restype = None
-        L.oracle_predict.argtypes = shp + [_dp, _dp]
-        for f in ("oracle_gsum", "oracle_gsum_hp"):
+        for f in ("oracle_predict", "oracle_predict_linear"):
+            getattr(L, f).restype = None
+            getattr(L, f).argtypes = shp + [_dp, _dp]
+        for f in ("oracle_gsum", "oracle_gsum_hp", "oracle_lsq_gsum"):
             getattr(L, f).restype = None
             getattr(L, f).argtypes = shp + [_dp, _dp, _dp]
         L.oracle_train_dgd.restype = None
@@ -120,6 +121,26 @@ def calc_loss_sum_hp(X, y, theta):
 
 def stable_loss_sum_hp(X, y, theta):
     return _loss("oracle_stable_loss_sum_hp", X, y, theta)
+
+
+def ridge_loss_sum(X, y, theta):
+    return _loss("oracle_ridge_loss_sum", X, y, theta)
+
+
+def predict_linear(X, theta):
+    X, n, d = _shape(X)
+    theta = _c(theta)
+    out = np.empty(n)
+    load().oracle_predict_linear(_p(X), n, d, d, _p(theta), _p(out))
+    return out
+
+
+def lsq_gsum(X, y, theta):
+    X, n, d = _shape(X)
+    y, theta = _c(y), _c(theta)
+    out = np.empty(d)
+    load().oracle_lsq_gsum(_p(X), n, d, d, _p(y), _p(theta), _p(out))
+    return out
 
 
 def theta_update(a, b):

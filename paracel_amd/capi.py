@@ -12,6 +12,7 @@ import numpy as np
 PLR_LOSS_REFERENCE = 0
 PLR_LOSS_STABLE = 1
 PLR_LOSS_NONE = 2
+PLR_LOSS_SQUARED = 3
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -29,6 +30,7 @@ SYMBOLS = [
     ("plr_dgd_delta", C.c_int, [_ctx, _dp, C.c_double, C.c_double, _dp, _dp]),
     ("plr_calc_loss", C.c_int, [_ctx, _dp, _dp, _i64p, C.c_uint]),
     ("plr_predict", C.c_int, [_ctx, _dp, _dp]),
+    ("plr_predict_linear", C.c_int, [_ctx, _dp, _dp]),
     ("plr_get_shape", C.c_int, [_ctx, _i64p, _i64p]),
     ("plr_get_timing", C.c_int, [_ctx, _dp, _dp, _i64p]),
     ("plr_reset_timing", C.c_int, [_ctx]),
@@ -173,6 +175,13 @@ class Plr:
         h = np.empty(n, dtype=np.float64)
         self._check(self._lib.plr_predict(self._h, _p(theta), _p(h)))
         return h
+
+    def predict_linear(self, theta):
+        n, d = self.shape
+        theta = _vec(theta, d, "theta")
+        z = np.empty(n, dtype=np.float64)
+        self._check(self._lib.plr_predict_linear(self._h, _p(theta), _p(z)))
+        return z
 
     # -- timing / info ----------------------------------------------------
     def timing(self):

@@ -237,7 +237,7 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
   return PLR_OK;
 }
 
-enum PassKind { kPassGrad, kPassDelta, kPassLoss, kPassPredict };
+enum PassKind { kPassGrad, kPassDelta, kPassLoss, kPassPredict, kPassPredictLinear };
 
 // theta -> device, streaming kernel (timed), finishing kernel, results ->
 // pinned host.  Returns after the stream has drained.
@@ -245,7 +245,7 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
              double alpha, double beta) {
   if (!c->have_data) return fail(c, PLR_ERR_NODATA, "no shard resident: call plr_set_data first");
   if (!theta) return fail(c, PLR_ERR_INVALID, "theta must not be NULL");
-  if (loss_mode > plr::kLossNone) return fail(c, PLR_ERR_INVALID, "unknown loss flag");
+  if (loss_mode > plr::kLossSquared) return fail(c, PLR_ERR_INVALID, "unknown loss flag");
   PLR_HIP(c, hipSetDevice(c->device));
   const Variant* v = c->var;
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
@@ -255,21 +255,23 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
   memcpy(c->h_theta, theta, (size_t)c->d * sizeof(double));
   PLR_HIP(c, hipMemcpyAsync(c->d_theta, c->h_theta, (size_t)c->d * sizeof(double),
                             hipMemcpyHostToDevice, c->stream));
-  if (kind == kPassPredict && !c->d_h && c->n > 0)
+  const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
+  if (predict && !c->d_h && c->n > 0)
     PLR_HIP(c, hipMalloc(&c->d_h, (size_t)c->n * sizeof(double)));
 
   PassArgs pa;
   pa.X = c->dX;
-  pa.y = (kind == kPassPredict) ? nullptr : c->dy;
+  pa.y = predict ? nullptr : c->dy;
   pa.theta = c->d_theta;
   pa.part_g = c->d_part_g;
   pa.part_loss = c->d_part_loss;
-  pa.h_out = (kind == kPassPredict) ? c->d_h : nullptr;
+  pa.h_out = predict ? c->d_h : nullptr;
   pa.n = c->n;
   pa.pitch = c->pitch;
   pa.ntiles = ceil_div(c->n, v->R);
   pa.nch_rt = c->nch_rt;
-  pa.loss_mode = (kind == kPassPredict) ? (unsigned)plr::kLossNone : loss_mode;
+  pa.loss_mode = predict ? (unsigned)plr::kLossNone : loss_mode;
+  pa.identity_link = (kind == kPassPredictLinear || loss_mode == plr::kLossSquared) ? 1 : 0;
 
   PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
   hipLaunchKernelGGL(v->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
@@ -277,7 +279,7 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
   PLR_HIP(c, hipGetLastError());
   PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
 
-  if (kind != kPassPredict) {
+  if (!predict) {
     FinishArgs fa;
     fa.part_g = c->d_part_g;
     fa.part_loss = c->d_part_loss;
@@ -422,14 +424,22 @@ int plr_calc_loss(plr_ctx* c, const double* theta, double* loss_sum, int64_t* n_
   return PLR_OK;
 }
 
-int plr_predict(plr_ctx* c, const double* theta, double* h_out) {
+static int predict_rows(plr_ctx* c, PassKind kind, const double* theta, double* out) {
   if (!c) return PLR_ERR_INVALID;
-  if (!h_out && c->n > 0) return fail(c, PLR_ERR_INVALID, "h_out must not be NULL");
-  int rc = run_pass(c, kPassPredict, theta, plr::kLossNone, 0., 0.);
+  if (!out && c->n > 0) return fail(c, PLR_ERR_INVALID, "output must not be NULL");
+  int rc = run_pass(c, kind, theta, plr::kLossNone, 0., 0.);
   if (rc != PLR_OK) return rc;
   if (c->n > 0)
-    PLR_HIP(c, hipMemcpy(h_out, c->d_h, (size_t)c->n * sizeof(double), hipMemcpyDeviceToHost));
+    PLR_HIP(c, hipMemcpy(out, c->d_h, (size_t)c->n * sizeof(double), hipMemcpyDeviceToHost));
   return PLR_OK;
+}
+
+int plr_predict(plr_ctx* c, const double* theta, double* h_out) {
+  return predict_rows(c, kPassPredict, theta, h_out);
+}
+
+int plr_predict_linear(plr_ctx* c, const double* theta, double* z_out) {
+  return predict_rows(c, kPassPredictLinear, theta, z_out);
 }
 
 int plr_probe_read_bandwidth(plr_ctx* c, int reps, double* gb_per_s) {

@@ -59,6 +59,7 @@ enum : unsigned {
   kLossReference = 0u,
   kLossStable = 1u,
   kLossNone = 2u,
+  kLossSquared = 3u,  // identity link: residual z - y, loss (z - y)^2
 };
 
 struct PassArgs {
@@ -73,6 +74,7 @@ struct PassArgs {
   int64_t ntiles;        // ceil(n / R)
   int nch_rt;            // chunks per wave actually used (<= NCH)
   unsigned loss_mode;
+  int identity_link;     // 1: h = z (linear model), 0: h = sigmoid(z)
 };
 
 // Row held by `lane` after the transposing reduction over R rows.
@@ -243,14 +245,21 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
   }
 
   // ---- sigmoid, residual, loss for the row this lane holds ----
-  const double e = exp(-z);
-  const double h = 1. / (1. + e);
+  double h;
+  if (a.identity_link) {
+    h = z;
+  } else {
+    const double e = exp(-z);
+    h = 1. / (1. + e);
+  }
   const double res = my_valid ? (h - yv) : 0.;
   if (a.h_out && my_valid && lane < R && w.wc == 0) a.h_out[myrow_g] = h;
   if (a.loss_mode != kLossNone) {
     double l;
     if (a.loss_mode == kLossReference) {
       l = -log((yv == 1.) ? h : 1. - h);
+    } else if (a.loss_mode == kLossSquared) {
+      l = (h - yv) * (h - yv);
     } else {
       const double sgn = (yv == 1.) ? -z : z;  // loss = log(1 + exp(sgn))
       l = log1p(exp(-fabs(sgn))) + fmax(sgn, 0.);

@@ -89,6 +89,24 @@ def test_calc_loss_and_predict(plr, oracle, gen, n, d):
     assert abs(loss2 - loss) <= 1e-12 * abs(loss)
 
 
+@pytest.mark.parametrize("n,d", [(999, 100), (2051, 1000), (70, 8193)])
+def test_linear_model_pieces(plr, oracle, gen, n, d):
+    # the ridge worker's loss and prediction (alg/regression/ridge/ridge.hpp:103-109,130-139)
+    # and the least-squares gradient, on the same streaming pass with the identity link
+    X, _, th = make(gen, n, d)
+    y = gen.gen_vec(99, gen.STREAM_THETA, n)
+    plr.set_data(X, y)
+    z = plr.predict_linear(th)
+    np.testing.assert_allclose(z, oracle.predict_linear(X, th), rtol=0, atol=1e-13)
+    loss, n_out = plr.calc_loss(th, 3)
+    want = oracle.ridge_loss_sum(X, y, th)
+    assert n_out == n and abs(loss - want) <= 1e-12 * want
+    g, loss2, _ = plr.loss_grad(th, 3)
+    assert rel(g, oracle.lsq_gsum(X, y, th)) <= GRAD_TOL
+    assert rel(g, X.T @ (X @ th - y)) <= 1e-12
+    assert abs(loss2 - want) <= 1e-12 * want
+
+
 def test_theta_zero_closed_forms(plr, gen):
     # theta = 0 => h = 1/2 exactly: gsum = X^T (1/2 - y) (a plain GEMV), loss = n ln 2
     X, y, _ = make(gen, 3001, 300)

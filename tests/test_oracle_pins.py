@@ -176,6 +176,20 @@ def test_loss_closed_forms_and_symmetry(oracle):
     assert abs(oracle.stable_loss_sum_hp(np.array([[40.0]]), np.zeros(1), np.ones(1)) - 40.0) <= 1e-14
 
 
+def test_ridge_pieces_against_numpy(oracle):
+    # ridge.hpp:103-109,130-139: squared residuals and the linear prediction
+    X, _, th = rand_case(300, 17, 11)
+    y = np.random.default_rng(12).normal(size=300)
+    z = X @ th
+    np.testing.assert_allclose(oracle.predict_linear(X, th), z, rtol=1e-13, atol=1e-14)
+    assert abs(oracle.ridge_loss_sum(X, y, th) - np.sum((z - y) ** 2)) <= 1e-12 * np.sum((z - y) ** 2)
+    assert rel(oracle.lsq_gsum(X, y, th), X.T @ (z - y)) <= 1e-13
+    # exact closed forms: theta = 0 -> loss = sum y^2, gsum = -X^T y; y = X theta -> 0
+    assert abs(oracle.ridge_loss_sum(X, y, np.zeros(17)) - np.sum(y * y)) <= 1e-12 * np.sum(y * y)
+    assert rel(oracle.lsq_gsum(X, y, np.zeros(17)), -(X.T @ y)) <= 1e-13
+    assert oracle.ridge_loss_sum(X, oracle.predict_linear(X, th), th) == 0.0
+
+
 def test_theta_update_is_elementwise_add(oracle):
     a, b = np.array([1.23, -4.0, 1e300]), np.array([3.21, 4.0, 1e300])
     np.testing.assert_array_equal(oracle.theta_update(a, b), a + b)   # test_proxy.cpp:45-54: 1.23+3.21
