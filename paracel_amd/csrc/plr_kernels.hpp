@@ -431,6 +431,17 @@ __global__ __launch_bounds__(256) void read_probe(const v2d* base, int64_t ntile
   if (acc.x + acc.y == 1.2345e300) sink[0] = acc.x;  // keeps the loads alive
 }
 
+// theta arrives in pinned, device-mapped host memory; this one-workgroup
+// kernel moves it into the zero-padded device copy the pass reads.  A kernel
+// on the pass's own stream instead of a copy command: no hand-over between
+// the copy engine and the compute queue in front of every step.
+__global__ __launch_bounds__(256) void stage_theta(const double* __restrict__ host_theta,
+                                                   double* __restrict__ dev_theta, int64_t d) {
+  for (int64_t i = threadIdx.x + (int64_t)blockIdx.x * blockDim.x; i < d;
+       i += (int64_t)gridDim.x * blockDim.x)
+    dev_theta[i] = host_theta[i];
+}
+
 struct FinishArgs {
   const double* part_g;   // [nparts][pitch]
   const double* part_loss;  // [nparts]
