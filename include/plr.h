@@ -85,6 +85,17 @@ int plr_loss_grad(plr_ctx* ctx, const double* theta, double* gsum,
 int plr_dgd_delta(plr_ctx* ctx, const double* theta, double alpha, double beta,
                   double* delta, double* loss_sum);
 
+/* `rounds` full-batch rounds with theta kept on the device: each round is
+ * lr.cpp:125-138 (delta at the current theta) followed by the reducer's
+ * theta += delta (update.cpp:26-32) -- the single-process training loop of
+ * tool/lr_serial.cpp:95-110, without a host round trip per round.  theta is
+ * read at entry and overwritten with the result.  loss_curve (nullable,
+ * `rounds` doubles) receives the loss sum (lr.cpp:322-330) at the theta each
+ * round STARTED from.  With a parameter server in the loop use plr_dgd_delta
+ * per round instead. */
+int plr_train_dgd(plr_ctx* ctx, double* theta, double alpha, double beta, int rounds,
+                  double* loss_curve);
+
 /* lr.cpp:322-330: the loss pass alone (no gradient). */
 int plr_calc_loss(plr_ctx* ctx, const double* theta, double* loss_sum,
                   int64_t* n_out, unsigned flags);

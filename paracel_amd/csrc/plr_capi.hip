@@ -79,6 +79,9 @@ struct plr_ctx {
   double* d_part_g = nullptr;   // grid x pitch
   double* d_part_loss = nullptr;  // max(grid, grid_nograd)
   double* d_h = nullptr;        // n (predict), lazily allocated
+  double* d_curve = nullptr;    // per-round losses of plr_train_dgd, lazily allocated
+  double* d_train_out = nullptr;  // d + 1: where training rounds put delta (never read back)
+  int curve_len = 0;
   double* h_theta = nullptr;    // pinned + device-mapped, theta_len
   double* h_theta_dev = nullptr;  // the device's address of h_theta
   double* h_out = nullptr;      // pinned + device-mapped, d + 1: finish_pass writes it
@@ -119,12 +122,15 @@ void free_shape(plr_ctx* c) {
   if (c->d_part_g) (void)hipFree(c->d_part_g);
   if (c->d_part_loss) (void)hipFree(c->d_part_loss);
   if (c->d_h) (void)hipFree(c->d_h);
+  if (c->d_curve) (void)hipFree(c->d_curve);
+  if (c->d_train_out) (void)hipFree(c->d_train_out);
   if (c->h_theta) (void)hipHostFree(c->h_theta);
   if (c->h_out) (void)hipHostFree(c->h_out);
-  c->dX = c->dy = c->d_theta = c->d_part_g = c->d_part_loss = c->d_h =
-      c->h_theta = c->h_theta_dev = c->h_out = c->h_out_dev = nullptr;
+  c->dX = c->dy = c->d_theta = c->d_part_g = c->d_part_loss = c->d_h = c->d_curve =
+      c->d_train_out = c->h_theta = c->h_theta_dev = c->h_out = c->h_out_dev = nullptr;
   c->n = c->d = c->pitch = 0;
   c->have_data = false;
+  c->curve_len = 0;
   c->var = nullptr;
   c->info.clear();
 }
@@ -228,7 +234,7 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
   if (row0 < 0 || nrows < 0 || row0 + nrows > c->n)
     return fail(c, PLR_ERR_INVALID, "row range outside the reserved shard");
   PLR_HIP(c, hipSetDevice(c->device));
-  if (ldx == c->pitch)  // same pitch on both sides: one linear copy
+  if (ldx == c->pitch && c->d == c->pitch)  // same pitch, no pad column: one linear copy
     PLR_HIP(c, hipMemcpy(c->dX + row0 * c->pitch, X,
                          (size_t)nrows * c->pitch * sizeof(double), hipMemcpyHostToDevice));
   else
@@ -242,29 +248,18 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
 
 enum PassKind { kPassGrad, kPassDelta, kPassLoss, kPassPredict, kPassPredictLinear };
 
-// theta -> device, streaming kernel (timed), finishing kernel, results ->
-// pinned host.  Returns after the stream has drained.
-int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
-             double alpha, double beta) {
-  if (!c->have_data) return fail(c, PLR_ERR_NODATA, "no shard resident: call plr_set_data first");
-  if (!theta) return fail(c, PLR_ERR_INVALID, "theta must not be NULL");
-  if (loss_mode > plr::kLossSquared) return fail(c, PLR_ERR_INVALID, "unknown loss flag");
-  PLR_HIP(c, hipSetDevice(c->device));
+// Enqueue one pass on the context's stream: streaming kernel (between the two
+// timing events) and finishing kernel.  theta must already be in d_theta.
+// `out` receives d values + the loss; train_round >= 0 makes the finishing
+// kernel also apply delta to the device theta and store the loss in
+// d_curve[train_round].
+int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, double beta,
+                 double* out, int train_round) {
   const Variant* v = c->var;
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
+  const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
   const int grid = grad ? c->grid : c->grid_nograd;
   const int threads = plr::kWave * v->wcol * v->wrow;
-
-  memcpy(c->h_theta, theta, (size_t)c->d * sizeof(double));
-  {
-    const int sgrid = (int)((c->d + 1023) / 1024 > 64 ? 64 : (c->d + 1023) / 1024);
-    hipLaunchKernelGGL(plr::stage_theta, dim3(sgrid), dim3(256), 0, c->stream,
-                       (const double*)c->h_theta_dev, c->d_theta, c->d);
-    PLR_HIP(c, hipGetLastError());
-  }
-  const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
-  if (predict && !c->d_h && c->n > 0)
-    PLR_HIP(c, hipMalloc(&c->d_h, (size_t)c->n * sizeof(double)));
 
   PassArgs pa;
   pa.X = c->dX;
@@ -291,28 +286,61 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
     fa.part_g = c->d_part_g;
     fa.part_loss = c->d_part_loss;
     fa.theta = c->d_theta;
-    fa.out = c->h_out_dev;
+    fa.out = out;
     fa.pitch = c->pitch;
     fa.d = c->d;
     fa.n = c->n;
     fa.nparts = grid;
-    fa.delta_mode = (kind == kPassDelta) ? 1 : 0;
+    fa.delta_mode = (kind == kPassDelta) ? (train_round >= 0 ? 2 : 1) : 0;
     fa.have_grad = grad ? 1 : 0;
     fa.alpha = alpha;
     fa.coff2 = 2. * beta * alpha;
+    fa.theta_rw = c->d_theta;
+    fa.loss_slot = (train_round >= 0 && c->d_curve) ? c->d_curve + train_round : nullptr;
     const int fgrid = grad ? (int)ceil_div(c->d, plr::kFinCols) : 1;
     hipLaunchKernelGGL(plr::finish_pass, dim3(fgrid),
                        dim3(plr::kFinCols * plr::kFinSlices), 0, c->stream, fa);
     PLR_HIP(c, hipGetLastError());
   }
-  // (measured: hipStreamSynchronize returns ~7 us sooner than a hipStreamQuery poll loop)
-  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  return PLR_OK;
+}
+
+// theta (host) -> pinned staging -> device copy, by a kernel on the stream
+int stage_theta_from_host(plr_ctx* c, const double* theta) {
+  memcpy(c->h_theta, theta, (size_t)c->d * sizeof(double));
+  const int sgrid = (int)((c->d + 1023) / 1024 > 64 ? 64 : (c->d + 1023) / 1024);
+  hipLaunchKernelGGL(plr::stage_theta, dim3(sgrid), dim3(256), 0, c->stream,
+                     (const double*)c->h_theta_dev, c->d_theta, c->d);
+  PLR_HIP(c, hipGetLastError());
+  return PLR_OK;
+}
+
+int account_timing(plr_ctx* c) {
   float ms = 0.f;
   PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
   c->last_ms = ms;
   c->sum_ms += ms;
   c->launches += 1;
   return PLR_OK;
+}
+
+// One synchronous pass: theta in, kernels, results in the mapped host buffer.
+int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
+             double alpha, double beta) {
+  if (!c->have_data) return fail(c, PLR_ERR_NODATA, "no shard resident: call plr_set_data first");
+  if (!theta) return fail(c, PLR_ERR_INVALID, "theta must not be NULL");
+  if (loss_mode > plr::kLossSquared) return fail(c, PLR_ERR_INVALID, "unknown loss flag");
+  PLR_HIP(c, hipSetDevice(c->device));
+  const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
+  if (predict && !c->d_h && c->n > 0)
+    PLR_HIP(c, hipMalloc(&c->d_h, (size_t)c->n * sizeof(double)));
+  int rc = stage_theta_from_host(c, theta);
+  if (rc != PLR_OK) return rc;
+  rc = enqueue_pass(c, kind, loss_mode, alpha, beta, c->h_out_dev, -1);
+  if (rc != PLR_OK) return rc;
+  // (measured: hipStreamSynchronize returns ~7 us sooner than a hipStreamQuery poll loop)
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  return account_timing(c);
 }
 
 }  // namespace
@@ -412,6 +440,41 @@ int plr_dgd_delta(plr_ctx* c, const double* theta, double alpha, double beta,
   memcpy(delta, c->h_out, (size_t)c->d * sizeof(double));
   if (loss_sum) *loss_sum = c->h_out[c->d];
   return PLR_OK;
+}
+
+int plr_train_dgd(plr_ctx* c, double* theta, double alpha, double beta, int rounds,
+                  double* loss_curve) {
+  if (!c) return PLR_ERR_INVALID;
+  if (!c->have_data) return fail(c, PLR_ERR_NODATA, "no shard resident: call plr_set_data first");
+  if (!theta || rounds < 0) return fail(c, PLR_ERR_INVALID, "need theta and rounds >= 0");
+  if (rounds == 0) return PLR_OK;
+  PLR_HIP(c, hipSetDevice(c->device));
+  if (c->curve_len < rounds) {
+    if (c->d_curve) PLR_HIP(c, hipFree(c->d_curve));
+    c->d_curve = nullptr;
+    PLR_HIP(c, hipMalloc(&c->d_curve, (size_t)rounds * sizeof(double)));
+    c->curve_len = rounds;
+  }
+  if (!c->d_train_out)
+    PLR_HIP(c, hipMalloc(&c->d_train_out, (size_t)(c->d + 1) * sizeof(double)));
+  int rc = stage_theta_from_host(c, theta);
+  if (rc != PLR_OK) return rc;
+  const unsigned loss_mode = loss_curve ? plr::kLossReference : plr::kLossNone;
+  // every round is enqueued back to back; theta never leaves the device
+  for (int rd = 0; rd < rounds; ++rd) {
+    rc = enqueue_pass(c, kPassDelta, loss_mode, alpha, beta, c->d_train_out, rd);
+    if (rc != PLR_OK) return rc;
+  }
+  PLR_HIP(c, hipMemcpyAsync(c->h_theta, c->d_theta, (size_t)c->d * sizeof(double),
+                            hipMemcpyDeviceToHost, c->stream));
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  memcpy(theta, c->h_theta, (size_t)c->d * sizeof(double));
+  if (loss_curve)
+    PLR_HIP(c, hipMemcpy(loss_curve, c->d_curve, (size_t)rounds * sizeof(double),
+                         hipMemcpyDeviceToHost));
+  // the timing events were re-recorded every round: only the last round's pair is meaningful
+  rc = account_timing(c);
+  return rc;
 }
 
 int plr_calc_loss(plr_ctx* c, const double* theta, double* loss_sum, int64_t* n_out,

@@ -451,8 +451,12 @@ struct FinishArgs {
   int64_t d;
   int64_t n;
   int nparts;
-  int delta_mode;         // 0: out = gsum; 1: out = -alpha*gsum - coff2*n*theta
+  int delta_mode;         // 0: out = gsum; 1: out = -alpha*gsum - coff2*n*theta;
+                          // 2: as 1, and theta_rw += delta (the server-side add,
+                          //    done in place on the device copy of theta)
   int have_grad;
+  double* theta_rw;       // delta_mode 2 only: the device theta to update
+  double* loss_slot;      // nullable: also store the loss sum here
   double alpha;
   double coff2;
 };
@@ -479,8 +483,11 @@ __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a
       double g = sm[0][cx];
 #pragma unroll
       for (int k = 1; k < kFinSlices; ++k) g += sm[k][cx];
-      if (a.delta_mode)
-        g = -a.alpha * g - (a.coff2 * (double)a.n) * a.theta[col];
+      if (a.delta_mode) {
+        const double th = a.theta[col];
+        g = -a.alpha * g - (a.coff2 * (double)a.n) * th;
+        if (a.delta_mode == 2) a.theta_rw[col] = th + g;  // this thread owns column col
+      }
       a.out[col] = g;
     }
     __syncthreads();
@@ -496,7 +503,10 @@ __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a
 #pragma unroll
       for (int k = 1; k < kFinSlices; ++k) t += sm[k][cx];
       t = wave_sum(t);
-      if (threadIdx.x == 0) a.out[a.d] = t;
+      if (threadIdx.x == 0) {
+        a.out[a.d] = t;
+        if (a.loss_slot) *a.loss_slot = t;
+      }
     }
   }
 }

@@ -188,6 +188,18 @@ def test_pitched_input(plr, oracle, gen):
     assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
 
 
+def test_host_pitch_equal_to_device_pitch_with_pad_column(plr, oracle, gen):
+    # d odd -> device pitch d+1; a host buffer with the same pitch holds foreign values in
+    # that extra column, which must not reach the device's zero pad column
+    X, y, th = make(gen, 300, 333)
+    wide = np.full((300, 334), np.nan)
+    wide[:, :333] = X
+    plr.set_data(wide[:, :333], y)
+    g, loss, _ = plr.loss_grad(th)
+    assert np.all(np.isfinite(g)) and np.isfinite(loss)
+    assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
+
+
 def test_saturated_rows_stable_vs_reference_loss(plr, oracle, gen):
     # rows scaled x100 saturate the sigmoid: the reference formula returns
     # +inf once exp(-z) < 2^-53 (lr.cpp:328 with h == 1.0); the stable form
@@ -283,3 +295,28 @@ def test_config1_trajectory_100_iterations(plr, oracle, gen):
     assert rel(theta, theta_ref) <= 1e-8
     loss, n = plr.calc_loss(theta)
     assert abs(loss / n - oracle.calc_loss(X, y, theta_ref)) <= 1e-9
+
+
+def test_device_resident_training_matches_oracle_and_per_round_path(plr, oracle, gen):
+    # tool/lr_serial.cpp:95-110: rounds of delta + theta += delta, theta kept on the device
+    cfg = gen.configs()["c1_dense_100k_x_100"].scaled(30000)
+    X, y = cfg.rows(0, cfg.n)
+    alpha, beta = cfg.lr / cfg.n, cfg.beta
+    plr.set_data(X, y)
+    theta, curve = plr.train_dgd(np.zeros(cfg.d), alpha, beta, 100, want_curve=True)
+    theta_ref = oracle.train_dgd(X, y, np.zeros(cfg.d), alpha, beta, 100)
+    assert rel(theta, theta_ref) <= 1e-8
+    # the same rounds driven from the host, one plr_dgd_delta per round: identical bits
+    th = np.zeros(cfg.d)
+    losses = []
+    for _ in range(100):
+        delta, l = plr.dgd_delta(th, alpha, beta)
+        losses.append(l)
+        th = th + delta
+    np.testing.assert_array_equal(theta, th)
+    np.testing.assert_array_equal(curve, np.array(losses))
+    assert abs(curve[0] - cfg.n * np.log(2.0)) <= 1e-12 * cfg.n and curve[-1] < curve[0]
+    # zero rounds leave theta alone; no curve requested works too
+    t0 = gen.gen_vec(5, gen.STREAM_THETA, cfg.d)
+    np.testing.assert_array_equal(plr.train_dgd(t0, alpha, beta, 0), t0)
+    np.testing.assert_array_equal(plr.train_dgd(np.zeros(cfg.d), alpha, beta, 100), theta)
