@@ -45,6 +45,9 @@ def parse_args():
     ap.add_argument("--rows", type=int, default=0, help="override n (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-rows", type=int, default=0)
+    ap.add_argument("--train", action="store_true",
+                    help="device-resident training rounds (plr_train_dgd, theta stays in HBM) "
+                         "with the final theta checked against the CPU oracle")
     ap.add_argument("--e2e", action="store_true",
                     help="end-to-end rounds through the host parameter server (C++ worker + "
                          "plr_ps_server over ZeroMQ) instead of the bare gradient step")
@@ -106,6 +109,47 @@ def cpu_baseline(cfg, Xs, ys, theta):
         "loss_pass_seconds_pcore_scaled": tlp * scale,
         "cpu_model": model,
     }
+
+
+def run_train(a, cfg):
+    """steps rounds of delta + theta += delta on the device (tool/lr_serial.cpp:95-110)."""
+    import numpy as np
+
+    from paracel_amd import Plr
+
+    ctx = Plr(0)
+    X, y = cfg.rows(0, cfg.n)
+    ctx.set_data(X, y)
+    theta0 = np.zeros(cfg.d)
+    ctx.train_dgd(theta0, cfg.alpha, cfg.beta, max(1, a.warmup))
+    t0 = time.perf_counter()
+    theta = ctx.train_dgd(theta0, cfg.alpha, cfg.beta, a.steps)
+    sec = time.perf_counter() - t0
+    out = {
+        "metric": "lr_train_iters_per_sec", "value": a.steps / sec, "unit": "iters/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": 1e3 * sec / a.steps,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
+        "data": "synthetic",
+        "config": {"workload": cfg.name + " device-resident training", "n": cfg.n, "d": cfg.d,
+                   "step": "plr_train_dgd: delta at theta (fused pass) + theta += delta, theta "
+                           "kept in HBM for all rounds", "alpha": cfg.alpha, "beta": cfg.beta,
+                   "kernel": ctx.kernel_info()},
+        "theta_rel_err_vs_cpu": None,
+    }
+    if not a.no_cpu_baseline:
+        from oracle import oracle
+
+        t0 = time.perf_counter()
+        theta_cpu = oracle.train_dgd(X, y, theta0, cfg.alpha, cfg.beta, a.steps)
+        sec_cpu = time.perf_counter() - t0
+        out["theta_rel_err_vs_cpu"] = float(np.linalg.norm(theta - theta_cpu) /
+                                            np.linalg.norm(theta_cpu))
+        out["cpu_baseline"] = {"value": a.steps / sec_cpu, "unit": "iters/s", "cores": 1,
+                               "kind": "port",
+                               "sample": "all %d rounds on the full shard, 1 core "
+                                         "(tool/lr_serial.cpp learning loop restated)" % a.steps}
+    ctx.close()
+    print(json.dumps(out), flush=True)
 
 
 def run_e2e(a, cfg):
@@ -193,6 +237,9 @@ def main():
         cfg = cfg.scaled(a.rows)
     if a.e2e:
         run_e2e(a, cfg)
+        return
+    if a.train:
+        run_train(a, cfg)
         return
     theta = cfg.theta()
 
