@@ -41,3 +41,22 @@ def test_product_does_not_touch_the_oracle():
                     if "oracle" in open(os.path.join(dp, f), errors="ignore").read():
                         bad.append(os.path.join(dp, f))
     assert not bad, bad
+
+
+def test_no_silent_cpu_path_without_a_gpu():
+    """Without a usable GPU the library must refuse to create a context (loudly, with a
+    message) -- there is no CPU fallback to fall into.  On a GPU box this test checks the
+    out-of-range device id instead."""
+    import pytest
+
+    from paracel_amd import Plr, PlrError
+
+    try:
+        import torch
+
+        have_gpu = torch.cuda.device_count() > 0
+    except Exception:  # torch is only used to count devices without initialising HIP here
+        have_gpu = os.path.exists("/dev/kfd")
+    with pytest.raises(PlrError) as e:
+        Plr(4096 if have_gpu else 0)
+    assert e.value.code in (-1, -2) and len(str(e.value)) > 20
