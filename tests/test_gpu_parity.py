@@ -36,6 +36,9 @@ SHAPES = [
     (515, 129), (1000, 255), (4099, 256), (333, 257), (1001, 512), (2051, 1000),
     (700, 1024), (300, 1025), (260, 2047), (130, 4097), (70, 8193), (40, 16384),
     (37, 16385), (21, 19456),
+    # several tiles per row group and a partial last tile, for every tile height
+    (40003, 256), (20005, 512), (9001, 1000), (6149, 2047), (3077, 4097), (2053, 8193),
+    (8195, 100), (515, 16384),
 ]
 
 
