@@ -258,9 +258,11 @@ def main():
     for _ in range(a.warmup):
         ctx.loss_grad(theta)
     ctx.reset_timing()
+    ctx.synchronize()
     t0 = time.perf_counter()
     for _ in range(a.steps):
         g, loss, n = ctx.loss_grad(theta)   # synchronous: returns after the stream drained
+    ctx.synchronize()
     elapsed = time.perf_counter() - t0
     _, kern_ms_sum, launches = ctx.timing()
     assert launches == a.steps and n == cfg.n

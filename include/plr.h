@@ -107,6 +107,11 @@ int plr_predict(plr_ctx* ctx, const double* theta, double* h_out);
  * (the linear model's prediction; n doubles out). */
 int plr_predict_linear(plr_ctx* ctx, const double* theta, double* z_out);
 
+/* Block until everything this context (and the device) was asked to do has
+ * finished.  The compute entry points already return drained; this is the
+ * explicit fence benchmarks put on both sides of a timed region. */
+int plr_synchronize(plr_ctx* ctx);
+
 /* Shape of the resident shard (0,0 before plr_set_data). */
 int plr_get_shape(const plr_ctx* ctx, int64_t* n, int64_t* d);
 

@@ -32,6 +32,7 @@ SYMBOLS = [
     ("plr_calc_loss", C.c_int, [_ctx, _dp, _dp, _i64p, C.c_uint]),
     ("plr_predict", C.c_int, [_ctx, _dp, _dp]),
     ("plr_predict_linear", C.c_int, [_ctx, _dp, _dp]),
+    ("plr_synchronize", C.c_int, [_ctx]),
     ("plr_get_shape", C.c_int, [_ctx, _i64p, _i64p]),
     ("plr_get_timing", C.c_int, [_ctx, _dp, _dp, _i64p]),
     ("plr_reset_timing", C.c_int, [_ctx]),
@@ -191,6 +192,9 @@ class Plr:
         z = np.empty(n, dtype=np.float64)
         self._check(self._lib.plr_predict_linear(self._h, _p(theta), _p(z)))
         return z
+
+    def synchronize(self):
+        self._check(self._lib.plr_synchronize(self._h))
 
     # -- timing / info ----------------------------------------------------
     def timing(self):

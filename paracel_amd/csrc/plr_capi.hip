@@ -531,6 +531,14 @@ int plr_probe_read_bandwidth(plr_ctx* c, int reps, double* gb_per_s) {
   return PLR_OK;
 }
 
+int plr_synchronize(plr_ctx* c) {
+  if (!c) return PLR_ERR_INVALID;
+  PLR_HIP(c, hipSetDevice(c->device));
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  PLR_HIP(c, hipDeviceSynchronize());
+  return PLR_OK;
+}
+
 int plr_get_shape(const plr_ctx* c, int64_t* n, int64_t* d) {
   if (!c) return PLR_ERR_INVALID;
   if (n) *n = c->n;
