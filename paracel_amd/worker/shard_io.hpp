@@ -3,10 +3,13 @@
 // is parsed once (std::stod over ~20 GB of text per 8 GB of doubles is the
 // real end-to-end cost of a file-fed run).
 //
-//   load_lines : the reference's "linesplit" rule -- np equal byte ranges,
-//                the last one running to the end; a range owns the lines that
-//                START inside it (include/load/partition.hpp:57-86,121-139,
-//                reached from paralg::paracel_load, include/ps.hpp:178-197).
+//   expand_input: a file, a directory (every file below it) or a glob pattern
+//                (include/utils/ext_utility.hpp:113-160).
+//   load_lines : the reference's "linesplit" rule -- the files are laid end
+//                to end, cut into np equal byte ranges, the last one running
+//                to the end; a range owns the lines that START inside it
+//                (include/load/partition.hpp:57-86,121-175, reached from
+//                paralg::paracel_load, include/ps.hpp:178-197).
 //   parse_lines: logistic_regression::local_parser (lr.cpp:76-93):
 //                "f1,...,fk,label" -> [1.0, f1..fk] and the label; empty
 //                fields are dropped as str_split does
@@ -18,6 +21,7 @@
 //                magic, version, input size and input mtime all match.
 #pragma once
 
+#include <glob.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
@@ -31,29 +35,90 @@
 
 namespace plr_ps {
 
-inline std::vector<std::string> load_lines(const std::string& fn, int rank, int np) {
-  std::ifstream f(fn, std::ios::ate);
-  if (!f) throw std::runtime_error("cannot open " + fn);
-  const long sz = f.tellg();
+inline bool is_regular_file(const std::string& f) {
+  struct stat st;
+  return stat(f.c_str(), &st) == 0 && S_ISREG(st.st_mode);
+}
+inline bool is_directory(const std::string& f) {
+  struct stat st;
+  return stat(f.c_str(), &st) == 0 && S_ISDIR(st.st_mode);
+}
+
+inline std::vector<std::string> glob_paths(const std::string& pattern) {
+  glob_t g;
+  std::vector<std::string> out;
+  if (glob(pattern.c_str(), GLOB_TILDE, nullptr, &g) == 0)
+    for (size_t i = 0; i < g.gl_pathc; ++i) out.push_back(g.gl_pathv[i]);
+  globfree(&g);
+  return out;
+}
+
+inline void expand_dir(const std::string& dir, std::vector<std::string>& out) {
+  const std::string base = (!dir.empty() && dir.back() == '/') ? dir : dir + "/";
+  for (const std::string& name : glob_paths(base + "*")) {
+    if (is_regular_file(name)) out.push_back(name);
+    else if (is_directory(name)) expand_dir(name, out);
+  }
+}
+
+// 'demo.txt' | 'demo_dir' | 'demo_dir/*.csv'
+inline std::vector<std::string> expand_input(const std::string& name) {
+  std::vector<std::string> out;
+  if (is_regular_file(name)) out.push_back(name);
+  else if (is_directory(name)) expand_dir(name, out);
+  else out = glob_paths(name);
+  return out;
+}
+
+inline std::vector<std::string> load_lines(const std::string& input, int rank, int np) {
+  const std::vector<std::string> files = expand_input(input);
+  if (files.empty()) throw std::runtime_error("cannot open " + input);
+  std::vector<long> displs(files.size() + 1, 0);  // byte offset of each file in the union
+  for (size_t i = 0; i < files.size(); ++i) {
+    std::ifstream f(files[i], std::ios::ate);
+    if (!f) throw std::runtime_error("cannot open " + files[i]);
+    displs[i + 1] = displs[i] + (long)f.tellg();
+  }
+  const long sz = displs.back();
   const long bk = sz / np;
   const long st = (long)rank * bk;
   const long en = (rank == np - 1) ? sz : (long)(rank + 1) * bk;
   std::vector<std::string> lines;
-  long offset = st;
-  f.seekg(0);
-  if (offset) {
-    // step back one byte and finish the line in progress: if that byte is the
-    // newline itself, the next line starts exactly at `st` and is ours
-    f.seekg(offset - 1);
-    std::string l;
-    std::getline(f, l);
-    offset += (long)l.size();
+  if (st >= en) return lines;
+  size_t fst = 0, fen = 0;  // first and last file the range touches
+  for (size_t i = 0; i < files.size(); ++i) {
+    if (st >= displs[i]) fst = i;
+    if (en > displs[i + 1]) fen = i + 1;
   }
-  while (offset < en) {
-    std::string l;
-    if (!std::getline(f, l)) break;
-    offset += (long)l.size() + 1;
-    lines.push_back(l);
+  if (fen >= files.size()) fen = files.size() - 1;
+  bool from_file_start = false;
+  for (size_t fi = fst; fi <= fen; ++fi) {
+    long offset = from_file_start ? 0 : st - displs[fi];
+    std::ifstream f(files[fi]);
+    if (offset) {
+      // step back one byte and finish the line in progress: if that byte is
+      // the newline itself, the next line starts exactly at `st` and is ours
+      f.seekg(offset - 1);
+      std::string l;
+      std::getline(f, l);
+      offset += (long)l.size();
+    }
+    if (fi == fen) {
+      while (offset + displs[fi] < en) {
+        std::string l;
+        if (!std::getline(f, l)) break;
+        offset += (long)l.size() + 1;
+        lines.push_back(l);
+      }
+    } else {
+      from_file_start = true;
+      for (;;) {  // to the end of this file (the reference stops at an empty line)
+        std::string l;
+        std::getline(f, l);
+        if (l.empty()) break;
+        lines.push_back(l);
+      }
+    }
   }
   return lines;
 }
@@ -128,9 +193,11 @@ inline std::string cache_path(const std::string& input, int rank, int np) {
   return input + ".plrshard." + std::to_string(rank) + "of" + std::to_string(np);
 }
 
+// The cache covers inputs that are one regular file; directories and globs
+// are parsed every time (their member list can change under the same name).
 inline bool source_stamp(const std::string& input, int64_t& size, int64_t& mtime_ns) {
   struct stat st;
-  if (stat(input.c_str(), &st) != 0) return false;
+  if (stat(input.c_str(), &st) != 0 || !S_ISREG(st.st_mode)) return false;
   size = (int64_t)st.st_size;
   mtime_ns = (int64_t)st.st_mtim.tv_sec * 1000000000LL + st.st_mtim.tv_nsec;
   return true;

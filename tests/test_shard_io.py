@@ -61,6 +61,27 @@ def test_partition_when_a_boundary_hits_a_newline(tmp_path):
     assert sum(owned, []) == lines
 
 
+@pytest.mark.parametrize("np_", [1, 2, 3, 5, 8])
+def test_directory_and_glob_inputs_are_one_byte_stream(tmp_path, np_):
+    # files laid end to end in glob order, then the same byte-range rule
+    # (include/load/partition.hpp:57-86,141-175)
+    d = tmp_path / "parts"
+    d.mkdir()
+    (d / "sub").mkdir()
+    all_lines = []
+    for name, n, seed in (("a.csv", 40, 1), ("b.csv", 7, 2), ("sub/c.csv", 25, 3)):
+        all_lines.append(make_csv(d / name, n, 4, seed))
+    flat = sum(all_lines, [])
+    for spec, want in ((d, flat), (str(d) + "/*.csv", all_lines[0] + all_lines[1])):
+        got = []
+        for r in range(np_):
+            out = run("lines", spec, r, np_)
+            assert out.returncode == 0, out.stderr
+            got.extend(out.stdout.splitlines())
+        assert got == want
+    assert run("lines", str(d) + "/*.nothing", 0, 1).returncode == 1
+
+
 def test_parser_matches_oracle_and_cache_roundtrip(tmp_path, oracle):
     f = tmp_path / "c.csv"
     lines = make_csv(f, 300, 7, 2)
