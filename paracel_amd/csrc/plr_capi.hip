@@ -8,6 +8,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
 #include <string>
 
 #include "plr_kernels.hpp"
@@ -234,13 +235,56 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
   if (row0 < 0 || nrows < 0 || row0 + nrows > c->n)
     return fail(c, PLR_ERR_INVALID, "row range outside the reserved shard");
   PLR_HIP(c, hipSetDevice(c->device));
-  if (ldx == c->pitch && c->d == c->pitch)  // same pitch, no pad column: one linear copy
+  if (ldx == c->pitch && c->d == c->pitch) {  // same pitch, no pad column: one linear copy
     PLR_HIP(c, hipMemcpy(c->dX + row0 * c->pitch, X,
                          (size_t)nrows * c->pitch * sizeof(double), hipMemcpyHostToDevice));
-  else
-    PLR_HIP(c, hipMemcpy2D(c->dX + row0 * c->pitch, (size_t)c->pitch * sizeof(double), X,
-                           (size_t)ldx * sizeof(double), (size_t)c->d * sizeof(double),
-                           (size_t)nrows, hipMemcpyHostToDevice));
+  } else {
+    // Different pitches: a strided copy command moves one row per transfer
+    // (~1 GB/s).  Repack the rows at the device pitch into two pinned staging
+    // buffers on the host and send those as linear copies, the packing of one
+    // overlapping the transfer of the other.
+    const int64_t chunk_rows =
+        std::max<int64_t>(1, std::min<int64_t>(nrows, (int64_t)(32u << 20) / (c->pitch * 8)));
+    const size_t stage_bytes = (size_t)chunk_rows * c->pitch * sizeof(double);
+    double* stage[2] = {nullptr, nullptr};
+    hipEvent_t done[2] = {nullptr, nullptr};
+    int rc = PLR_OK;
+    auto cleanup = [&]() {
+      for (int k = 0; k < 2; ++k) {
+        if (done[k]) (void)hipEventDestroy(done[k]);
+        if (stage[k]) (void)hipHostFree(stage[k]);
+      }
+    };
+    for (int k = 0; k < 2 && rc == PLR_OK; ++k) {
+      if (hipHostMalloc(&stage[k], stage_bytes, hipHostMallocDefault) != hipSuccess ||
+          hipEventCreate(&done[k]) != hipSuccess) {
+        (void)hipGetLastError();
+        rc = fail(c, PLR_ERR_NOMEM, "cannot allocate the pinned upload staging buffers");
+      }
+    }
+    int k = 0;
+    for (int64_t r0 = 0; r0 < nrows && rc == PLR_OK; r0 += chunk_rows, k ^= 1) {
+      const int64_t m = std::min<int64_t>(chunk_rows, nrows - r0);
+      if (r0 >= 2 * chunk_rows && hipEventSynchronize(done[k]) != hipSuccess)
+        rc = fail(c, PLR_ERR_HIP, "upload: waiting for a staging buffer failed");
+      for (int64_t r = 0; r < m && rc == PLR_OK; ++r) {
+        double* dst = stage[k] + r * c->pitch;
+        memcpy(dst, X + (r0 + r) * ldx, (size_t)c->d * sizeof(double));
+        for (int64_t j = c->d; j < c->pitch; ++j) dst[j] = 0.;
+      }
+      if (rc == PLR_OK &&
+          (hipMemcpyAsync(c->dX + (row0 + r0) * c->pitch, stage[k],
+                          (size_t)m * c->pitch * sizeof(double), hipMemcpyHostToDevice,
+                          c->stream) != hipSuccess ||
+           hipEventRecord(done[k], c->stream) != hipSuccess))
+        rc = fail(c, PLR_ERR_HIP, "upload: host-to-device copy failed");
+    }
+    if (hipStreamSynchronize(c->stream) != hipSuccess && rc == PLR_OK)
+      rc = fail(c, PLR_ERR_HIP, "upload: stream synchronisation failed");
+    (void)hipGetLastError();
+    cleanup();
+    if (rc != PLR_OK) return rc;
+  }
   PLR_HIP(c, hipMemcpy(c->dy + row0, y, (size_t)nrows * sizeof(double),
                        hipMemcpyHostToDevice));
   return PLR_OK;
