@@ -31,8 +31,12 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # WRITE_SIZE runs, scaled by what the same counters read for a copy kernel of
 # known size; None until measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
-    # FETCH_SIZE 3932597.4 x 2.000 KiB + WRITE_SIZE 2008.0 x 1.000 KiB per dispatch
-    "c2_headline_1m_x_1000": 8056015667,
+    # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000) KiB per shard_pass dispatch; see profiles/
+    "c2_headline_1m_x_1000": 8055607504,
+    "c3_tall_10m_x_256": 20560472309,
+    "c4_wide_200k_x_16384": 26261494739,
+    "c4b_wide_200k_x_16385": 26466443874,
+    "c5_e2e_2m_x_512": 8210210591,
 }
 
 
