@@ -81,6 +81,19 @@ def upload(ctx, cfg, chunk_rows=131072, keep_rows=0):
     return None, None
 
 
+def reference_build_status():
+    """The reference's own lr_serial needs Boost, Eigen3, msgpack-c and gflags headers
+    (include/ps.hpp); say whether this box has them (it is timed only if it can be built)."""
+    need = {"boost": ["boost/version.hpp"], "eigen3": ["eigen3/Eigen/Dense", "Eigen/Dense"],
+            "msgpack-c": ["msgpack.hpp"], "gflags": ["gflags/gflags.h"]}
+    roots = ["/usr/include", "/usr/local/include", "/opt/conda/include"]
+    missing = [k for k, hs in need.items()
+               if not any(os.path.exists(os.path.join(r, h)) for r in roots for h in hs)]
+    if missing:
+        return "reference lr_serial not buildable on this box: missing " + ", ".join(missing)
+    return "reference dependencies present (reference binary not timed by this script)"
+
+
 def cpu_baseline(cfg, Xs, ys, theta):
     """Reference traversal on the host cores: 1 core (tool/lr_serial, prun.py -w 1)
     and P local workers (mpirun -n P bin/lr), on the row sample, scaled to n."""
@@ -112,6 +125,7 @@ def cpu_baseline(cfg, Xs, ys, theta):
         "loss_pass_seconds_1core_scaled": tl1 * scale,
         "loss_pass_seconds_pcore_scaled": tlp * scale,
         "cpu_model": model,
+        "reference_build": reference_build_status(),
     }
 
 
