@@ -34,7 +34,7 @@ typedef enum {
   PLR_ERR_HIP = -2,         /* a HIP runtime call failed                    */
   PLR_ERR_NOMEM = -3,       /* device or pinned allocation failed           */
   PLR_ERR_NODATA = -4,      /* no shard resident yet                        */
-  PLR_ERR_UNSUPPORTED = -5  /* shape outside what the kernels cover         */
+  PLR_ERR_UNSUPPORTED = -5  /* device is not a gfx950 part                  */
 } plr_status;
 
 /* loss formula selector for plr_loss_grad / plr_calc_loss */

@@ -52,7 +52,21 @@ const Variant kVariants[] = {
     PLR_VARIANT(19, 1, 8, 1, 2, true),    // d <= 19456 (152 KiB of theta in LDS)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
-constexpr int64_t kMaxCols = 19456;
+constexpr int64_t kMaxFusedCols = 19456;
+
+// Rows wider than that are processed in column blocks of 16384, in two sweeps
+// over X (dot products of all blocks, then residuals, then the rank-1
+// updates of all blocks): X is read twice, but any width works.
+constexpr int kBlkNch = 16, kBlkWcol = 8;
+constexpr int64_t kBlockCols = (int64_t)kBlkNch * kBlkWcol * plr::kChunkCols;  // 16384
+// [allch]
+const pass_fn kBlockDot[2] = {
+    plr::shard_pass<kBlkNch, 1, kBlkWcol, 1, 2, false, false, true, plr::kPassDot>,
+    plr::shard_pass<kBlkNch, 1, kBlkWcol, 1, 2, false, true, true, plr::kPassDot>};
+const pass_fn kBlockAxpy[2] = {
+    plr::shard_pass<kBlkNch, 1, kBlkWcol, 1, 2, true, false, true, plr::kPassAxpy>,
+    plr::shard_pass<kBlkNch, 1, kBlkWcol, 1, 2, true, true, true, plr::kPassAxpy>};
+const Variant kBlockVariant = {kBlkNch, 1, kBlkWcol, 1, true, {{nullptr, nullptr}, {nullptr, nullptr}}};
 
 std::string g_create_error;
 
@@ -75,6 +89,9 @@ struct plr_ctx {
   int nch_rt = 0;
   int grid = 0, grid_nograd = 0;
   bool allch = false;
+  bool blocked = false;         // rows wider than the widest fused variant: column blocks
+  double* d_z = nullptr;        // n: blocked rows only, x.theta accumulated over the blocks
+  double* d_res = nullptr;      // n: blocked rows only, residual per row
   int64_t theta_len = 0;
   double* d_theta = nullptr;    // theta_len doubles, zero padded
   double* d_part_g = nullptr;   // grid x pitch
@@ -124,14 +141,17 @@ void free_shape(plr_ctx* c) {
   if (c->d_part_loss) (void)hipFree(c->d_part_loss);
   if (c->d_h) (void)hipFree(c->d_h);
   if (c->d_curve) (void)hipFree(c->d_curve);
+  if (c->d_z) (void)hipFree(c->d_z);
+  if (c->d_res) (void)hipFree(c->d_res);
   if (c->d_train_out) (void)hipFree(c->d_train_out);
   if (c->h_theta) (void)hipHostFree(c->h_theta);
   if (c->h_out) (void)hipHostFree(c->h_out);
-  c->dX = c->dy = c->d_theta = c->d_part_g = c->d_part_loss = c->d_h = c->d_curve =
+  c->dX = c->dy = c->d_theta = c->d_part_g = c->d_part_loss = c->d_h = c->d_curve = c->d_z = c->d_res =
       c->d_train_out = c->h_theta = c->h_theta_dev = c->h_out = c->h_out_dev = nullptr;
   c->n = c->d = c->pitch = 0;
   c->have_data = false;
   c->curve_len = 0;
+  c->blocked = false;
   c->var = nullptr;
   c->info.clear();
 }
@@ -140,10 +160,36 @@ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Pick the kernel variant and persistent grid for an n x d shard.
 int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
-  if (d > kMaxCols)
-    return fail(c, PLR_ERR_UNSUPPORTED,
-                "d = " + std::to_string(d) + " exceeds the widest kernel variant (" +
-                    std::to_string(kMaxCols) + " columns)");
+  if (d > kMaxFusedCols) {
+    const int64_t pitch = (d + 15) & ~int64_t(15);
+    const int threads = plr::kWave * kBlkWcol;
+    c->var = &kBlockVariant;
+    c->blocked = true;
+    c->pitch = pitch;
+    c->nch_rt = kBlkNch;
+    c->allch = false;
+    // theta padded so that the last (narrower) block still reads whole slabs
+    c->theta_len = ceil_div(pitch, kBlockCols) * kBlockCols;
+    int occ = 0, occ2 = 0;
+    PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                   &occ, reinterpret_cast<const void*>(kBlockAxpy[0]), threads, 0));
+    PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                   &occ2, reinterpret_cast<const void*>(kBlockDot[0]), threads, 0));
+    if (occ2 < occ) occ = occ2;
+    if (occ < 1) return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
+    int64_t g = (int64_t)c->num_cu * occ;
+    if (g > n) g = n;
+    if (g < 1) g = 1;
+    c->grid = c->grid_nograd = (int)g;
+    char b[256];
+    snprintf(b, sizeof b,
+             "column-blocked shard_pass<NCH=%d,R=1,WCOL=%d> two sweeps over %lld blocks of %lld "
+             "columns, pitch=%lld grid=%d x %d threads",
+             kBlkNch, kBlkWcol, (long long)ceil_div(pitch, kBlockCols), (long long)kBlockCols,
+             (long long)pitch, c->grid, threads);
+    c->info = b;
+    return PLR_OK;
+  }
   // even pitch so that every row start is 16-byte aligned; wide rows are
   // aligned to 128 B (<= 0.7 % more bytes, +3 % bandwidth when d is odd)
   const int64_t pitch = (d >= 2048) ? ((d + 15) & ~int64_t(15)) : ((d + 1) & ~int64_t(1));
@@ -208,6 +254,10 @@ int alloc_shape(plr_ctx* c, int64_t n, int64_t d) {
   PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)c->theta_len * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_g, (size_t)c->grid * c->pitch * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_loss, (size_t)gmax * sizeof(double)));
+  if (c->blocked && n > 0) {
+    PLR_HIP(c, hipMalloc(&c->d_z, (size_t)n * sizeof(double)));
+    PLR_HIP(c, hipMalloc(&c->d_res, (size_t)n * sizeof(double)));
+  }
   PLR_HIP(c, hipHostMalloc(&c->h_theta, (size_t)c->theta_len * sizeof(double),
                            hipHostMallocMapped | hipHostMallocCoherent));
   PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_theta_dev), c->h_theta, 0));
@@ -319,10 +369,61 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   pa.loss_mode = predict ? (unsigned)plr::kLossNone : loss_mode;
   pa.identity_link = (kind == kPassPredictLinear || loss_mode == plr::kLossSquared) ? 1 : 0;
 
+  pa.width = c->pitch;
+  pa.z_buf = nullptr;
+  pa.z_accumulate = 0;
+  pa.res_in = nullptr;
+
   PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
-  hipLaunchKernelGGL(v->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
-                     c->stream, pa);
-  PLR_HIP(c, hipGetLastError());
+  if (!c->blocked) {
+    hipLaunchKernelGGL(v->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
+                       c->stream, pa);
+    PLR_HIP(c, hipGetLastError());
+  } else if (c->n > 0) {
+    // sweep 1: z = x.theta, one launch per column block, accumulated in d_z
+    pa.z_buf = c->d_z;
+    pa.h_out = nullptr;
+    for (int64_t col0 = 0; col0 < c->pitch; col0 += kBlockCols) {
+      const int64_t w = std::min<int64_t>(kBlockCols, c->pitch - col0);
+      PassArgs pb = pa;
+      pb.X = c->dX + col0;
+      pb.theta = c->d_theta + col0;
+      pb.width = w;
+      pb.nch_rt = (int)ceil_div(ceil_div(w, plr::kChunkCols), kBlkWcol);
+      pb.z_accumulate = col0 > 0 ? 1 : 0;
+      hipLaunchKernelGGL(kBlockDot[w == kBlockCols ? 1 : 0], dim3(grid), dim3(threads), 0,
+                         c->stream, pb);
+      PLR_HIP(c, hipGetLastError());
+    }
+    // residual, prediction and loss per row
+    hipLaunchKernelGGL(plr::residual_pass, dim3(grid), dim3(256), 0, c->stream,
+                       (const double*)c->d_z, (const double*)pa.y, grad ? c->d_res : nullptr,
+                       predict ? c->d_h : nullptr, c->d_part_loss, c->n, pa.loss_mode,
+                       pa.identity_link);
+    PLR_HIP(c, hipGetLastError());
+    // sweep 2: rank-1 updates, block by block
+    if (grad) {
+      pa.res_in = c->d_res;
+      for (int64_t col0 = 0; col0 < c->pitch; col0 += kBlockCols) {
+        const int64_t w = std::min<int64_t>(kBlockCols, c->pitch - col0);
+        PassArgs pb = pa;
+        pb.X = c->dX + col0;
+        pb.theta = c->d_theta + col0;
+        pb.part_g = c->d_part_g + col0;
+        pb.width = w;
+        pb.nch_rt = (int)ceil_div(ceil_div(w, plr::kChunkCols), kBlkWcol);
+        hipLaunchKernelGGL(kBlockAxpy[w == kBlockCols ? 1 : 0], dim3(grid), dim3(threads), 0,
+                           c->stream, pb);
+        PLR_HIP(c, hipGetLastError());
+      }
+    }
+  } else {
+    // empty shard: the finishing kernel needs zeroed partials
+    PLR_HIP(c, hipMemsetAsync(c->d_part_loss, 0, (size_t)grid * sizeof(double), c->stream));
+    if (grad)
+      PLR_HIP(c, hipMemsetAsync(c->d_part_g, 0, (size_t)grid * c->pitch * sizeof(double),
+                                c->stream));
+  }
   PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
 
   if (!predict) {
@@ -335,6 +436,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     fa.d = c->d;
     fa.n = c->n;
     fa.nparts = grid;
+    fa.nparts_loss = grid;
     fa.delta_mode = (kind == kPassDelta) ? (train_round >= 0 ? 2 : 1) : 0;
     fa.have_grad = grad ? 1 : 0;
     fa.alpha = alpha;

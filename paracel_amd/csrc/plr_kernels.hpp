@@ -70,12 +70,49 @@ struct PassArgs {
   double* part_loss;     // [grid]
   double* h_out;         // n, or nullptr (predict)
   int64_t n;
-  int64_t pitch;         // doubles per row in X, even, >= d
+  int64_t pitch;         // doubles per row in X (row stride), even, >= d
+  int64_t width;         // columns this launch covers, starting at X / theta /
+                         // part_g as passed (even; == pitch unless the row is
+                         // processed in column blocks)
   int64_t ntiles;        // ceil(n / R)
   int nch_rt;            // chunks per wave actually used (<= NCH)
   unsigned loss_mode;
   int identity_link;     // 1: h = z (linear model), 0: h = sigmoid(z)
+  // column-blocked rows (kPassDot / kPassAxpy launches)
+  double* z_buf;         // n: x.theta accumulated over the column blocks
+  int z_accumulate;      // 0: this block stores its partial dot, 1: adds to it
+  const double* res_in;  // n: residual per row, computed between the two sweeps
 };
+
+// What one launch of shard_pass does with a tile.
+enum : int {
+  kPassFused = 0,  // dot, sigmoid/residual/loss, rank-1 update: X read once
+  kPassDot = 1,    // only the partial dot of this column block -> z_buf
+  kPassAxpy = 2,   // only the rank-1 update, residual taken from res_in
+};
+
+// h, residual's model output and the loss term of one row from z = x.theta
+// (reference lr.cpp:69-72 and :325-329; ridge.hpp:105-107 for the identity link)
+__device__ __forceinline__ void row_terms(double z, double yv, unsigned loss_mode,
+                                          int identity_link, double& h, double& l) {
+  if (identity_link) {
+    h = z;
+  } else {
+    const double e = exp(-z);
+    h = 1. / (1. + e);
+  }
+  l = 0.;
+  if (loss_mode != kLossNone) {
+    if (loss_mode == kLossReference) {
+      l = -log((yv == 1.) ? h : 1. - h);
+    } else if (loss_mode == kLossSquared) {
+      l = (h - yv) * (h - yv);
+    } else {
+      const double sgn = (yv == 1.) ? -z : z;  // loss = log(1 + exp(sgn))
+      l = log1p(exp(-fabs(sgn))) + fmax(sgn, 0.);
+    }
+  }
+}
 
 // Row held by `lane` after the transposing reduction over R rows.
 template <int R>
@@ -166,7 +203,7 @@ struct WaveCtx {
 
 // Issue every load of one tile of R rows (uniform base + 32-bit lane offset).
 // FULL = every row of the tile exists; ALLCH = the wave uses all NCH chunks.
-template <int NCH, int R, bool FULL, bool ALLCH>
+template <int NCH, int R, bool FULL, bool ALLCH, int MODE>
 __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
                                           const double* tile_base, int64_t row0,
                                           v2d (&x)[R][NCH], double& yv) {
@@ -182,14 +219,18 @@ __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
             rowp + w.lane_off + (uint32_t)(c * kChunkCols * sizeof(double))));
     }
   }
+  // the per-row scalar that goes with the tile: the label, or (second sweep
+  // of a column-blocked row) the residual
   yv = 0.;
-  if ((FULL || row0 + w.my_row < a.n) && a.y) yv = a.y[row0 + w.my_row];
+  const double* per_row = (MODE == kPassAxpy) ? a.res_in : a.y;
+  if (MODE != kPassDot && (FULL || row0 + w.my_row < a.n) && per_row)
+    yv = per_row[row0 + w.my_row];
 }
 
 // Everything that happens on a loaded tile: dots, lane reduction,
 // sigmoid/residual/loss, rank-1 update of the gradient slab.
 // THL: theta is read from the wave's LDS slab (thl) instead of registers.
-template <int NCH, int R, int WCOL, bool GRAD, bool FULL, bool THL>
+template <int NCH, int R, int WCOL, bool GRAD, bool FULL, bool THL, int MODE>
 __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w,
                                              int64_t row0, v2d (&x)[R][NCH], double yv,
                                              const v2d (&th)[NCH], const v2d* thl,
@@ -210,60 +251,56 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
       }
   }
 
-  // ---- per-lane partial dots ----
-  typename RowVec<R>::type p;
-  {
-    double s0[R], s1[R];
+  double res;
+  if constexpr (MODE == kPassAxpy) {
+    res = my_valid ? yv : 0.;  // yv carries the residual in this sweep
+  } else {
+    // ---- per-lane partial dots ----
+    typename RowVec<R>::type p;
+    {
+      double s0[R], s1[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) s0[r] = s1[r] = 0.;
+      for (int r = 0; r < R; ++r) s0[r] = s1[r] = 0.;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const v2d t = THL ? thl[c * kWave] : th[c];
+      for (int c = 0; c < NCH; ++c) {
+        const v2d t = THL ? thl[c * kWave] : th[c];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          s0[r] = fma(x[r][c].x, t.x, s0[r]);
+          s1[r] = fma(x[r][c].y, t.y, s1[r]);
+        }
+      }
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        s0[r] = fma(x[r][c].x, t.x, s0[r]);
-        s1[r] = fma(x[r][c].y, t.y, s1[r]);
+        if constexpr (R == 1)
+          p = s0[r] + s1[r];
+        else
+          p[r] = s0[r] + s1[r];
       }
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      if constexpr (R == 1)
-        p = s0[r] + s1[r];
-      else
-        p[r] = s0[r] + s1[r];
-    }
-  }
-  double z = reduce_rows<R>(p, lane);
+    double z = reduce_rows<R>(p, lane);
 
-  if (WCOL > 1) {
-    if (lane < R) zbuf[w.wc * R + w.my_row] = z;
-    __syncthreads();
-    double s = 0.;
+    if (WCOL > 1) {
+      if (lane < R) zbuf[w.wc * R + w.my_row] = z;
+      __syncthreads();
+      double s = 0.;
 #pragma unroll
-    for (int k = 0; k < WCOL; ++k) s += zbuf[k * R + w.my_row];
-    z = s;
-  }
-
-  // ---- sigmoid, residual, loss for the row this lane holds ----
-  double h;
-  if (a.identity_link) {
-    h = z;
-  } else {
-    const double e = exp(-z);
-    h = 1. / (1. + e);
-  }
-  const double res = my_valid ? (h - yv) : 0.;
-  if (a.h_out && my_valid && lane < R && w.wc == 0) a.h_out[myrow_g] = h;
-  if (a.loss_mode != kLossNone) {
-    double l;
-    if (a.loss_mode == kLossReference) {
-      l = -log((yv == 1.) ? h : 1. - h);
-    } else if (a.loss_mode == kLossSquared) {
-      l = (h - yv) * (h - yv);
-    } else {
-      const double sgn = (yv == 1.) ? -z : z;  // loss = log(1 + exp(sgn))
-      l = log1p(exp(-fabs(sgn))) + fmax(sgn, 0.);
+      for (int k = 0; k < WCOL; ++k) s += zbuf[k * R + w.my_row];
+      z = s;
     }
+
+    if constexpr (MODE == kPassDot) {
+      // first sweep of a column-blocked row: only the partial dot leaves
+      if (my_valid && lane < R && w.wc == 0)
+        a.z_buf[myrow_g] = a.z_accumulate ? a.z_buf[myrow_g] + z : z;
+      return;
+    }
+
+    // ---- sigmoid, residual, loss for the row this lane holds ----
+    double h, l;
+    row_terms(z, yv, a.loss_mode, a.identity_link, h, l);
+    res = my_valid ? (h - yv) : 0.;
+    if (a.h_out && my_valid && lane < R && w.wc == 0) a.h_out[myrow_g] = h;
     if (my_valid && lane < R && w.wc == 0) loss_acc += l;
   }
 
@@ -291,7 +328,9 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
 //        so no wave has an unused chunk slot and no load is predicated
 // THL  : theta lives in LDS (one slab per wave) instead of registers -- for
 //        wide rows, where theta + accumulators + tile would not fit
-template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD, bool ALLCH, bool THL>
+// MODE : kPassFused, or one of the two sweeps of a column-blocked row
+template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD, bool ALLCH, bool THL,
+          int MODE = kPassFused>
 __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a) {
   static_assert(WCOL == 1 || WROW == 1, "column-split workgroups own one row group");
   static_assert((R & (R - 1)) == 0 && R <= kWave, "R must be a power of two");
@@ -300,14 +339,14 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   const int wc = (WCOL > 1) ? wave : 0;
   const int wr = (WCOL > 1) ? 0 : wave;
 
-  const int64_t chunks = (a.pitch + kChunkCols - 1) / kChunkCols;
+  const int64_t chunks = (a.width + kChunkCols - 1) / kChunkCols;
   const int64_t slab_c0 = (int64_t)wc * a.nch_rt;          // first chunk of this wave
   int64_t left = chunks - slab_c0;
   const int my_nch = ALLCH ? NCH : (int)(left < 0 ? 0 : (left > a.nch_rt ? a.nch_rt : left));
   const int64_t slab_col0 = slab_c0 * kChunkCols;
   const int64_t col0 = slab_col0 + 2 * lane;
   // the chunk that straddles the end of the row, if this wave owns it
-  const int tail_cols = (int)(a.pitch % kChunkCols);
+  const int tail_cols = (int)(a.width % kChunkCols);
   const int ragged_c = (tail_cols != 0 && slab_c0 + my_nch == chunks && my_nch > 0)
                            ? my_nch - 1 : -1;
   const bool lane_in_ragged = 2 * lane < tail_cols;
@@ -353,15 +392,15 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   for (; tile < nfull; tile += ngroups, par ^= 1) {
     v2d x[R][NCH];
     double yv;
-    load_tile<NCH, R, true, ALLCH>(a, w, xbase + tile * tile_stride, tile * R, x, yv);
-    compute_tile<NCH, R, WCOL, GRAD, true, THL>(a, w, tile * R, x, yv, thr, thl, acc,
+    load_tile<NCH, R, true, ALLCH, MODE>(a, w, xbase + tile * tile_stride, tile * R, x, yv);
+    compute_tile<NCH, R, WCOL, GRAD, true, THL, MODE>(a, w, tile * R, x, yv, thr, thl, acc,
                                                 loss_acc, zx + par * kZ);
   }
   if (tile < a.ntiles) {
     v2d x[R][NCH];
     double yv;
-    load_tile<NCH, R, false, ALLCH>(a, w, xbase + tile * tile_stride, tile * R, x, yv);
-    compute_tile<NCH, R, WCOL, GRAD, false, THL>(a, w, tile * R, x, yv, thr, thl, acc,
+    load_tile<NCH, R, false, ALLCH, MODE>(a, w, xbase + tile * tile_stride, tile * R, x, yv);
+    compute_tile<NCH, R, WCOL, GRAD, false, THL, MODE>(a, w, tile * R, x, yv, thr, thl, acc,
                                                  loss_acc, zx + par * kZ);
   }
 
@@ -396,7 +435,7 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
       }
     }
   }
-  {
+  if constexpr (MODE == kPassFused) {  // the sweeps of a blocked row carry no loss
     __shared__ double lx[WCOL * WROW];
     const double wl = wave_sum(loss_acc);
     if (lane == 0) lx[wave] = wl;
@@ -431,6 +470,33 @@ __global__ __launch_bounds__(256) void read_probe(const v2d* base, int64_t ntile
   if (acc.x + acc.y == 1.2345e300) sink[0] = acc.x;  // keeps the loads alive
 }
 
+// Between the two sweeps of a column-blocked row: z (complete dot products)
+// -> h, residual and loss per row.  One thread per row, grid-stride; each
+// thread adds its rows' loss terms in row order, the workgroup folds them in
+// a fixed order into part_loss[block].
+__global__ __launch_bounds__(256) void residual_pass(const double* __restrict__ z,
+                                                     const double* __restrict__ y,
+                                                     double* __restrict__ res,
+                                                     double* __restrict__ h_out,
+                                                     double* __restrict__ part_loss, int64_t n,
+                                                     unsigned loss_mode, int identity_link) {
+  __shared__ double lx[4];
+  double loss_acc = 0.;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const double yv = y ? y[i] : 0.;
+    double h, l;
+    row_terms(z[i], yv, loss_mode, identity_link, h, l);
+    if (res) res[i] = h - yv;
+    if (h_out) h_out[i] = h;
+    loss_acc += l;
+  }
+  const double wl = wave_sum(loss_acc);
+  if ((threadIdx.x & (kWave - 1)) == 0) lx[threadIdx.x / kWave] = wl;
+  __syncthreads();
+  if (threadIdx.x == 0) part_loss[blockIdx.x] = ((lx[0] + lx[1]) + lx[2]) + lx[3];
+}
+
 // theta arrives in pinned, device-mapped host memory; this one-workgroup
 // kernel moves it into the zero-padded device copy the pass reads.  A kernel
 // on the pass's own stream instead of a copy command: no hand-over between
@@ -450,7 +516,8 @@ struct FinishArgs {
   int64_t pitch;
   int64_t d;
   int64_t n;
-  int nparts;
+  int nparts;             // rows of part_g
+  int nparts_loss;        // entries of part_loss
   int delta_mode;         // 0: out = gsum; 1: out = -alpha*gsum - coff2*n*theta;
                           // 2: as 1, and theta_rw += delta (the server-side add,
                           //    done in place on the device copy of theta)
@@ -494,7 +561,7 @@ __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a
   }
   if (blockIdx.x == 0) {
     double s = 0.;
-    for (int p = threadIdx.x; p < a.nparts; p += kFinCols * kFinSlices)
+    for (int p = threadIdx.x; p < a.nparts_loss; p += kFinCols * kFinSlices)
       s += a.part_loss[p];
     sm[sl][cx] = s;
     __syncthreads();

@@ -149,6 +149,9 @@ def configs():
                                        1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
         "c4b_wide_200k_x_16385": Config("c4b_wide_200k_x_16385", 200_000, 16385, 0x5EED0004, NORMAL,
                                         1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
+        # wider than the widest fused kernel: the column-blocked two-sweep path
+        "x_verywide_100k_x_32768": Config("x_verywide_100k_x_32768", 100_000, 32768, 0x5EED0006,
+                                          NORMAL, 1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
         # end-to-end through the host parameter server
         "c5_e2e_2m_x_512": Config("c5_e2e_2m_x_512", 2_000_000, 512, 0x5EED0005, NORMAL,
                                   1.0 / np.sqrt(512), lam=0.01, theta0_zero=True),

@@ -110,6 +110,30 @@ def test_linear_model_pieces(plr, oracle, gen, n, d):
     assert abs(loss2 - want) <= 1e-12 * want
 
 
+@pytest.mark.parametrize("n,d", [(19, 19457), (300, 33000), (1030, 20001), (64, 65536)])
+def test_rows_wider_than_the_fused_kernels(plr, oracle, gen, n, d):
+    # past 19456 columns the row is processed in column blocks, two sweeps over X
+    print("case n=%d d=%d" % (n, d), flush=True)
+    X, y, th = make(gen, n, d)
+    plr.set_data(X, y)
+    print(plr.kernel_info(), flush=True)
+    g, loss, n_out = plr.loss_grad(th)
+    assert n_out == n
+    assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
+    want = oracle.calc_loss_sum(X, y, th)
+    assert abs(loss - want) <= LOSS_TOL * want
+    g2, loss2, _ = plr.loss_grad(th)
+    np.testing.assert_array_equal(g, g2)
+    assert loss == loss2
+    delta, _ = plr.dgd_delta(th, 0.1 / n, 0.005)
+    assert rel(delta, oracle.dgd_delta(X, y, th, 0.1 / n, 0.005)) <= GRAD_TOL
+    l3, _ = plr.calc_loss(th, 1)
+    assert abs(l3 - want) <= LOSS_TOL * want
+    assert np.max(np.abs(plr.predict(th) - oracle.predict(X, th))) <= 1e-14
+    t5 = plr.train_dgd(np.zeros(d), 0.1 / n, 0.005, 5)
+    assert rel(t5, oracle.train_dgd(X, y, np.zeros(d), 0.1 / n, 0.005, 5)) <= 1e-10
+
+
 def test_theta_zero_closed_forms(plr, gen):
     # theta = 0 => h = 1/2 exactly: gsum = X^T (1/2 - y) (a plain GEMV), loss = n ln 2
     X, y, _ = make(gen, 3001, 300)
@@ -264,9 +288,6 @@ def test_errors(plr):
     with pytest.raises(PlrError) as e:
         plr.loss_grad(np.zeros(0))
     assert e.value.code == -4  # PLR_ERR_NODATA
-    with pytest.raises(PlrError) as e:
-        plr.alloc_data(10, 19457)
-    assert e.value.code == -5  # PLR_ERR_UNSUPPORTED
     with pytest.raises(PlrError) as e:
         plr.alloc_data(10, 0)
     assert e.value.code == -1
