@@ -66,6 +66,26 @@ const pass_fn kBlockDot[2] = {
 const pass_fn kBlockAxpy[2] = {
     plr::shard_pass<kBlkNch, 1, kBlkWcol, 1, 2, true, false, true, plr::kPassAxpy>,
     plr::shard_pass<kBlkNch, 1, kBlkWcol, 1, 2, true, true, true, plr::kPassAxpy>};
+// Narrow rows (d <= 64): power-of-two pitch, several whole rows per chunk.
+struct PackedVariant {
+  int logp, U, wrow;
+  pass_fn fn[2];  // [grad]
+};
+#define PLR_PACKED(LOGP, U, WROW, MINW)                       \
+  {LOGP, U, WROW,                                             \
+   {plr::packed_pass<LOGP, U, WROW, MINW, false>, plr::packed_pass<LOGP, U, WROW, MINW, true>}}
+// indexed by log2(pitch) - 1; tile shapes from sweeps (6.3-7.0 TB/s for pitch
+// 8..64; pitch 2 and 4 are bound by one exp/log per 16-32 bytes)
+const PackedVariant kPacked[] = {
+    PLR_PACKED(1, 4, 4, 4),  // pitch 2
+    PLR_PACKED(2, 4, 4, 3),  // pitch 4
+    PLR_PACKED(3, 2, 4, 3),  // pitch 8
+    PLR_PACKED(4, 2, 4, 2),  // pitch 16
+    PLR_PACKED(5, 2, 2, 1),  // pitch 32
+    PLR_PACKED(6, 1, 2, 1),  // pitch 64
+};
+constexpr int64_t kMaxPackedCols = 64;
+
 const Variant kBlockVariant = {kBlkNch, 1, kBlkWcol, 1, true, {{nullptr, nullptr}, {nullptr, nullptr}}};
 
 std::string g_create_error;
@@ -89,6 +109,7 @@ struct plr_ctx {
   int nch_rt = 0;
   int grid = 0, grid_nograd = 0;
   bool allch = false;
+  const PackedVariant* packed = nullptr;  // d <= 64: packed-row kernel
   bool blocked = false;         // rows wider than the widest fused variant: column blocks
   double* d_z = nullptr;        // n: blocked rows only, x.theta accumulated over the blocks
   double* d_res = nullptr;      // n: blocked rows only, residual per row
@@ -152,6 +173,7 @@ void free_shape(plr_ctx* c) {
   c->have_data = false;
   c->curve_len = 0;
   c->blocked = false;
+  c->packed = nullptr;
   c->var = nullptr;
   c->info.clear();
 }
@@ -160,6 +182,37 @@ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Pick the kernel variant and persistent grid for an n x d shard.
 int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
+  if (d <= kMaxPackedCols) {
+    int logp = 1;
+    while ((int64_t(1) << logp) < d) ++logp;
+    const PackedVariant* pv = &kPacked[logp - 1];
+    const int threads = plr::kWave * pv->wrow;
+    c->packed = pv;
+    c->var = &kBlockVariant;  // unused by the packed path, kept non-null
+    c->pitch = int64_t(1) << logp;
+    c->nch_rt = 1;
+    c->allch = false;
+    c->theta_len = plr::kChunkCols;
+    int occ = 0, occ2 = 0;
+    PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                   &occ, reinterpret_cast<const void*>(pv->fn[1]), threads, 0));
+    PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                   &occ2, reinterpret_cast<const void*>(pv->fn[0]), threads, 0));
+    if (occ < 1 || occ2 < 1)
+      return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
+    const int64_t ntiles = ceil_div(n, (int64_t)plr::kWave * pv->U);
+    const int64_t want = std::max<int64_t>(1, ceil_div(ntiles, pv->wrow));
+    c->grid = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ);
+    c->grid_nograd = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ2);
+    char b[256];
+    snprintf(b, sizeof b,
+             "packed_pass<pitch=%lld,U=%d,WROW=%d> %d rows per tile, grid=%d x %d threads "
+             "(occupancy %d blocks/CU, %d CUs)",
+             (long long)c->pitch, pv->U, pv->wrow, plr::kWave * pv->U, c->grid, threads, occ,
+             c->num_cu);
+    c->info = b;
+    return PLR_OK;
+  }
   if (d > kMaxFusedCols) {
     const int64_t pitch = (d + 15) & ~int64_t(15);
     const int threads = plr::kWave * kBlkWcol;
@@ -245,7 +298,7 @@ int alloc_shape(plr_ctx* c, int64_t n, int64_t d) {
   // lanes of the chunk that straddles the end of the last row read (and then
   // discard) up to one slab past it: keep that much slack mapped
   const size_t xbytes = (size_t)n * c->pitch * sizeof(double) +
-                        (size_t)c->theta_len * sizeof(double);
+                        std::max<size_t>((size_t)c->theta_len * sizeof(double), 64u << 10);
   if (n > 0) {
     PLR_HIP(c, hipMalloc(&c->dX, xbytes));
     PLR_HIP(c, hipMalloc(&c->dy, (size_t)n * sizeof(double)));
@@ -353,7 +406,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
   const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
   const int grid = grad ? c->grid : c->grid_nograd;
-  const int threads = plr::kWave * v->wcol * v->wrow;
+  const int threads = c->packed ? plr::kWave * c->packed->wrow : plr::kWave * v->wcol * v->wrow;
 
   PassArgs pa;
   pa.X = c->dX;
@@ -375,7 +428,10 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   pa.res_in = nullptr;
 
   PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
-  if (!c->blocked) {
+  if (c->packed) {
+    hipLaunchKernelGGL(c->packed->fn[grad ? 1 : 0], dim3(grid), dim3(threads), 0, c->stream, pa);
+    PLR_HIP(c, hipGetLastError());
+  } else if (!c->blocked) {
     hipLaunchKernelGGL(v->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
                        c->stream, pa);
     PLR_HIP(c, hipGetLastError());

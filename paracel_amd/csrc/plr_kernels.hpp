@@ -449,6 +449,157 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   }
 }
 
+// ---------------------------------------------------------------------------
+// Narrow rows (d <= 64).  With a row shorter than a 128-column chunk most lanes
+// of shard_pass would idle, so the shard is stored with a power-of-two pitch
+// P = 2..64 and a chunk (128 consecutive doubles, one dwordx4 per lane) holds
+// 128/P WHOLE rows: lane l owns the column pair 2*(l % SL) of row l / SL of
+// every chunk, SL = P/2 lanes per row.  A group of SL chunks carries 64 rows;
+// the transposing butterfly over the SL lanes of a row leaves every lane with
+// ONE distinct row of the group, so the 64 lanes evaluate 64 different
+// sigmoids / loss terms at once.  The residuals travel back inside the row's
+// lane segment (ds_bpermute), the rank-1 update runs on the registers the
+// rows were loaded into, and the per-lane accumulators (one column pair
+// each) are folded over the segments once, at the end.  U groups per tile
+// keep 16-32 KiB of loads in flight per wave.
+//
+// Same reference loops as shard_pass (lr.cpp:69-72,132-138,322-330,361-363).
+template <int LOGP, int U, int WROW, int MINW, bool GRAD>
+__global__ __launch_bounds__(kWave* WROW, MINW) void packed_pass(PassArgs a) {
+  constexpr int P = 1 << LOGP;       // pitch in doubles
+  constexpr int SL = P / 2;          // lanes per row
+  constexpr int RPC = kWave / SL;    // rows per chunk
+  constexpr int kTileRows = kWave * U;
+  static_assert(LOGP >= 1 && LOGP <= 6, "packed rows are 2..64 doubles wide");
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wr = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int pos = lane & (SL - 1);   // which column pair of the row
+  const int seg = lane / SL;         // which row of a chunk
+  const int my_chunk = row_of_lane<SL>(pos);  // chunk of the group whose row ends up here
+
+  const v2d th = *reinterpret_cast<const v2d*>(a.theta + 2 * pos);
+  v2d acc = v2d{0., 0.};
+  double loss_acc = 0.;
+
+  const int64_t group0 = (int64_t)blockIdx.x * WROW + wr;
+  const int64_t ngroups = (int64_t)gridDim.x * WROW;
+  const int64_t nfull = a.n / kTileRows;
+  const int64_t ntiles = (a.n + kTileRows - 1) / kTileRows;
+
+  auto tile_body = [&](int64_t tile, auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
+    const int64_t row0 = tile * kTileRows;
+    const v2d* base = reinterpret_cast<const v2d*>(a.X + row0 * P) + lane;
+    v2d x[U][SL];
+#pragma unroll
+    for (int g = 0; g < U; ++g)
+#pragma unroll
+      for (int c = 0; c < SL; ++c) {
+        const int k = g * SL + c;
+        x[g][c] = load_x(base + (int64_t)k * kWave);
+        if (!FULL && row0 + (int64_t)k * RPC + seg >= a.n) x[g][c] = v2d{0., 0.};
+      }
+    double yv[U];
+    int64_t myrow[U];
+#pragma unroll
+    for (int g = 0; g < U; ++g) {
+      myrow[g] = row0 + ((int64_t)g * SL + my_chunk) * RPC + seg;
+      yv[g] = 0.;
+      if ((FULL || myrow[g] < a.n) && a.y) yv[g] = a.y[myrow[g]];
+    }
+#pragma unroll
+    for (int g = 0; g < U; ++g) {
+      typename RowVec<SL>::type p;
+#pragma unroll
+      for (int c = 0; c < SL; ++c) {
+        const double t = fma(x[g][c].x, th.x, x[g][c].y * th.y);
+        if constexpr (SL == 1)
+          p = t;
+        else
+          p[c] = t;
+      }
+      // reduce over the SL lanes of a row; lane (seg, pos) keeps chunk my_chunk
+      double z;
+      if constexpr (SL == 1) {
+        z = p;
+      } else {
+#pragma unroll
+        for (int s = 0; s < ilog2(SL); ++s) {
+          const int cnt = SL >> (s + 1);
+          const int m = 1 << s;
+          const bool up = (lane & m) != 0;
+#pragma unroll
+          for (int k = 0; k < cnt; ++k) {
+            const double lo = p[k], hi = p[k + cnt];
+            const double send = up ? lo : hi;
+            const double keep = up ? hi : lo;
+            p[k] = keep + __shfl_xor(send, m, kWave);
+          }
+        }
+        z = p[0];
+      }
+      const bool valid = FULL || myrow[g] < a.n;
+      double h, l;
+      row_terms(z, yv[g], a.loss_mode, a.identity_link, h, l);
+      const double res = valid ? (h - yv[g]) : 0.;
+      if (a.h_out && valid) a.h_out[myrow[g]] = h;
+      if (valid) loss_acc += l;
+      if (GRAD) {
+#pragma unroll
+        for (int c = 0; c < SL; ++c) {
+          // the residual of this lane's row in chunk c sits in the lane of
+          // the same segment that kept chunk c
+          const double rr =
+              (SL == 1) ? res : __shfl(res, (lane & ~(SL - 1)) | lane_of_row<SL>(c), kWave);
+          acc.x = fma(rr, x[g][c].x, acc.x);
+          acc.y = fma(rr, x[g][c].y, acc.y);
+        }
+      }
+    }
+  };
+
+  int64_t tile = group0;
+#pragma clang loop unroll(disable)
+  for (; tile < nfull; tile += ngroups) tile_body(tile, std::true_type{});
+  if (tile < ntiles) tile_body(tile, std::false_type{});
+
+  if (GRAD) {
+    // fold the row segments: lanes 0..SL-1 end up with the wave's totals
+#pragma unroll
+    for (int m = SL; m < kWave; m <<= 1) {
+      acc.x += __shfl_xor(acc.x, m, kWave);
+      acc.y += __shfl_xor(acc.y, m, kWave);
+    }
+    __shared__ v2d gx[(WROW > 1) ? (WROW - 1) * SL : 1];
+    if (WROW > 1) {
+      if (wr > 0 && lane < SL) gx[(wr - 1) * SL + lane] = acc;
+      __syncthreads();
+    }
+    if (wr == 0 && lane < SL) {
+      v2d s = acc;
+#pragma unroll
+      for (int w = 1; w < WROW; ++w) {
+        const v2d o = gx[(w - 1) * SL + lane];
+        s.x += o.x;
+        s.y += o.y;
+      }
+      *reinterpret_cast<v2d*>(a.part_g + (int64_t)blockIdx.x * P + 2 * lane) = s;
+    }
+  }
+  {
+    __shared__ double lx[WROW];
+    const double wl = wave_sum(loss_acc);
+    if (lane == 0) lx[wr] = wl;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      double s = 0.;
+#pragma unroll
+      for (int w = 0; w < WROW; ++w) s += lx[w];
+      a.part_loss[blockIdx.x] = s;
+    }
+  }
+}
+
 // Pure streaming read of a buffer with shard_pass's access pattern (a wave
 // takes contiguous 8 KiB tiles, interleaved over the grid) and next to no
 // arithmetic: what it sustains is the read ceiling the fused pass is up

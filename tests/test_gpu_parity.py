@@ -134,6 +134,38 @@ def test_rows_wider_than_the_fused_kernels(plr, oracle, gen, n, d):
     assert rel(t5, oracle.train_dgd(X, y, np.zeros(d), 0.1 / n, 0.005, 5)) <= 1e-10
 
 
+NARROW = [(n, d) for d in (1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 48, 63, 64)
+          for n in (1, 65, 100003)] + [(63, 7), (64, 7), (127, 32), (128, 32), (255, 64), (256, 2),
+                                       (257, 2), (511, 4), (513, 8), (1000000, 6)]
+
+
+@pytest.mark.parametrize("n,d", NARROW)
+def test_narrow_rows_packed_kernel(plr, oracle, gen, n, d):
+    # d <= 64: power-of-two device pitch, several whole rows per 128-double chunk
+    print("case n=%d d=%d" % (n, d), flush=True)
+    X, y, th = make(gen, n, d, scale=1.0 / np.sqrt(d), theta_scale=1.0)
+    plr.set_data(X, y)
+    g, loss, n_out = plr.loss_grad(th)
+    assert n_out == n
+    assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
+    want = oracle.calc_loss_sum(X, y, th)
+    assert abs(loss - want) <= LOSS_TOL * want
+    g2, loss2, _ = plr.loss_grad(th)
+    np.testing.assert_array_equal(g, g2)
+    assert loss2 == loss
+    if n <= 1000:
+        delta, _ = plr.dgd_delta(th, 0.1 / n, 0.005)
+        assert rel(delta, oracle.dgd_delta(X, y, th, 0.1 / n, 0.005)) <= GRAD_TOL
+        np.testing.assert_allclose(plr.predict(th), oracle.predict(X, th), rtol=0, atol=1e-14)
+        ls, _ = plr.calc_loss(th, 1)
+        assert abs(ls - want) <= LOSS_TOL * want
+        lq, _ = plr.calc_loss(th, 3)
+        wq = oracle.ridge_loss_sum(X, y, th)
+        assert abs(lq - wq) <= 1e-12 * wq
+        np.testing.assert_allclose(plr.predict_linear(th), oracle.predict_linear(X, th), rtol=0,
+                                   atol=1e-13)
+
+
 def test_theta_zero_closed_forms(plr, gen):
     # theta = 0 => h = 1/2 exactly: gsum = X^T (1/2 - y) (a plain GEMV), loss = n ln 2
     X, y, _ = make(gen, 3001, 300)
