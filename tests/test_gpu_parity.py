@@ -376,3 +376,38 @@ def test_device_resident_training_matches_oracle_and_per_round_path(plr, oracle,
     t0 = gen.gen_vec(5, gen.STREAM_THETA, cfg.d)
     np.testing.assert_array_equal(plr.train_dgd(t0, alpha, beta, 0), t0)
     np.testing.assert_array_equal(plr.train_dgd(np.zeros(cfg.d), alpha, beta, 100), theta)
+
+
+def _random_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        # widths spread over every kernel family, biased towards chunk / variant boundaries
+        kind = rng.integers(0, 4)
+        if kind == 0:
+            d = int(rng.integers(1, 130))
+        elif kind == 1:
+            d = int(rng.choice([128, 256, 512, 1024, 2048, 4096, 8192]) + rng.integers(-3, 4))
+        elif kind == 2:
+            d = int(rng.integers(130, 9000))
+        else:
+            d = int(rng.integers(9000, 24000))
+        n = int(rng.integers(1, max(2, min(3000, 3_000_000 // d))))
+        out.append((n, d))
+    return out
+
+
+def test_random_shape_sweep(plr, oracle, gen):
+    # 60 seeded shapes across all kernel families, gradient + loss against the oracle
+    worst = 0.0
+    for n, d in _random_shapes(60, 20240607):
+        print("case n=%d d=%d" % (n, d), flush=True)
+        X, y, th = make(gen, n, d, seed=n * 131 + d)
+        plr.set_data(X, y)
+        g, loss, n_out = plr.loss_grad(th)
+        e = rel(g, oracle.gsum(X, y, th))
+        worst = max(worst, e)
+        assert n_out == n and e <= GRAD_TOL, (n, d, e, plr.kernel_info())
+        want = oracle.calc_loss_sum(X, y, th)
+        assert abs(loss - want) <= LOSS_TOL * want, (n, d, plr.kernel_info())
+    print("worst gradient rel-L2 over the sweep: %.3e" % worst)
