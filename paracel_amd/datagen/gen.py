@@ -149,6 +149,9 @@ def configs():
                                        1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
         "c4b_wide_200k_x_16385": Config("c4b_wide_200k_x_16385", 200_000, 16385, 0x5EED0004, NORMAL,
                                         1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
+        # narrow rows: the packed-row kernel (several whole rows per 128-double chunk)
+        "x_narrow_30m_x_16": Config("x_narrow_30m_x_16", 30_000_000, 16, 0x5EED0007, NORMAL, 0.25,
+                                    lam=0.01),
         # wider than the widest fused kernel: the column-blocked two-sweep path
         "x_verywide_100k_x_32768": Config("x_verywide_100k_x_32768", 100_000, 32768, 0x5EED0006,
                                           NORMAL, 1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
