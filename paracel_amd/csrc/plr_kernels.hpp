@@ -679,12 +679,13 @@ struct FinishArgs {
   double coff2;
 };
 
-constexpr int kFinCols = 64;
-constexpr int kFinSlices = 16;
+constexpr int kFinCols = 16;
+constexpr int kFinSlices = 64;
 
 // Sums the per-workgroup partials: thread (col, slice) adds parts slice,
-// slice+16, ... in order; the 16 slice sums meet in LDS and are added in
-// slice order.  Block 0 also folds the loss partials the same way.
+// slice+64, ... in order (a short chain: the kernel is bound by load latency,
+// not bandwidth); the 64 slice sums meet in LDS and are added in slice order.
+// Block 0 also folds the loss partials the same way.
 __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a) {
   __shared__ double sm[kFinSlices][kFinCols];
   const int cx = threadIdx.x % kFinCols;
@@ -692,9 +693,11 @@ __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a
   const int64_t col = (int64_t)blockIdx.x * kFinCols + cx;
   if (a.have_grad) {
     double s = 0.;
-    if (col < a.d)
+    if (col < a.d) {
+#pragma unroll 4
       for (int p = sl; p < a.nparts; p += kFinSlices)
         s += a.part_g[(int64_t)p * a.pitch + col];
+    }
     sm[sl][cx] = s;
     __syncthreads();
     if (sl == 0 && col < a.d) {
@@ -716,10 +719,11 @@ __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a
       s += a.part_loss[p];
     sm[sl][cx] = s;
     __syncthreads();
-    if (threadIdx.x < kFinCols) {
-      double t = sm[0][cx];
+    if (threadIdx.x < kWave) {  // the whole first wave: wave_sum needs all 64 lanes
+      const double* flat = &sm[0][0];
+      double t = flat[threadIdx.x];
 #pragma unroll
-      for (int k = 1; k < kFinSlices; ++k) t += sm[k][cx];
+      for (int k = 1; k < kFinCols * kFinSlices / kWave; ++k) t += flat[threadIdx.x + k * kWave];
       t = wave_sum(t);
       if (threadIdx.x == 0) {
         a.out[a.d] = t;
