@@ -58,12 +58,13 @@ def parse_args():
     return ap.parse_args()
 
 
-def upload(ctx, cfg, chunk_rows=131072, keep_rows=0):
+def upload(ctx, cfg, chunk_bytes=1 << 30, keep_rows=0):
     """Generate the shard on the host in row chunks and stream it to HBM.
     Returns the first keep_rows rows (for the CPU baseline sample)."""
     import numpy as np
 
     ctx.alloc_data(cfg.n, cfg.d)
+    chunk_rows = max(1, chunk_bytes // (8 * cfg.d))
     keepX, keepy = [], []
     kept = 0
     buf = np.empty((min(chunk_rows, cfg.n), cfg.d))  # reused: first touch of fresh pages is slow

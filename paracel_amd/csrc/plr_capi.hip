@@ -118,6 +118,9 @@ struct plr_ctx {
   double* d_part_g = nullptr;   // grid x pitch
   double* d_part_loss = nullptr;  // max(grid, grid_nograd)
   double* d_h = nullptr;        // n (predict), lazily allocated
+  double* up_stage[2] = {nullptr, nullptr};  // pinned repack buffers for pitched uploads
+  hipEvent_t up_done[2] = {nullptr, nullptr};
+  size_t up_stage_bytes = 0;
   double* d_curve = nullptr;    // per-round losses of plr_train_dgd, lazily allocated
   double* d_train_out = nullptr;  // d + 1: where training rounds put delta (never read back)
   int curve_len = 0;
@@ -153,8 +156,19 @@ int fail(plr_ctx* c, int code, const std::string& msg) {
     }                                                                        \
   } while (0)
 
+void release_upload_staging(plr_ctx* c) {
+  for (int k = 0; k < 2; ++k) {
+    if (c->up_done[k]) (void)hipEventDestroy(c->up_done[k]);
+    if (c->up_stage[k]) (void)hipHostFree(c->up_stage[k]);
+    c->up_done[k] = nullptr;
+    c->up_stage[k] = nullptr;
+  }
+  c->up_stage_bytes = 0;
+}
+
 void free_shape(plr_ctx* c) {
   (void)hipSetDevice(c->device);
+  release_upload_staging(c);
   if (c->dX) (void)hipFree(c->dX);
   if (c->dy) (void)hipFree(c->dy);
   if (c->d_theta) (void)hipFree(c->d_theta);
@@ -346,25 +360,26 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
     // (~1 GB/s).  Repack the rows at the device pitch into two pinned staging
     // buffers on the host and send those as linear copies, the packing of one
     // overlapping the transfer of the other.
-    const int64_t chunk_rows =
-        std::max<int64_t>(1, std::min<int64_t>(nrows, (int64_t)(32u << 20) / (c->pitch * 8)));
+    const int64_t chunk_rows = std::max<int64_t>(1, (int64_t)(32u << 20) / (c->pitch * 8));
     const size_t stage_bytes = (size_t)chunk_rows * c->pitch * sizeof(double);
-    double* stage[2] = {nullptr, nullptr};
-    hipEvent_t done[2] = {nullptr, nullptr};
     int rc = PLR_OK;
-    auto cleanup = [&]() {
-      for (int k = 0; k < 2; ++k) {
-        if (done[k]) (void)hipEventDestroy(done[k]);
-        if (stage[k]) (void)hipHostFree(stage[k]);
+    if (c->up_stage_bytes < stage_bytes) {  // kept for the shard's lifetime: chunked uploads reuse them
+      release_upload_staging(c);
+      for (int k = 0; k < 2 && rc == PLR_OK; ++k) {
+        if (hipHostMalloc(&c->up_stage[k], stage_bytes, hipHostMallocDefault) != hipSuccess ||
+            hipEventCreate(&c->up_done[k]) != hipSuccess) {
+          (void)hipGetLastError();
+          rc = fail(c, PLR_ERR_NOMEM, "cannot allocate the pinned upload staging buffers");
+        }
       }
-    };
-    for (int k = 0; k < 2 && rc == PLR_OK; ++k) {
-      if (hipHostMalloc(&stage[k], stage_bytes, hipHostMallocDefault) != hipSuccess ||
-          hipEventCreate(&done[k]) != hipSuccess) {
-        (void)hipGetLastError();
-        rc = fail(c, PLR_ERR_NOMEM, "cannot allocate the pinned upload staging buffers");
+      if (rc != PLR_OK) {
+        release_upload_staging(c);
+        return rc;
       }
+      c->up_stage_bytes = stage_bytes;
     }
+    double** stage = c->up_stage;
+    hipEvent_t* done = c->up_done;
     int k = 0;
     for (int64_t r0 = 0; r0 < nrows && rc == PLR_OK; r0 += chunk_rows, k ^= 1) {
       const int64_t m = std::min<int64_t>(chunk_rows, nrows - r0);
@@ -385,7 +400,6 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
     if (hipStreamSynchronize(c->stream) != hipSuccess && rc == PLR_OK)
       rc = fail(c, PLR_ERR_HIP, "upload: stream synchronisation failed");
     (void)hipGetLastError();
-    cleanup();
     if (rc != PLR_OK) return rc;
   }
   PLR_HIP(c, hipMemcpy(c->dy + row0, y, (size_t)nrows * sizeof(double),
