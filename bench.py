@@ -102,8 +102,8 @@ def cpu_baseline(cfg, Xs, ys, theta):
 
     m = Xs.shape[0]
     cores = max(1, min(16, os.cpu_count() or 1))
-    t1, _, tl1, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=1, reps=2)
-    tp, _, tlp, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=cores, reps=5)
+    t1, _, tl1, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=1, reps=4)
+    tp, _, tlp, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=cores, reps=20)
     scale = cfg.n / float(m)
     model = ""
     try:

@@ -34,22 +34,51 @@ struct Variant {
     {plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, false, THL>,          \
      plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, true, THL>}}}
 
-// Ordered by the number of 128-column chunks they cover (wcol * nch).  Tile
-// shapes and register budgets (MINW = waves per SIMD the allocation leaves
-// room for) come from sweeps on MI355X: one or two resident waves per SIMD,
-// each with 16-32 KiB of loads in flight, stream fastest; any variant that
-// spills registers loses a third of the bandwidth or more.
+// One variant per (waves side by side, chunks per wave) pair that a row width
+// can map to exactly: a row of C chunks uses one wave with C chunks up to
+// C = 8, then ceil(C/8) chunks per wave on as many waves as that takes
+// (<= 8), so at most one wave of the workgroup is partly idle.  Tile heights
+// and register budgets (MINW = waves per SIMD the allocation leaves room for)
+// come from sweeps on MI355X: one or two resident waves per SIMD, each with
+// 16-48 KiB of loads in flight, stream fastest; any variant that spills
+// registers loses a third of the bandwidth or more.  From 65 chunks on theta
+// lives in LDS and a variant covers every per-wave count up to its NCH.
 const Variant kVariants[] = {
-    PLR_VARIANT(1, 16, 1, 4, 2, false),   // d <= 128
-    PLR_VARIANT(2, 32, 1, 4, 1, false),   // d <= 256
-    PLR_VARIANT(4, 16, 1, 2, 1, false),   // d <= 512
-    PLR_VARIANT(8, 4, 1, 4, 1, false),    // d <= 1024
-    PLR_VARIANT(2, 8, 8, 1, 2, false),    // d <= 2048
-    PLR_VARIANT(4, 4, 8, 1, 2, false),    // d <= 4096
-    PLR_VARIANT(8, 4, 8, 1, 2, true),     // d <= 8192
-    PLR_VARIANT(16, 1, 8, 1, 2, true),    // d <= 16384
-    PLR_VARIANT(17, 1, 8, 1, 2, true),    // d <= 17408
-    PLR_VARIANT(19, 1, 8, 1, 2, true),    // d <= 19456 (152 KiB of theta in LDS)
+    // one wave per row
+    PLR_VARIANT(1, 16, 1, 4, 2, false),
+    PLR_VARIANT(2, 32, 1, 4, 1, false),
+    PLR_VARIANT(3, 16, 1, 2, 1, false),
+    PLR_VARIANT(4, 16, 1, 2, 1, false),
+    PLR_VARIANT(5, 8, 1, 2, 1, false),
+    PLR_VARIANT(6, 8, 1, 2, 1, false),
+    PLR_VARIANT(7, 4, 1, 4, 1, false),
+    PLR_VARIANT(8, 4, 1, 4, 1, false),
+    // 2 chunks per wave: 9..16 chunks
+    PLR_VARIANT(2, 16, 5, 1, 2, false),
+    PLR_VARIANT(2, 16, 6, 1, 2, false),
+    PLR_VARIANT(2, 16, 7, 1, 2, false),
+    PLR_VARIANT(2, 8, 8, 1, 2, false),
+    // 3 chunks per wave: 17..24
+    PLR_VARIANT(3, 8, 6, 1, 2, false),
+    PLR_VARIANT(3, 8, 7, 1, 2, false),
+    PLR_VARIANT(3, 8, 8, 1, 2, false),
+    // 4..7 chunks per wave: 25..56
+    PLR_VARIANT(4, 4, 7, 1, 2, false),
+    PLR_VARIANT(4, 4, 8, 1, 2, false),
+    PLR_VARIANT(5, 4, 7, 1, 2, false),
+    PLR_VARIANT(5, 4, 8, 1, 2, false),
+    PLR_VARIANT(6, 4, 7, 1, 2, false),
+    PLR_VARIANT(6, 4, 8, 1, 2, false),
+    PLR_VARIANT(7, 4, 7, 1, 2, false),
+    PLR_VARIANT(7, 4, 8, 1, 2, false),
+    // 8 chunks per wave and up: theta in LDS
+    PLR_VARIANT(8, 4, 8, 1, 2, true),     // 57..64
+    PLR_VARIANT(10, 2, 8, 1, 2, true),    // ..80
+    PLR_VARIANT(12, 2, 8, 1, 2, true),    // ..96
+    PLR_VARIANT(14, 1, 8, 1, 2, true),    // ..112
+    PLR_VARIANT(16, 1, 8, 1, 2, true),    // ..128
+    PLR_VARIANT(17, 1, 8, 1, 2, true),    // ..136
+    PLR_VARIANT(19, 1, 8, 1, 2, true),    // ..152 (152 KiB of theta in LDS)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int64_t kMaxFusedCols = 19456;
@@ -261,16 +290,32 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   // aligned to 128 B (<= 0.7 % more bytes, +3 % bandwidth when d is odd)
   const int64_t pitch = (d >= 2048) ? ((d + 15) & ~int64_t(15)) : ((d + 1) & ~int64_t(1));
   const int64_t chunks = ceil_div(pitch, plr::kChunkCols);
+  // (waves, chunks per wave) for this width, then the variant that has them
+  int want_w, want_k;
+  if (chunks <= 8) {
+    want_w = 1;
+    want_k = (int)chunks;
+  } else if (chunks <= 64) {
+    want_k = (int)ceil_div(chunks, 8);
+    want_w = (int)ceil_div(chunks, want_k);
+  } else {
+    want_w = 8;
+    want_k = (int)ceil_div(chunks, 8);
+  }
   const Variant* v = nullptr;
-  for (int i = 0; i < kNumVariants; ++i)
-    if ((int64_t)kVariants[i].nch * kVariants[i].wcol >= chunks) {
-      v = &kVariants[i];
+  for (int i = 0; i < kNumVariants; ++i) {
+    const Variant& k = kVariants[i];
+    const bool fits = (want_k >= 8 && want_w == 8) ? (k.thl && k.wcol == 8 && k.nch >= want_k)
+                                                   : (!k.thl && k.wcol == want_w && k.nch == want_k);
+    if (fits) {
+      v = &k;
       break;
     }
+  }
   if (!v) return fail(c, PLR_ERR_UNSUPPORTED, "no kernel variant covers this width");
   c->var = v;
   c->pitch = pitch;
-  c->nch_rt = (int)ceil_div(chunks, v->wcol);
+  c->nch_rt = (int)ceil_div(chunks, v->wcol);  // == v->nch except for the theta-in-LDS variants
   c->allch = (chunks == (int64_t)v->nch * v->wcol);
   c->theta_len = (int64_t)v->wcol * c->nch_rt * plr::kChunkCols;
   const int threads = plr::kWave * v->wcol * v->wrow;
