@@ -23,41 +23,79 @@ typedef void (*pass_fn)(PassArgs);
 struct Variant {
   int nch, R, wcol, wrow;
   bool thl;
-  // [grad][allch]
+  int tl;  // tail loads per tile (0: the row ends inside or at the end of a chunk)
+  // [grad][allch]; one-wave rows always match their variant exactly, so they
+  // carry only the allch instances
   pass_fn fn[2][2];
 };
 
+// several waves side by side over the columns
 #define PLR_VARIANT(NCH, R, WCOL, WROW, MINW, THL)                         \
-  {NCH, R, WCOL, WROW, THL,                                                \
+  {NCH, R, WCOL, WROW, THL, 0,                                             \
    {{plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, false, THL>,         \
      plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, true, THL>},         \
     {plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, false, THL>,          \
      plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, true, THL>}}}
+// one wave per row: NCH full chunks (the last may be ragged when TL == 0),
+// plus, with TL > 0, up to 128*TL/R leftover columns
+#define PLR_ROW(NCH, R, WROW, MINW, TL)                                                      \
+  {NCH, R, 1, WROW, false, TL,                                                               \
+   {{nullptr, plr::shard_pass<NCH, R, 1, WROW, MINW, false, true, false, plr::kPassFused, TL>}, \
+    {nullptr, plr::shard_pass<NCH, R, 1, WROW, MINW, true, true, false, plr::kPassFused, TL>}}}
 
-// One variant per (waves side by side, chunks per wave) pair that a row width
-// can map to exactly: a row of C chunks uses one wave with C chunks up to
-// C = 8, then ceil(C/8) chunks per wave on as many waves as that takes
-// (<= 8), so at most one wave of the workgroup is partly idle.  Tile heights
-// and register budgets (MINW = waves per SIMD the allocation leaves room for)
-// come from sweeps on MI355X: one or two resident waves per SIMD, each with
-// 16-48 KiB of loads in flight, stream fastest; any variant that spills
-// registers loses a third of the bandwidth or more.  From 65 chunks on theta
-// lives in LDS and a variant covers every per-wave count up to its NCH.
+// A row of C chunks (128 columns each) is handled by one wave up to C = 16,
+// then by ceil(C/8) chunks per wave on as many waves side by side as that
+// takes (<= 8), so at most one wave of the workgroup is partly idle.  A row
+// that ends up to 32-64 columns past a chunk boundary takes the variant with
+// that many full chunks and a tail stage.  Tile heights and register budgets
+// (MINW = waves per SIMD the allocation leaves room for) come from sweeps on
+// MI355X: one or two resident waves per SIMD, each with 16-48 KiB of loads in
+// flight, stream fastest; any variant that spills registers loses a third of
+// the bandwidth or more.  From 65 chunks on theta lives in LDS and a variant
+// covers every per-wave count up to its NCH.
 const Variant kVariants[] = {
-    // one wave per row
-    PLR_VARIANT(1, 16, 1, 4, 2, false),
-    PLR_VARIANT(2, 32, 1, 4, 1, false),
-    PLR_VARIANT(3, 16, 1, 2, 1, false),
-    PLR_VARIANT(4, 16, 1, 2, 1, false),
-    PLR_VARIANT(5, 8, 1, 2, 1, false),
-    PLR_VARIANT(6, 8, 1, 2, 1, false),
-    PLR_VARIANT(7, 4, 1, 4, 1, false),
-    PLR_VARIANT(8, 4, 1, 4, 1, false),
-    // 2 chunks per wave: 9..16 chunks
-    PLR_VARIANT(2, 16, 5, 1, 2, false),
-    PLR_VARIANT(2, 16, 6, 1, 2, false),
-    PLR_VARIANT(2, 16, 7, 1, 2, false),
-    PLR_VARIANT(2, 8, 8, 1, 2, false),
+    // one wave per row, exact chunk counts
+    PLR_ROW(1, 16, 4, 2, 0),
+    PLR_ROW(2, 32, 4, 1, 0),
+    PLR_ROW(3, 16, 2, 1, 0),
+    PLR_ROW(4, 16, 2, 1, 0),
+    PLR_ROW(5, 8, 2, 1, 0),
+    PLR_ROW(6, 8, 2, 1, 0),
+    PLR_ROW(7, 4, 4, 1, 0),
+    PLR_ROW(8, 4, 4, 1, 0),
+    PLR_ROW(9, 4, 4, 1, 0),
+    PLR_ROW(10, 4, 4, 1, 0),
+    PLR_ROW(11, 4, 4, 1, 0),
+    PLR_ROW(12, 2, 4, 1, 0),
+    PLR_ROW(13, 4, 4, 1, 0),
+    PLR_ROW(14, 4, 4, 1, 0),
+    PLR_ROW(15, 2, 4, 1, 0),
+    PLR_ROW(16, 2, 4, 1, 0),
+    // one wave per row with a tail stage (capacity 128*TL/R columns)
+    PLR_ROW(1, 32, 4, 1, 2),   // 8
+    PLR_ROW(1, 32, 4, 1, 4),   // 16
+    PLR_ROW(1, 16, 4, 2, 4),   // 32
+    PLR_ROW(1, 8, 4, 2, 4),    // 64
+    PLR_ROW(2, 16, 4, 1, 1),   // 8
+    PLR_ROW(2, 16, 4, 1, 2),   // 16
+    PLR_ROW(2, 16, 4, 1, 4),   // 32
+    PLR_ROW(2, 8, 4, 2, 4),    // 64
+    PLR_ROW(3, 8, 4, 1, 1),    // 16
+    PLR_ROW(3, 8, 4, 1, 2),    // 32
+    PLR_ROW(4, 8, 4, 1, 1),    // 16
+    PLR_ROW(4, 8, 4, 1, 2),    // 32
+    PLR_ROW(6, 4, 4, 1, 1),    // 32
+    PLR_ROW(7, 4, 4, 1, 1),    // 32
+    PLR_ROW(8, 4, 4, 1, 1),    // 32
+    PLR_ROW(8, 4, 4, 1, 2),    // 64
+    PLR_ROW(9, 4, 4, 1, 1),    // 32
+    PLR_ROW(10, 4, 4, 1, 1),   // 32
+    PLR_ROW(11, 4, 4, 1, 1),   // 32
+    PLR_ROW(12, 2, 4, 1, 1),   // 64
+    PLR_ROW(13, 2, 4, 1, 1),   // 64
+    PLR_ROW(14, 2, 4, 1, 1),   // 64
+    PLR_ROW(15, 2, 4, 1, 1),   // 64
+    PLR_ROW(16, 2, 4, 1, 1),   // 64
     // 3 chunks per wave: 17..24
     PLR_VARIANT(3, 8, 6, 1, 2, false),
     PLR_VARIANT(3, 8, 7, 1, 2, false),
@@ -80,6 +118,7 @@ const Variant kVariants[] = {
     PLR_VARIANT(17, 1, 8, 1, 2, true),    // ..136
     PLR_VARIANT(19, 1, 8, 1, 2, true),    // ..152 (152 KiB of theta in LDS)
 };
+constexpr int kMaxRowChunks = 16;  // widest one-wave row
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int64_t kMaxFusedCols = 19456;
 
@@ -115,7 +154,7 @@ const PackedVariant kPacked[] = {
 };
 constexpr int64_t kMaxPackedCols = 64;
 
-const Variant kBlockVariant = {kBlkNch, 1, kBlkWcol, 1, true, {{nullptr, nullptr}, {nullptr, nullptr}}};
+const Variant kBlockVariant = {kBlkNch, 1, kBlkWcol, 1, true, 0, {{nullptr, nullptr}, {nullptr, nullptr}}};
 
 std::string g_create_error;
 
@@ -138,6 +177,7 @@ struct plr_ctx {
   int nch_rt = 0;
   int grid = 0, grid_nograd = 0;
   bool allch = false;
+  int tail_cols = 0;            // columns handled by the variant's tail stage
   const PackedVariant* packed = nullptr;  // d <= 64: packed-row kernel
   bool blocked = false;         // rows wider than the widest fused variant: column blocks
   double* d_z = nullptr;        // n: blocked rows only, x.theta accumulated over the blocks
@@ -217,6 +257,7 @@ void free_shape(plr_ctx* c) {
   c->curve_len = 0;
   c->blocked = false;
   c->packed = nullptr;
+  c->tail_cols = 0;
   c->var = nullptr;
   c->info.clear();
 }
@@ -290,34 +331,64 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   // aligned to 128 B (<= 0.7 % more bytes, +3 % bandwidth when d is odd)
   const int64_t pitch = (d >= 2048) ? ((d + 15) & ~int64_t(15)) : ((d + 1) & ~int64_t(1));
   const int64_t chunks = ceil_div(pitch, plr::kChunkCols);
-  // (waves, chunks per wave) for this width, then the variant that has them
-  int want_w, want_k;
-  if (chunks <= 8) {
-    want_w = 1;
-    want_k = (int)chunks;
-  } else if (chunks <= 64) {
-    want_k = (int)ceil_div(chunks, 8);
-    want_w = (int)ceil_div(chunks, want_k);
-  } else {
-    want_w = 8;
-    want_k = (int)ceil_div(chunks, 8);
-  }
   const Variant* v = nullptr;
-  for (int i = 0; i < kNumVariants; ++i) {
-    const Variant& k = kVariants[i];
-    const bool fits = (want_k >= 8 && want_w == 8) ? (k.thl && k.wcol == 8 && k.nch >= want_k)
-                                                   : (!k.thl && k.wcol == want_w && k.nch == want_k);
-    if (fits) {
-      v = &k;
-      break;
+  int tail = 0;
+  // a few columns past a chunk boundary: the tail-stage variant with the
+  // smallest capacity that holds them
+  const int64_t full = pitch / plr::kChunkCols, rem = pitch % plr::kChunkCols;
+  if (rem != 0 && full >= 1 && full <= kMaxRowChunks) {
+    int best_cap = 1 << 30;
+    for (int i = 0; i < kNumVariants; ++i) {
+      const Variant& k = kVariants[i];
+      if (k.tl == 0 || k.nch != full) continue;
+      const int cap = plr::kChunkCols * k.tl / k.R;
+      if (cap >= rem && cap < best_cap) {
+        v = &k;
+        best_cap = cap;
+      }
+    }
+    if (v) tail = (int)rem;
+  }
+  if (!v) {
+    // (waves, chunks per wave) for this width, then the variant that has them
+    int want_w, want_k;
+    if (chunks <= kMaxRowChunks) {
+      want_w = 1;
+      want_k = (int)chunks;
+    } else if (chunks <= 64) {
+      want_k = (int)ceil_div(chunks, 8);
+      want_w = (int)ceil_div(chunks, want_k);
+    } else {
+      want_w = 8;
+      want_k = (int)ceil_div(chunks, 8);
+    }
+    for (int i = 0; i < kNumVariants; ++i) {
+      const Variant& k = kVariants[i];
+      if (k.tl != 0) continue;
+      const bool fits = (want_k >= 8 && want_w == 8)
+                            ? (k.thl && k.wcol == 8 && k.nch >= want_k)
+                            : (!k.thl && k.wcol == want_w && k.nch == want_k);
+      if (fits) {
+        v = &k;
+        break;
+      }
     }
   }
   if (!v) return fail(c, PLR_ERR_UNSUPPORTED, "no kernel variant covers this width");
   c->var = v;
   c->pitch = pitch;
-  c->nch_rt = (int)ceil_div(chunks, v->wcol);  // == v->nch except for the theta-in-LDS variants
-  c->allch = (chunks == (int64_t)v->nch * v->wcol);
-  c->theta_len = (int64_t)v->wcol * c->nch_rt * plr::kChunkCols;
+  c->tail_cols = tail;
+  if (tail) {
+    c->nch_rt = v->nch;
+    c->allch = true;
+    c->theta_len = (int64_t)(v->nch + 1) * plr::kChunkCols;
+  } else {
+    c->nch_rt = (int)ceil_div(chunks, v->wcol);  // == v->nch except for the theta-in-LDS variants
+    c->allch = (chunks == (int64_t)v->nch * v->wcol);
+    c->theta_len = (int64_t)v->wcol * c->nch_rt * plr::kChunkCols;
+  }
+  if (!v->fn[1][c->allch] || !v->fn[0][c->allch])
+    return fail(c, PLR_ERR_UNSUPPORTED, "kernel variant lacks the instance this width needs");
   const int threads = plr::kWave * v->wcol * v->wrow;
   const int64_t ntiles = ceil_div(n, v->R);
   const int64_t want = ceil_div(ntiles, v->wrow);
@@ -337,10 +408,10 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   c->grid_nograd = (int)g2;
   char b[256];
   snprintf(b, sizeof b,
-           "shard_pass<NCH=%d,R=%d,WCOL=%d,WROW=%d,ALLCH=%d> nch_rt=%d pitch=%lld grid=%d x %d "
-           "threads (occupancy %d blocks/CU, %d CUs)",
-           v->nch, v->R, v->wcol, v->wrow, (int)c->allch, c->nch_rt, (long long)pitch, c->grid,
-           threads, occ, c->num_cu);
+           "shard_pass<NCH=%d,R=%d,WCOL=%d,WROW=%d,ALLCH=%d,TL=%d> nch_rt=%d tail=%d pitch=%lld "
+           "grid=%d x %d threads (occupancy %d blocks/CU, %d CUs)",
+           v->nch, v->R, v->wcol, v->wrow, (int)c->allch, v->tl, c->nch_rt, tail,
+           (long long)pitch, c->grid, threads, occ, c->num_cu);
   c->info = b;
   return PLR_OK;
 }
@@ -478,6 +549,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   pa.pitch = c->pitch;
   pa.ntiles = ceil_div(c->n, v->R);
   pa.nch_rt = c->nch_rt;
+  pa.tail_cols = c->tail_cols;
   pa.loss_mode = predict ? (unsigned)plr::kLossNone : loss_mode;
   pa.identity_link = (kind == kPassPredictLinear || loss_mode == plr::kLossSquared) ? 1 : 0;
 

@@ -17,9 +17,15 @@
 //     row's partial, log2(64/R) plain butterfly steps finish it.  So the
 //     exp/log of a row is evaluated once per tile by the lane that holds
 //     it, not 64 times, and R-1+log2(64/R) lane exchanges replace 6R.
-//   * d > 1024: WCOL waves of a workgroup split the columns; their partial
+//   * Rows of more than 16 chunks: WCOL waves of a workgroup split the columns; their partial
 //     dots meet in LDS (double-buffered, one barrier per tile) and are summed
 //     in wave order.
+//   * A row that ends a few columns past a chunk boundary (the file path
+//     always adds a bias column, so 256 features arrive as 257 columns) does
+//     not get a nearly empty chunk of its own: the TL > 0 variants cover the
+//     leftover columns of ALL rows of a tile with TL loads, 64*TL/R lanes per
+//     row, reduce them inside those lane segments and fold them into the
+//     row's dot product and the gradient separately.
 //   * Rows are spread over the grid tile-interleaved (tile t goes to row
 //     group t mod G), so at any moment the grid streams one contiguous window
 //     of X.
@@ -76,6 +82,8 @@ struct PassArgs {
                          // processed in column blocks)
   int64_t ntiles;        // ceil(n / R)
   int nch_rt;            // chunks per wave actually used (<= NCH)
+  int tail_cols;         // TL > 0 variants: columns past the last full chunk
+                         // (even, <= 128*TL/R); width = chunks*128 + tail_cols
   unsigned loss_mode;
   int identity_link;     // 1: h = z (linear model), 0: h = sigmoid(z)
   // column-blocked rows (kPassDot / kPassAxpy launches)
@@ -199,14 +207,29 @@ struct WaveCtx {
   bool lane_in_ragged;
   int my_row;         // row of the tile whose dot product ends up in this lane
   uint32_t lane_off;  // byte offset of this lane inside a chunk
+  // tail stage (TL > 0): this lane's place among the leftover columns
+  bool tail_in;       // the lane's column pair exists
+  int tail_row;       // row, within one tail load, that the lane reads
+  int tail_slot;      // lane holding the tail dot of row my_row
+  uint32_t tail_off;  // byte offset of the lane's pair from the tile base
+  int tail_src[4];    // per tail load: lane holding the residual of its row
+};
+
+// Geometry of the tail stage: a tile's R rows are covered by TL loads of
+// R/TL rows each, kWave*TL/R adjacent lanes per row.
+template <int R, int TL>
+struct TailGeo {
+  static constexpr int kRowsPerLoad = R / (TL > 0 ? TL : 1);
+  static constexpr int kLanesPerRow = kWave / kRowsPerLoad;
 };
 
 // Issue every load of one tile of R rows (uniform base + 32-bit lane offset).
 // FULL = every row of the tile exists; ALLCH = the wave uses all NCH chunks.
-template <int NCH, int R, bool FULL, bool ALLCH, int MODE>
+template <int NCH, int R, bool FULL, bool ALLCH, int MODE, int TL>
 __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
                                           const double* tile_base, int64_t row0,
-                                          v2d (&x)[R][NCH], double& yv) {
+                                          v2d (&x)[R][NCH], v2d (&xt)[TL > 0 ? TL : 1],
+                                          double& yv) {
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const char* rowp = reinterpret_cast<const char*>(tile_base + (int64_t)r * a.pitch);
@@ -217,6 +240,17 @@ __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
       if (rv && (ALLCH || c < w.my_nch))  // uniform
         x[r][c] = load_x(reinterpret_cast<const v2d*>(
             rowp + w.lane_off + (uint32_t)(c * kChunkCols * sizeof(double))));
+    }
+  }
+  if constexpr (TL > 0) {
+    constexpr int kRpl = TailGeo<R, TL>::kRowsPerLoad;
+#pragma unroll
+    for (int j = 0; j < TL; ++j) {
+      xt[j] = v2d{0., 0.};
+      if (w.tail_in && (FULL || row0 + j * kRpl + w.tail_row < a.n))
+        xt[j] = load_x(reinterpret_cast<const v2d*>(
+            reinterpret_cast<const char*>(tile_base + (int64_t)(j * kRpl) * a.pitch) +
+            w.tail_off));
     }
   }
   // the per-row scalar that goes with the tile: the label, or (second sweep
@@ -230,11 +264,12 @@ __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
 // Everything that happens on a loaded tile: dots, lane reduction,
 // sigmoid/residual/loss, rank-1 update of the gradient slab.
 // THL: theta is read from the wave's LDS slab (thl) instead of registers.
-template <int NCH, int R, int WCOL, bool GRAD, bool FULL, bool THL, int MODE>
+template <int NCH, int R, int WCOL, bool GRAD, bool FULL, bool THL, int MODE, int TL>
 __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w,
-                                             int64_t row0, v2d (&x)[R][NCH], double yv,
-                                             const v2d (&th)[NCH], const v2d* thl,
-                                             v2d (&acc)[NCH], double& loss_acc,
+                                             int64_t row0, v2d (&x)[R][NCH],
+                                             const v2d (&xt)[TL > 0 ? TL : 1], double yv,
+                                             const v2d (&th)[NCH], const v2d* thl, v2d tht,
+                                             v2d (&acc)[NCH], v2d& acct, double& loss_acc,
                                              double* zbuf) {
   const int lane = w.lane;
   const int64_t myrow_g = row0 + w.my_row;
@@ -280,6 +315,23 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
     }
     double z = reduce_rows<R>(p, lane);
 
+    if constexpr (TL > 0) {
+      // leftover columns: segment sums, then each row's sum to the lane that
+      // holds the row
+      constexpr int kRpl = TailGeo<R, TL>::kRowsPerLoad;
+      constexpr int kLpr = TailGeo<R, TL>::kLanesPerRow;
+      double tz = 0.;
+#pragma unroll
+      for (int j = 0; j < TL; ++j) {
+        double t = fma(xt[j].x, tht.x, xt[j].y * tht.y);
+#pragma unroll
+        for (int m = 1; m < kLpr; m <<= 1) t += __shfl_xor(t, m, kWave);
+        const double got = __shfl(t, w.tail_slot, kWave);
+        if (TL == 1 || w.my_row / kRpl == j) tz = got;
+      }
+      z += tz;
+    }
+
     if (WCOL > 1) {
       if (lane < R) zbuf[w.wc * R + w.my_row] = z;
       __syncthreads();
@@ -315,6 +367,14 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
         acc[c].y = fma(rr, x[r][c].y, acc[c].y);
       }
     }
+    if constexpr (TL > 0) {
+#pragma unroll
+      for (int j = 0; j < TL; ++j) {
+        const double rr = __shfl(res, w.tail_src[j], kWave);
+        acct.x = fma(rr, xt[j].x, acct.x);
+        acct.y = fma(rr, xt[j].y, acct.y);
+      }
+    }
   }
 }
 
@@ -329,27 +389,33 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
 // THL  : theta lives in LDS (one slab per wave) instead of registers -- for
 //        wide rows, where theta + accumulators + tile would not fit
 // MODE : kPassFused, or one of the two sweeps of a column-blocked row
+// TL   : 0, or the number of loads per tile that cover the columns past the
+//        NCH full chunks (a.tail_cols of them, at most 128*TL/R)
 template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD, bool ALLCH, bool THL,
-          int MODE = kPassFused>
+          int MODE = kPassFused, int TL = 0>
 __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a) {
   static_assert(WCOL == 1 || WROW == 1, "column-split workgroups own one row group");
   static_assert((R & (R - 1)) == 0 && R <= kWave, "R must be a power of two");
+  static_assert(TL == 0 || (WCOL == 1 && ALLCH && !THL && MODE == kPassFused && TL <= R &&
+                            TL <= 4 && (TL & (TL - 1)) == 0),
+                "the tail stage goes with one-wave rows of exactly NCH full chunks");
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform
   const int wc = (WCOL > 1) ? wave : 0;
   const int wr = (WCOL > 1) ? 0 : wave;
 
-  const int64_t chunks = (a.width + kChunkCols - 1) / kChunkCols;
+  // with a tail stage the chunks are the NCH full ones
+  const int64_t chunks = (TL > 0) ? NCH : (a.width + kChunkCols - 1) / kChunkCols;
   const int64_t slab_c0 = (int64_t)wc * a.nch_rt;          // first chunk of this wave
   int64_t left = chunks - slab_c0;
   const int my_nch = ALLCH ? NCH : (int)(left < 0 ? 0 : (left > a.nch_rt ? a.nch_rt : left));
   const int64_t slab_col0 = slab_c0 * kChunkCols;
   const int64_t col0 = slab_col0 + 2 * lane;
   // the chunk that straddles the end of the row, if this wave owns it
-  const int tail_cols = (int)(a.width % kChunkCols);
-  const int ragged_c = (tail_cols != 0 && slab_c0 + my_nch == chunks && my_nch > 0)
+  const int rag_cols = (TL > 0) ? 0 : (int)(a.width % kChunkCols);
+  const int ragged_c = (rag_cols != 0 && slab_c0 + my_nch == chunks && my_nch > 0)
                            ? my_nch - 1 : -1;
-  const bool lane_in_ragged = 2 * lane < tail_cols;
+  const bool lane_in_ragged = 2 * lane < rag_cols;
   WaveCtx w;
   w.lane = lane;
   w.wc = wc;
@@ -358,6 +424,21 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   w.lane_in_ragged = lane_in_ragged;
   w.my_row = row_of_lane<R>(lane & (R - 1));
   w.lane_off = (uint32_t)(2 * lane * sizeof(double));
+  constexpr int kRpl = TailGeo<R, TL>::kRowsPerLoad;
+  constexpr int kLpr = TailGeo<R, TL>::kLanesPerRow;
+  constexpr int64_t kBodyCols = (int64_t)NCH * kChunkCols;
+  const int tail_pair = lane & (kLpr - 1);
+  v2d tht = v2d{0., 0.}, acct = v2d{0., 0.};
+  if constexpr (TL > 0) {
+    w.tail_in = 2 * tail_pair < a.tail_cols;
+    w.tail_row = lane / kLpr;
+    w.tail_slot = (w.my_row % kRpl) * kLpr;
+    w.tail_off = (uint32_t)(((int64_t)w.tail_row * a.pitch + kBodyCols + 2 * tail_pair) *
+                            sizeof(double));
+#pragma unroll
+    for (int j = 0; j < TL; ++j) w.tail_src[j] = lane_of_row<R>(j * kRpl + w.tail_row);
+    if (w.tail_in) tht = *reinterpret_cast<const v2d*>(a.theta + kBodyCols + 2 * tail_pair);
+  }
 
   // theta slab -> registers, or -> this wave's private LDS slab (theta is
   // zero-padded on the device)
@@ -390,49 +471,60 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   int par = 0;  // which half of zx the next tile uses (alternates per tile)
 #pragma clang loop unroll(disable)
   for (; tile < nfull; tile += ngroups, par ^= 1) {
-    v2d x[R][NCH];
+    v2d x[R][NCH], xt[TL > 0 ? TL : 1];
     double yv;
-    load_tile<NCH, R, true, ALLCH, MODE>(a, w, xbase + tile * tile_stride, tile * R, x, yv);
-    compute_tile<NCH, R, WCOL, GRAD, true, THL, MODE>(a, w, tile * R, x, yv, thr, thl, acc,
-                                                loss_acc, zx + par * kZ);
+    load_tile<NCH, R, true, ALLCH, MODE, TL>(a, w, xbase + tile * tile_stride, tile * R, x, xt,
+                                             yv);
+    compute_tile<NCH, R, WCOL, GRAD, true, THL, MODE, TL>(a, w, tile * R, x, xt, yv, thr, thl,
+                                                          tht, acc, acct, loss_acc,
+                                                          zx + par * kZ);
   }
   if (tile < a.ntiles) {
-    v2d x[R][NCH];
+    v2d x[R][NCH], xt[TL > 0 ? TL : 1];
     double yv;
-    load_tile<NCH, R, false, ALLCH, MODE>(a, w, xbase + tile * tile_stride, tile * R, x, yv);
-    compute_tile<NCH, R, WCOL, GRAD, false, THL, MODE>(a, w, tile * R, x, yv, thr, thl, acc,
-                                                 loss_acc, zx + par * kZ);
+    load_tile<NCH, R, false, ALLCH, MODE, TL>(a, w, xbase + tile * tile_stride, tile * R, x, xt,
+                                              yv);
+    compute_tile<NCH, R, WCOL, GRAD, false, THL, MODE, TL>(a, w, tile * R, x, xt, yv, thr, thl,
+                                                           tht, acc, acct, loss_acc,
+                                                           zx + par * kZ);
   }
 
   // ---- combine the workgroup's partials in a fixed order ----
   if (GRAD) {
     double* out = a.part_g + (int64_t)blockIdx.x * a.pitch;
-    if (WROW == 1) {
+    __shared__ v2d gx[(WROW > 1) ? (WROW - 1) * kWave : 1];
+    // one column pair per lane: sum over the workgroup's row groups in wave
+    // order (uniform call: every wave of the workgroup passes through)
+    auto emit = [&](v2d v, bool mine, double* dst) {
+      if (WROW == 1) {
+        if (mine) *reinterpret_cast<v2d*>(dst) = v;
+      } else {
+        if (wr > 0) gx[(wr - 1) * kWave + lane] = v;
+        __syncthreads();
+        if (wr == 0) {
 #pragma unroll
-      for (int c = 0; c < NCH; ++c)
-        if (c < my_nch && (c != ragged_c || lane_in_ragged))
-          *reinterpret_cast<v2d*>(out + col0 + (int64_t)c * kChunkCols) = acc[c];
-    } else {
-      __shared__ v2d gx[(WROW > 1) ? (WROW - 1) * kWave : 1];
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        if (c < my_nch) {  // uniform over the workgroup (WCOL == 1 here)
-          if (wr > 0) gx[(wr - 1) * kWave + lane] = acc[c];
-          __syncthreads();
-          if (wr == 0) {
-            v2d s = acc[c];
-#pragma unroll
-            for (int w = 1; w < WROW; ++w) {
-              const v2d o = gx[(w - 1) * kWave + lane];
-              s.x += o.x;
-              s.y += o.y;
-            }
-            if (c != ragged_c || lane_in_ragged)
-              *reinterpret_cast<v2d*>(out + col0 + (int64_t)c * kChunkCols) = s;
+          for (int k = 1; k < WROW; ++k) {
+            const v2d o = gx[(k - 1) * kWave + lane];
+            v.x += o.x;
+            v.y += o.y;
           }
-          __syncthreads();
+          if (mine) *reinterpret_cast<v2d*>(dst) = v;
         }
+        __syncthreads();
       }
+    };
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+      if (c < my_nch)  // uniform over the workgroup when WROW > 1 (WCOL == 1 there)
+        emit(acc[c], c != ragged_c || lane_in_ragged, out + col0 + (int64_t)c * kChunkCols);
+    if constexpr (TL > 0) {
+      // the leftover columns: fold the row segments of the wave first
+#pragma unroll
+      for (int m = kLpr; m < kWave; m <<= 1) {
+        acct.x += __shfl_xor(acct.x, m, kWave);
+        acct.y += __shfl_xor(acct.y, m, kWave);
+      }
+      emit(acct, lane < kLpr && w.tail_in, out + kBodyCols + 2 * tail_pair);
     }
   }
   if constexpr (MODE == kPassFused) {  // the sweeps of a blocked row carry no loss

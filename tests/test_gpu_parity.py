@@ -58,6 +58,46 @@ def test_loss_grad_matches_oracle(plr, oracle, gen, n, d):
     assert abs(loss - loss_ref) <= LOSS_TOL * abs(loss_ref)
 
 
+# rows that end a few columns past a 128-column chunk boundary (the file path's
+# bias column makes 2^k + 1 the common width): (full chunks, leftover columns)
+# for every tail-stage variant at its smallest and largest leftover, odd and
+# even widths, with row counts that leave partial tiles and partial tail loads
+TAIL_CASES = [(k, t) for k in (1, 2) for t in (1, 2, 7, 8, 9, 16, 17, 31, 32, 33, 63, 64)] + \
+             [(k, t) for k in (3, 4) for t in (1, 15, 16, 17, 32)] + \
+             [(k, t) for k in (6, 7, 9, 10, 11) for t in (1, 32)] + \
+             [(8, t) for t in (1, 31, 32, 33, 64)] + \
+             [(k, t) for k in (12, 13, 14, 15, 16) for t in (1, 64)]
+
+
+@pytest.mark.parametrize("k,t", TAIL_CASES)
+def test_rows_just_past_a_chunk_boundary(plr, oracle, gen, k, t):
+    d = 128 * k + t
+    for n in (1, 3, 77, 1543):
+        print("case n=%d d=%d" % (n, d), flush=True)
+        X, y, th = make(gen, n, d, seed=0x7A11 + d)
+        plr.set_data(X, y)
+        if n == 1:
+            print(plr.kernel_info(), flush=True)
+            if d < 2048:
+                assert "tail=%d" % (t + (t & 1)) in plr.kernel_info()
+        g, loss, n_out = plr.loss_grad(th)
+        assert n_out == n
+        assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
+        loss_ref = oracle.calc_loss_sum(X, y, th)
+        assert abs(loss - loss_ref) <= LOSS_TOL * abs(loss_ref)
+        # the passes without a gradient take their own instances
+        l2, _ = plr.calc_loss(th)
+        assert abs(l2 - loss_ref) <= LOSS_TOL * abs(loss_ref)
+        h = plr.predict(th)
+        assert np.max(np.abs(h - oracle.predict(X, th))) <= 1e-14
+    # the last column matters: a spike there must show in its gradient entry alone
+    X2 = X.copy()
+    X2[:, d - 1] += 1.0
+    plr.set_data(X2, y)
+    g2, _, _ = plr.loss_grad(np.zeros(d))
+    assert rel(g2, X2.T @ (0.5 - y)) <= GRAD_TOL
+
+
 @pytest.mark.parametrize("n,d", [(1000, 100), (2051, 1000), (333, 257), (70, 8193), (37, 16385)])
 def test_dgd_delta_matches_oracle(plr, oracle, gen, n, d):
     X, y, th = make(gen, n, d)
