@@ -55,6 +55,11 @@ def parse_args():
     ap.add_argument("--e2e", action="store_true",
                     help="end-to-end rounds through the host parameter server (C++ worker + "
                          "plr_ps_server over ZeroMQ) instead of the bare gradient step")
+    ap.add_argument("--no-dense-ps", action="store_true",
+                    help="with --e2e: start the server with its dense-vector fast path off")
+    ap.add_argument("--ps-roundtrip", action="store_true",
+                    help="host only: microseconds per paracel_read / paracel_bupdate round trip "
+                         "against plr_ps_server, dense fast path on and off")
     return ap.parse_args()
 
 
@@ -180,7 +185,12 @@ def run_e2e(a, cfg):
     import numpy as np
 
     pkg = os.path.join(ROOT, "paracel_amd")
-    srv = subprocess.Popen([os.path.join(pkg, "plr_ps_server")], stdout=subprocess.PIPE, text=True)
+    if cfg.spec.kind != 0 or cfg.spec.zero_prob != 0.0 or cfg.spec.outlier_mod != 0:
+        raise SystemExit("bench.py --e2e: the worker's --synthetic mode generates plain normal "
+                         "shards only (c1, c2, c5)")
+    srv = subprocess.Popen([os.path.join(pkg, "plr_ps_server")] +
+                           (["--no-dense"] if a.no_dense_ps else []),
+                           stdout=subprocess.PIPE, text=True)
     try:
         info = srv.stdout.readline().strip()
         with tempfile.TemporaryDirectory() as td:
@@ -206,6 +216,7 @@ def run_e2e(a, cfg):
         "config": {"workload": cfg.name + " via parameter server", "n": cfg.n, "d": cfg.d,
                    "step": "paracel_read theta -> plr_dgd_delta -> paracel_bupdate delta "
                            "(ZeroMQ REQ/REP, msgpack, dlopen'ed lr_theta_update)",
+                   "ps_dense_fast_path": not a.no_dense_ps,
                    "alpha": cfg.alpha, "beta": cfg.beta},
         "gpu_only_iters_per_sec": rep["gpu_only_iters_per_sec"],
         "gpu_kernel_ms_per_iter": rep["gpu_kernel_ms_per_iter"],
@@ -235,12 +246,43 @@ def run_e2e(a, cfg):
     print(json.dumps(out), flush=True)
 
 
+def run_ps_roundtrip(a):
+    """Host only: what a DGD round costs besides the gradient -- the two
+    parameter-server calls, timed by plr_ps_roundtrip with the server's dense
+    fast path on and off."""
+    import subprocess
+
+    pkg = os.path.join(ROOT, "paracel_amd")
+    out = {"metric": "ps_round_trip_us", "unit": "us", "widths": {}, "iters": 2000}
+    for mode in ("dense", "packed"):
+        srv = subprocess.Popen([os.path.join(pkg, "plr_ps_server")] +
+                               ([] if mode == "dense" else ["--no-dense"]),
+                               stdout=subprocess.PIPE, text=True)
+        try:
+            info = srv.stdout.readline().strip()
+            r = subprocess.run([os.path.join(pkg, "plr_ps_roundtrip"), "--server_info", info,
+                                "--update_file", os.path.join(pkg, "liblr_update.so"),
+                                "--d", "100,512,1001,16385", "--iters", "2000"],
+                               capture_output=True, text=True, check=True)
+        finally:
+            srv.kill()
+            srv.wait()
+        for line in r.stdout.strip().splitlines():
+            rec = json.loads(line)
+            out["widths"].setdefault(str(rec["d"]), {})[mode] = {
+                "read_us": rec["read_us"], "bupdate_us": rec["bupdate_us"]}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     a = parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU's shard: this build has no multi-GPU path "
               "(run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+    if a.ps_roundtrip:
+        run_ps_roundtrip(a)
+        return
 
     import numpy as np  # noqa: F401
 

@@ -54,10 +54,10 @@ def build_copy_probe():
 def build_worker():
     """Host side of the worker path (g++): parameter-server process, reducer
     plugin, GPU LR worker, shard tool ->
-    paracel_amd/{plr_ps_server,liblr_update.so,plr_lr_worker,plr_shard_tool}"""
+    paracel_amd/{plr_ps_server,liblr_update.so,plr_lr_worker,plr_shard_tool,plr_ps_roundtrip}"""
     _run(["make", "-B", "-C", os.path.join(_HERE, "worker")])
     return [os.path.join(_HERE, f) for f in ("plr_ps_server", "liblr_update.so", "plr_lr_worker",
-                                             "plr_shard_tool")]
+                                             "plr_shard_tool", "plr_ps_roundtrip")]
 
 
 def build_all():

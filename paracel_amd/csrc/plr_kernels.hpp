@@ -17,9 +17,9 @@
 //     row's partial, log2(64/R) plain butterfly steps finish it.  So the
 //     exp/log of a row is evaluated once per tile by the lane that holds
 //     it, not 64 times, and R-1+log2(64/R) lane exchanges replace 6R.
-//   * Rows of more than 16 chunks: WCOL waves of a workgroup split the columns; their partial
-//     dots meet in LDS (double-buffered, one barrier per tile) and are summed
-//     in wave order.
+//   * Rows of more than 16 chunks: WCOL waves of a workgroup split the
+//     columns; their partial dots meet in LDS (double-buffered, one barrier
+//     per tile) and are summed in wave order.
 //   * A row that ends a few columns past a chunk boundary (the file path
 //     always adds a bias column, so 256 features arrive as 257 columns) does
 //     not get a nearly empty chunk of its own: the TL > 0 variants cover the

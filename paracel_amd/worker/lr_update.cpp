@@ -8,6 +8,8 @@
 
 extern "C" {
 extern plr_ps::update_result lr_theta_update;
+// dense twin (see ps_plugin.hpp): the same additions on unpacked doubles
+void lr_theta_update_dense(double* theta, const double* delta, size_t n);
 }
 
 static std::vector<double> add_delta(std::vector<double> theta, std::vector<double> delta) {
@@ -17,3 +19,7 @@ static std::vector<double> add_delta(std::vector<double> theta, std::vector<doub
 }
 
 plr_ps::update_result lr_theta_update = plr_ps::update_proxy(add_delta);
+
+void lr_theta_update_dense(double* theta, const double* delta, size_t n) {
+  for (size_t i = 0; i < n; ++i) theta[i] = theta[i] + delta[i];
+}

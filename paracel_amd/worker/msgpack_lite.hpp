@@ -86,9 +86,31 @@ inline void enc(std::string& o, double d) {
   put_be(o, u, 8);
 }
 
-inline void enc(std::string& o, const std::vector<double>& v) {
-  const size_t n = v.size();
-  o.reserve(o.size() + 5 + 9 * n);
+// A run of n float64 elements (cb + 8 bytes big-endian each, 9n bytes) in one
+// pass without per-byte appends: model vectors are 10^3..10^5 doubles and
+// cross the wire twice per round.
+inline void enc_f64_run(char* dst, const double* v, size_t n) {
+  for (size_t i = 0; i < n; ++i, dst += 9) {
+    uint64_t u;
+    memcpy(&u, v + i, 8);
+    u = __builtin_bswap64(u);
+    dst[0] = (char)0xcb;
+    memcpy(dst + 1, &u, 8);
+  }
+}
+// false (v partly written) if an element is not tagged float64
+inline bool dec_f64_run(const unsigned char* src, double* v, size_t n) {
+  for (size_t i = 0; i < n; ++i, src += 9) {
+    if (src[0] != 0xcb) return false;
+    uint64_t u;
+    memcpy(&u, src + 1, 8);
+    u = __builtin_bswap64(u);
+    memcpy(v + i, &u, 8);
+  }
+  return true;
+}
+
+inline void enc_array_header(std::string& o, size_t n) {
   if (n < 16) {
     o.push_back((char)(0x90 | n));
   } else if (n < 65536) {
@@ -98,8 +120,16 @@ inline void enc(std::string& o, const std::vector<double>& v) {
     o.push_back((char)0xdd);
     put_be(o, n, 4);
   }
-  for (double d : v) enc(o, d);
 }
+
+inline void enc(std::string& o, const double* v, size_t n) {
+  o.reserve(o.size() + 5 + 9 * n);
+  enc_array_header(o, n);
+  const size_t at = o.size();
+  o.resize(at + 9 * n);
+  enc_f64_run(&o[at], v, n);
+}
+inline void enc(std::string& o, const std::vector<double>& v) { enc(o, v.data(), v.size()); }
 
 struct Reader {
   const unsigned char* p;
@@ -184,6 +214,12 @@ inline void dec(Reader& r, std::vector<double>& v) {
   else if (t == 0xdd) n = r.be(4);
   else throw std::runtime_error("msgpack: not an array");
   v.resize(n);
+  // all-float64 arrays (what a packed vector<double> always is) in one pass;
+  // anything else (integers or float32 among the elements) element by element
+  if ((size_t)(r.end - r.p) >= 9 * n && dec_f64_run(r.p, v.data(), n)) {
+    r.p += 9 * n;
+    return;
+  }
   for (size_t i = 0; i < n; ++i) dec(r, v[i]);
 }
 
@@ -221,6 +257,52 @@ T unpack(const std::string& s) {
   return v;
 }
 
+// A framed field seen in place as an array of n float64 elements (the packed
+// form of vector<double>): elems points at the first cb tag.  False if the
+// field is anything else, or shorter than its header claims.  The element
+// tags are checked by dec_f64_run when the run is read.
+struct F64ArrayView {
+  const unsigned char* elems;
+  size_t n;
+};
+inline bool view_f64_array(const char* field, size_t len, F64ArrayView& out) {
+  if (len < sizeof(size_t) + 1) return false;
+  size_t body;
+  memcpy(&body, field, sizeof body);
+  if (len - sizeof body < body || body < 1) return false;
+  const unsigned char* p = (const unsigned char*)field + sizeof body;
+  const unsigned char* end = p + body;
+  const uint8_t t = *p++;
+  size_t n;
+  if ((t & 0xf0) == 0x90) {
+    n = t & 0x0f;
+  } else if (t == 0xdc) {
+    if (end - p < 2) return false;
+    n = ((size_t)p[0] << 8) | p[1];
+    p += 2;
+  } else if (t == 0xdd) {
+    if (end - p < 4) return false;
+    n = ((size_t)p[0] << 24) | ((size_t)p[1] << 16) | ((size_t)p[2] << 8) | p[3];
+    p += 4;
+  } else {
+    return false;
+  }
+  if ((size_t)(end - p) != 9 * n) return false;
+  out.elems = p;
+  out.n = n;
+  return true;
+}
+
+// Append the framed form of n doubles to a request buffer without an
+// intermediate string (same bytes as pack(std::vector<double>)).
+inline void append_packed(std::string& o, const double* v, size_t n) {
+  const size_t at = o.size();
+  o.append(sizeof(size_t), '\0');
+  detail::enc(o, v, n);
+  const size_t body = o.size() - at - sizeof(size_t);
+  memcpy(&o[at], &body, sizeof body);
+}
+
 // Request assembly: fields joined by the literal separator
 // (include/paracel_types.hpp:49, include/client.hpp:523-539); the server
 // splits on it and drops a trailing empty field
@@ -251,6 +333,29 @@ inline std::vector<std::string> split_fields(const std::string& scrip) {
   }
   if (!out.empty() && out.back().empty()) out.pop_back();
   return out;
+}
+
+
+// The same split without copying the fields: (pointer, length) pairs into scrip.
+struct FieldView {
+  const char* p;
+  size_t n;
+  std::string str() const { return std::string(p, n); }
+};
+inline void split_field_views(const std::string& scrip, std::vector<FieldView>& out) {
+  out.clear();
+  const size_t sl = sizeof(kSeparator) - 1;
+  size_t st = 0;
+  for (;;) {
+    const size_t en = scrip.find(kSeparator, st);
+    if (en == std::string::npos) {
+      out.push_back(FieldView{scrip.data() + st, scrip.size() - st});
+      break;
+    }
+    out.push_back(FieldView{scrip.data() + st, en - st});
+    st = en + sl;
+  }
+  if (!out.empty() && out.back().n == 0) out.pop_back();
 }
 
 }  // namespace plr_ps

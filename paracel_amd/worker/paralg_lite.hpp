@@ -62,6 +62,44 @@ class kvclt {
     r = req(3, paste({pack<std::string>("bupdate"), pack(key), pack(delta)}), val);
     return val;
   }
+
+  // Dense-vector forms of pull and bupdate: the same bytes on the wire, but
+  // the vector is encoded straight into the request buffer and decoded
+  // straight out of the reply message (no intermediate packed strings), and
+  // bupdate's reply -- the new value, which the non-SSP worker unpacks and
+  // drops (ps.hpp:753-770) -- is only checked, not decoded.
+  bool pull(const std::string& key, std::vector<double>& val) {
+    buf_.clear();
+    buf_.append(pack<std::string>("pull")).append(kSeparator).append(pack(key));
+    zmq_msg_t m;
+    roundtrip(0, buf_, &m);
+    const char* p = (const char*)zmq_msg_data(&m);
+    const size_t n = zmq_msg_size(&m);
+    bool ok = !(n == 5 && memcmp(p, "nokey", 5) == 0);
+    if (ok) {
+      F64ArrayView a;
+      if (view_f64_array(p, n, a)) {
+        val.resize(a.n);
+        if (!detail::dec_f64_run(a.elems, val.data(), a.n))
+          val = unpack<std::vector<double> >(std::string(p, n));
+      } else {
+        val = unpack<std::vector<double> >(std::string(p, n));
+      }
+    }
+    zmq_msg_close(&m);
+    return ok;
+  }
+  bool bupdate_drop(const std::string& key, const std::vector<double>& delta) {
+    buf_.clear();
+    buf_.append(pack<std::string>("bupdate")).append(kSeparator).append(pack(key));
+    buf_.append(kSeparator);
+    append_packed(buf_, delta.data(), delta.size());
+    zmq_msg_t m;
+    roundtrip(3, buf_, &m);
+    const bool ok = !(zmq_msg_size(&m) == 5 && memcmp(zmq_msg_data(&m), "nokey", 5) == 0);
+    zmq_msg_close(&m);
+    return ok;
+  }
   bool push_int(const std::string& key, int v) {
     bool stat = true;
     const bool r = req(4, paste({pack<std::string>("push_int"), pack(key), pack(v)}), stat);
@@ -74,8 +112,10 @@ class kvclt {
   }
 
  private:
-  template <class V>
-  bool req(int port_idx, const std::string& scrip, V& val) {
+  // one strictly alternating send/recv on the op family's REQ socket; the
+  // caller closes *m.  An empty reply is the reference's internal error
+  // (client.hpp:551).
+  void roundtrip(int port_idx, const std::string& scrip, zmq_msg_t* m) {
     void*& s = socks_[port_idx];
     if (!s) {
       s = zmq_socket(zctx_, ZMQ_REQ);
@@ -85,15 +125,22 @@ class kvclt {
     }
     if (zmq_send(s, scrip.data(), scrip.size(), 0) < 0)
       throw std::runtime_error(std::string("zmq_send: ") + zmq_strerror(zmq_errno()));
-    zmq_msg_t m;
-    zmq_msg_init(&m);
-    if (zmq_msg_recv(&m, s, 0) < 0) {
-      zmq_msg_close(&m);
+    zmq_msg_init(m);
+    if (zmq_msg_recv(m, s, 0) < 0) {
+      zmq_msg_close(m);
       throw std::runtime_error(std::string("zmq_recv: ") + zmq_strerror(zmq_errno()));
     }
+    if (zmq_msg_size(m) == 0) {
+      zmq_msg_close(m);
+      throw std::runtime_error("paracel internal error!");
+    }
+  }
+  template <class V>
+  bool req(int port_idx, const std::string& scrip, V& val) {
+    zmq_msg_t m;
+    roundtrip(port_idx, scrip, &m);
     std::string data((const char*)zmq_msg_data(&m), zmq_msg_size(&m));
     zmq_msg_close(&m);
-    if (data.empty()) throw std::runtime_error("paracel internal error!");  // client.hpp:551
     if (data == "nokey") return false;
     val = unpack<V>(data);
     return true;
@@ -103,6 +150,7 @@ class kvclt {
   std::vector<std::string> ports_;
   void* zctx_;
   void* socks_[5];
+  std::string buf_;  // request buffer of the dense forms, reused across rounds
 };
 
 class paralg {
@@ -174,6 +222,9 @@ class paralg {
     bool r = false;
     (void)srv(key).bupdate(key, delta, r);
     return r;
+  }
+  bool paracel_bupdate(const std::string& key, const std::vector<double>& delta) {
+    return srv(key).bupdate_drop(key, delta);
   }
   void paracel_sync() {}                       // ps.hpp:890-892 (MPI_Barrier; 1 worker)
   size_t get_worker_id() const { return rank_; }

@@ -13,8 +13,17 @@
 // The reference's servers report their ports to a collector process; this one
 // prints "host:p0,p1,p2,p3,p4" (the format of utils.hpp:80-92) on stdout.
 //
-// Usage: plr_ps_server [--host 127.0.0.1]      (runs until killed, like the
-// reference's start_server, which prun.py ends with killpg)
+// Dense-vector fast path (not in the reference; same bytes on the wire and in
+// the store): requests are split into views instead of copied fields, and a
+// bupdate whose stored value and delta are both packed vector<double> of one
+// length, under a reducer that exports a "<func>_dense" twin, is folded on
+// unpacked doubles and re-encoded into the stored bytes in place -- one
+// decode of each operand and one encode instead of the two by-value string
+// copies, two unpacks, one pack and two more copies of the packed path.
+// --no-dense switches it off (for A/B timing and tests).
+//
+// Usage: plr_ps_server [--host 127.0.0.1] [--no-dense]   (runs until killed,
+// like the reference's start_server, which prun.py ends with killpg)
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -33,6 +42,7 @@ using namespace plr_ps;
 static std::unordered_map<std::string, std::string> tbl_store;  // kv_def.hpp:23
 static std::unordered_map<std::string, int> ssp_tbl;            // kv_def.hpp:24
 static std::mutex store_mutex;                                   // server.hpp:36
+static bool dense_enabled = true;
 
 static bool recv_all(void* sock, std::string& out) {
   zmq_msg_t m;
@@ -49,44 +59,64 @@ static bool recv_all(void* sock, std::string& out) {
 
 static void reply(void* sock, const std::string& s) { zmq_send(sock, s.data(), s.size(), 0); }
 
+// Fold a packed delta into a packed stored value through the reducer's dense
+// twin.  True if done (stored holds the new value, same length as before);
+// false if either side is not an all-float64 array or the lengths differ --
+// the caller then takes the packed path.  acc/dl are the thread's scratch.
+static bool dense_fold(std::string& stored, const FieldView& delta, dense_update_fn f,
+                       std::vector<double>& acc, std::vector<double>& dl) {
+  F64ArrayView a, b;
+  if (!view_f64_array(stored.data(), stored.size(), a) ||
+      !view_f64_array(delta.p, delta.n, b) || a.n != b.n)
+    return false;
+  acc.resize(a.n);
+  dl.resize(b.n);
+  if (!detail::dec_f64_run(a.elems, acc.data(), a.n) ||
+      !detail::dec_f64_run(b.elems, dl.data(), b.n))
+    return false;
+  f(acc.data(), dl.data(), a.n);
+  detail::enc_f64_run(&stored[(const char*)a.elems - stored.data()], acc.data(), a.n);
+  return true;
+}
+
 static void op_thread(void* sock) {
   update_result update_f;
+  dense_update_fn dense_f = nullptr;
+  std::vector<double> acc, dl;
   std::string scrip;
+  std::vector<FieldView> msg;
   while (recv_all(sock, scrip)) {
-    std::vector<std::string> msg = split_fields(scrip);
+    split_field_views(scrip, msg);
     std::string op;
     try {
-      op = unpack<std::string>(msg.at(0));
+      op = unpack<std::string>(msg.at(0).str());
       if (op == "contains") {
         std::lock_guard<std::mutex> g(store_mutex);
-        reply(sock, pack<bool>(tbl_store.count(unpack<std::string>(msg.at(1))) != 0));
+        reply(sock, pack<bool>(tbl_store.count(unpack<std::string>(msg.at(1).str())) != 0));
       } else if (op == "pull") {
-        std::string val;
-        bool exist;
-        {
-          std::lock_guard<std::mutex> g(store_mutex);
-          auto it = tbl_store.find(unpack<std::string>(msg.at(1)));
-          exist = it != tbl_store.end();
-          if (exist) val = it->second;
-        }
-        reply(sock, exist ? val : std::string("nokey"));
+        // the stored bytes go out verbatim; zmq_send copies them, so sending
+        // under the lock saves a copy of the value
+        std::lock_guard<std::mutex> g(store_mutex);
+        auto it = tbl_store.find(unpack<std::string>(msg.at(1).str()));
+        if (it != tbl_store.end()) reply(sock, it->second);
+        else reply(sock, std::string("nokey"));
       } else if (op == "register_bupdate" || op == "register_update") {
         std::string err;
-        if (!load_update_plugin(unpack<std::string>(msg.at(1)), unpack<std::string>(msg.at(2)),
-                                update_f, err)) {
+        if (!load_update_plugin(unpack<std::string>(msg.at(1).str()),
+                                unpack<std::string>(msg.at(2).str()), update_f, err, &dense_f)) {
           fprintf(stderr, "%s\n", err.c_str());  // the reference aborts here
           abort();
         }
         reply(sock, pack<bool>(true));
       } else if (op == "push") {
         std::lock_guard<std::mutex> g(store_mutex);
-        tbl_store[unpack<std::string>(msg.at(1))] = msg.at(2);  // stored verbatim
+        tbl_store[unpack<std::string>(msg.at(1).str())] = msg.at(2).str();  // stored verbatim
         reply(sock, pack<bool>(true));
       } else if (op == "update" || op == "bupdate") {
         if (msg.size() == 5) {
           std::string err;
-          if (!load_update_plugin(unpack<std::string>(msg[3]), unpack<std::string>(msg[4]),
-                                  update_f, err)) {
+          if (!load_update_plugin(unpack<std::string>(msg[3].str()),
+                                  unpack<std::string>(msg[4].str()), update_f, err, &dense_f)) {
             fprintf(stderr, "%s\n", err.c_str());
             abort();
           }
@@ -95,23 +125,22 @@ static void op_thread(void* sock) {
           fprintf(stderr, "bupdate before register_bupdate on this port\n");
           abort();
         }
-        std::string result;
         {
           std::lock_guard<std::mutex> g(store_mutex);
-          const std::string key = unpack<std::string>(msg.at(1));
+          const std::string key = unpack<std::string>(msg.at(1).str());
           auto it = tbl_store.find(key);
           if (it == tbl_store.end()) {
-            tbl_store[key] = msg.at(2);  // first update of a missing key = set
-            result = msg[2];
-          } else {
-            it->second = update_f(it->second, msg.at(2));
-            result = it->second;
+            // first update of a missing key = set
+            it = tbl_store.emplace(key, msg.at(2).str()).first;
+          } else if (!(dense_enabled && dense_f &&
+                       dense_fold(it->second, msg.at(2), dense_f, acc, dl))) {
+            it->second = update_f(it->second, msg.at(2).str());
           }
+          reply(sock, it->second);  // the new value
         }
-        reply(sock, result);
       } else if (op == "remove") {
         std::lock_guard<std::mutex> g(store_mutex);
-        reply(sock, pack<bool>(tbl_store.erase(unpack<std::string>(msg.at(1))) != 0));
+        reply(sock, pack<bool>(tbl_store.erase(unpack<std::string>(msg.at(1).str())) != 0));
       } else if (op == "clear") {
         std::lock_guard<std::mutex> g(store_mutex);
         tbl_store.clear();
@@ -157,8 +186,10 @@ static void ssp_thread(void* sock) {
 
 int main(int argc, char** argv) {
   std::string host = "127.0.0.1";
-  for (int i = 1; i + 1 < argc; ++i)
-    if (!strcmp(argv[i], "--host")) host = argv[i + 1];
+  for (int i = 1; i < argc; ++i) {
+    if (!strcmp(argv[i], "--host") && i + 1 < argc) host = argv[++i];
+    else if (!strcmp(argv[i], "--no-dense")) dense_enabled = false;
+  }
   void* ctx = zmq_ctx_new();
   const int kThreads = 5;  // paracel_types.hpp:45 threads_num
   void* socks[kThreads];

@@ -24,10 +24,10 @@ ZMQ_REQ = 3
 
 
 def _need_host_binaries():
-    if not all(os.path.exists(os.path.join(PKG, f)) for f in
-               ("plr_ps_server", "liblr_update.so")):
-        subprocess.run(["make", "-C", os.path.join(PKG, "worker"), os.path.join("..", "plr_ps_server"),
-                        os.path.join("..", "liblr_update.so")], check=True)
+    names = ("plr_ps_server", "liblr_update.so", "plr_ps_roundtrip")
+    if not all(os.path.exists(os.path.join(PKG, f)) for f in names):
+        subprocess.run(["make", "-C", os.path.join(PKG, "worker")] +
+                       [os.path.join("..", f) for f in names], check=True)
 
 
 def field(obj):
@@ -78,11 +78,19 @@ class Zmq:
             self.lib.zmq_close(s)
 
 
-@pytest.fixture()
-def server():
+def _start_server(dense):
     _need_host_binaries()
-    p = subprocess.Popen([os.path.join(PKG, "plr_ps_server")], stdout=subprocess.PIPE, text=True)
+    cmd = [os.path.join(PKG, "plr_ps_server")] + ([] if dense else ["--no-dense"])
+    p = subprocess.Popen(cmd, stdout=subprocess.PIPE, text=True)
     info = p.stdout.readline().strip()
+    return p, info
+
+
+# every wire test runs against the server with its dense-vector fast path on
+# (the default) and off: the bytes on the wire must not depend on it
+@pytest.fixture(params=["dense", "packed"])
+def server(request):
+    p, info = _start_server(request.param == "dense")
     host, ports = info.split(":")
     z = Zmq()
     yield z, host, ports.split(","), info
@@ -152,3 +160,82 @@ def test_integers_arrive_as_doubles(server):
     z.req(host, ports[1], SEP.join([field("push"), field("ints"), field([1, -2, 300, 70000, -70000])]))
     r = z.req(host, ports[3], SEP.join([field("bupdate"), field("ints"), field([0.5] * 5)]))
     assert unfield(r) == [1.5, -1.5, 300.5, 70000.5, -69999.5]
+
+
+def test_dense_fold_gives_the_packed_reducers_bytes():
+    # the same push / bupdate sequence against both servers: every reply and the
+    # stored value must agree byte for byte, special values included
+    so = os.path.join(PKG, "liblr_update.so")
+    rng = np.random.default_rng(7)
+    n = 3001
+    theta = rng.normal(size=n)
+    theta[:8] = [0.0, -0.0, np.inf, -np.inf, np.nan, 5e-324, -1.7976931348623157e308, 1.0]
+    deltas = [rng.normal(size=n) * 10.0 ** rng.integers(-12, 12) for _ in range(6)]
+    deltas[2][:8] = [-0.0, 0.0, -np.inf, -np.inf, 1.0, -5e-324, -1.7976931348623157e308, 2.0 ** -53]
+    replies = {}
+    for mode in ("dense", "packed"):
+        p, info = _start_server(mode == "dense")
+        host, ports = info.split(":")
+        ports = ports.split(",")
+        z = Zmq()
+        try:
+            z.req(host, ports[3], SEP.join([field("register_bupdate"), field(so), field("lr_theta_update")]))
+            z.req(host, ports[1], SEP.join([field("push"), field("theta"), field(theta.tolist())]))
+            out = []
+            for dl in deltas:
+                out.append(z.req(host, ports[3], SEP.join([field("bupdate"), field("theta"),
+                                                           field(dl.tolist())])))
+            out.append(z.req(host, ports[0], SEP.join([field("pull"), field("theta")])))
+            # a delta of another length, and one carrying integers, take the packed path
+            out.append(z.req(host, ports[1], SEP.join([field("push"), field("short"),
+                                                       field([1.0, 2.0, 3.0])])))
+            out.append(z.req(host, ports[3], SEP.join([field("bupdate"), field("short"),
+                                                       field([1.0, 2.0, 3.0, 4.0])])))
+            out.append(z.req(host, ports[3], SEP.join([field("bupdate"), field("short"),
+                                                       field([1, 2.5, -3])])))
+            replies[mode] = out
+        finally:
+            z.close()
+            p.kill()
+            p.wait()
+    assert replies["dense"] == replies["packed"]
+    # and both are the plain additions
+    want = theta.copy()
+    with np.errstate(invalid="ignore", over="ignore"):
+        for dl in deltas:
+            want = want + dl
+    got = np.array(unfield(replies["dense"][len(deltas)]))
+    assert got.tobytes() == want.tobytes()
+    assert unfield(replies["dense"][-1]) == [3.0, 6.5, 3.0]
+
+
+def test_worker_client_round_trips_against_both_servers():
+    # the C++ client's dense pull / bupdate forms (the calls a DGD round makes):
+    # theta after warmup + iters additions, hashed by the tool, against numpy
+    so = os.path.join(PKG, "liblr_update.so")
+    widths = (1, 15, 16, 512, 70001)
+    iters, warmup = 7, 2
+    for mode in ("dense", "packed"):
+        p, info = _start_server(mode == "dense")
+        try:
+            r = subprocess.run([os.path.join(PKG, "plr_ps_roundtrip"), "--server_info", info,
+                                "--update_file", so, "--d", ",".join(map(str, widths)),
+                                "--iters", str(iters), "--warmup", str(warmup)],
+                               capture_output=True, text=True, timeout=120)
+            assert r.returncode == 0, r.stderr
+        finally:
+            p.kill()
+            p.wait()
+        lines = [__import__("json").loads(l) for l in r.stdout.strip().splitlines()]
+        assert [l["d"] for l in lines] == list(widths)
+        for l in lines:
+            d = l["d"]
+            i = np.arange(d)
+            th = 0.25 + i / 1048576.0
+            dl = ((i % 7) - 3) / 1024.0
+            for _ in range(iters + warmup):
+                th = th + dl
+            h = 1469598103934665603
+            for b in th.tobytes():
+                h = ((h ^ b) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+            assert l["theta_fnv1a"] == "%016x" % h
