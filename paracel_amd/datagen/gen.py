@@ -149,6 +149,11 @@ def configs():
                                        1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
         "c4b_wide_200k_x_16385": Config("c4b_wide_200k_x_16385", 200_000, 16385, 0x5EED0004, NORMAL,
                                         1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
+        # config 3 as the file path sees it: 256 features + the bias column (lr.cpp:83) -- a row
+        # that ends two columns past a chunk boundary (tail-stage kernel variant)
+        "x_bias_10m_x_257": Config("x_bias_10m_x_257", 10_000_000, 257, 0x5EED0008, UNIFORM, 1.0,
+                                   lam=0.001, outlier_mod=100, outlier_scale=100.0,
+                                   theta_scale=0.1),
         # narrow rows: the packed-row kernel (several whole rows per 128-double chunk)
         "x_narrow_30m_x_16": Config("x_narrow_30m_x_16", 30_000_000, 16, 0x5EED0007, NORMAL, 0.25,
                                     lam=0.01),
