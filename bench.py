@@ -37,7 +37,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c4_wide_200k_x_16384": 26261494739,
     "c4b_wide_200k_x_16385": 26466443874,
     "c5_e2e_2m_x_512": 8210210591,
-    "x_bias_10m_x_257": 21202464441,
+    "x_bias_10m_x_257": 21202464437,
 }
 
 
