@@ -416,11 +416,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   return PLR_OK;
 }
 
-int alloc_shape(plr_ctx* c, int64_t n, int64_t d) {
-  if (n < 0 || d < 1)
-    return fail(c, PLR_ERR_INVALID, "need n >= 0 and d >= 1");
-  PLR_HIP(c, hipSetDevice(c->device));
-  free_shape(c);
+int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d) {
   int rc = plan_shape(c, n, d);
   if (rc != PLR_OK) return rc;
   c->n = n;
@@ -458,6 +454,18 @@ int alloc_shape(plr_ctx* c, int64_t n, int64_t d) {
   PLR_HIP(c, hipStreamSynchronize(c->stream));
   c->have_data = true;
   return PLR_OK;
+}
+
+// Drop the resident shard (if any) and reserve an n x d one.  On failure the
+// context is left without a shard (shape 0 x 0), never half allocated.
+int alloc_shape(plr_ctx* c, int64_t n, int64_t d) {
+  if (n < 0 || d < 1)
+    return fail(c, PLR_ERR_INVALID, "need n >= 0 and d >= 1");
+  PLR_HIP(c, hipSetDevice(c->device));
+  free_shape(c);
+  const int rc = alloc_shape_buffers(c, n, d);
+  if (rc != PLR_OK) free_shape(c);  // keeps c->err
+  return rc;
 }
 
 int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,

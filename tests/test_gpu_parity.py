@@ -371,6 +371,27 @@ def test_errors(plr):
     assert e.value.code == -1
 
 
+def test_a_shard_that_does_not_fit_is_refused_cleanly(plr, oracle, gen):
+    from paracel_amd import PlrError
+
+    X, y, th = make(gen, 300, 257)
+    plr.set_data(X, y)
+    # 2^40 rows of 1000 doubles = 8 PB: the device allocation fails, nothing is computed
+    with pytest.raises(PlrError) as e:
+        plr.alloc_data(1 << 40, 1000)
+    assert e.value.code == -3  # PLR_ERR_NOMEM
+    assert "hipMalloc" in str(e.value)
+    # the context holds no shard afterwards (the old one was dropped, the new one never existed)
+    assert plr.shape == (0, 0)
+    with pytest.raises(PlrError) as e:
+        plr.loss_grad(np.zeros(0))
+    assert e.value.code == -4
+    # and is usable again
+    plr.set_data(X, y)
+    g, _, _ = plr.loss_grad(th)
+    assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
+
+
 def test_config1_trajectory_100_iterations(plr, oracle, gen):
     # dense n=100000 d=100, theta0=0, lr=0.1, lam=0.01 => alpha=lr/n, beta=lam/2;
     # 100 full-batch rounds of read theta -> delta -> theta += delta
