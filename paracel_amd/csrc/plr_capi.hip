@@ -43,11 +43,15 @@ struct Variant {
    {{nullptr, plr::shard_pass<NCH, R, 1, WROW, MINW, false, true, false, plr::kPassFused, TL>}, \
     {nullptr, plr::shard_pass<NCH, R, 1, WROW, MINW, true, true, false, plr::kPassFused, TL>}}}
 
-// A row of C chunks (128 columns each) is handled by one wave up to C = 16,
-// then by ceil(C/8) chunks per wave on as many waves side by side as that
-// takes (<= 8), so at most one wave of the workgroup is partly idle.  A row
-// that ends up to 32-64 columns past a chunk boundary takes the variant with
-// that many full chunks and a tail stage.  Tile heights and register budgets
+// A row of C chunks (128 columns each) is handled by one wave up to C = 32
+// (one exact variant per C; the last chunk may be ragged), then by ceil(C/8)
+// chunks per wave on as many waves side by side as that takes (<= 8), so at
+// most one wave of the workgroup is partly idle.  Between 17 and 32 chunks
+// the several-waves variants are 1-2 % faster when the row fills them exactly
+// (18, 21, 24, 28, 32 whole chunks) and up to 10 % slower otherwise, so only
+// those widths take them.  A row of up to 16 chunks that ends 32-64 columns
+// past a chunk boundary takes the variant with that many full chunks and a
+// tail stage.  Tile heights and register budgets
 // (MINW = waves per SIMD the allocation leaves room for) come from sweeps on
 // MI355X: one or two resident waves per SIMD, each with 16-48 KiB of loads in
 // flight, stream fastest; any variant that spills registers loses a third of
@@ -71,6 +75,22 @@ const Variant kVariants[] = {
     PLR_ROW(14, 4, 4, 1, 0),
     PLR_ROW(15, 2, 4, 1, 0),
     PLR_ROW(16, 2, 4, 1, 0),
+    PLR_ROW(17, 1, 4, 1, 0),
+    PLR_ROW(18, 1, 4, 1, 0),
+    PLR_ROW(19, 1, 4, 1, 0),
+    PLR_ROW(20, 1, 4, 1, 0),
+    PLR_ROW(21, 1, 4, 1, 0),
+    PLR_ROW(22, 1, 4, 1, 0),
+    PLR_ROW(23, 1, 4, 1, 0),
+    PLR_ROW(24, 1, 4, 1, 0),
+    PLR_ROW(25, 1, 4, 1, 0),
+    PLR_ROW(26, 1, 4, 1, 0),
+    PLR_ROW(27, 1, 4, 1, 0),
+    PLR_ROW(28, 1, 4, 1, 0),
+    PLR_ROW(29, 1, 4, 1, 0),
+    PLR_ROW(30, 1, 4, 1, 0),
+    PLR_ROW(31, 1, 4, 1, 0),
+    PLR_ROW(32, 1, 4, 1, 0),
     // one wave per row with a tail stage (capacity 128*TL/R columns)
     PLR_ROW(1, 32, 4, 1, 2),   // 8
     PLR_ROW(1, 32, 4, 1, 4),   // 16
@@ -118,7 +138,8 @@ const Variant kVariants[] = {
     PLR_VARIANT(17, 1, 8, 1, 2, true),    // ..136
     PLR_VARIANT(19, 1, 8, 1, 2, true),    // ..152 (152 KiB of theta in LDS)
 };
-constexpr int kMaxRowChunks = 16;  // widest one-wave row
+constexpr int kMaxTailChunks = 16;  // widest row with a tail-stage variant
+constexpr int kMaxRowChunks = 32;   // widest one-wave row
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int64_t kMaxFusedCols = 19456;
 
@@ -336,7 +357,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   // a few columns past a chunk boundary: the tail-stage variant with the
   // smallest capacity that holds them
   const int64_t full = pitch / plr::kChunkCols, rem = pitch % plr::kChunkCols;
-  if (rem != 0 && full >= 1 && full <= kMaxRowChunks) {
+  if (rem != 0 && full >= 1 && full <= kMaxTailChunks) {
     int best_cap = 1 << 30;
     for (int i = 0; i < kNumVariants; ++i) {
       const Variant& k = kVariants[i];
@@ -351,16 +372,15 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   }
   if (!v) {
     // (waves, chunks per wave) for this width, then the variant that has them
-    int want_w, want_k;
-    if (chunks <= kMaxRowChunks) {
-      want_w = 1;
-      want_k = (int)chunks;
-    } else if (chunks <= 64) {
+    int want_w = 8, want_k = (int)ceil_div(chunks, 8);  // beyond 64 chunks: theta in LDS
+    if (chunks <= 64) {
       want_k = (int)ceil_div(chunks, 8);
       want_w = (int)ceil_div(chunks, want_k);
-    } else {
-      want_w = 8;
-      want_k = (int)ceil_div(chunks, 8);
+      const bool fills_waves = rem == 0 && chunks == (int64_t)want_k * want_w;
+      if (chunks <= kMaxRowChunks && !(chunks > kMaxTailChunks && fills_waves)) {
+        want_w = 1;
+        want_k = (int)chunks;
+      }
     }
     for (int i = 0; i < kNumVariants; ++i) {
       const Variant& k = kVariants[i];

@@ -98,6 +98,31 @@ def test_rows_just_past_a_chunk_boundary(plr, oracle, gen, k, t):
     assert rel(g2, X2.T @ (0.5 - y)) <= GRAD_TOL
 
 
+@pytest.mark.parametrize("chunks", list(range(17, 33)))
+def test_rows_of_17_to_32_chunks(plr, oracle, gen, chunks):
+    # one exact kernel variant per chunk count; the widths that fill a
+    # several-waves variant exactly (18, 21, 24, 28, 32 chunks) take that one
+    for d in (128 * chunks, 128 * chunks - 1, 128 * (chunks - 1) + 17):
+        for n in (1, 5, 517):
+            print("case n=%d d=%d" % (n, d), flush=True)
+            X, y, th = make(gen, n, d, seed=0xC0DE + d)
+            plr.set_data(X, y)
+            if n == 1:
+                print(plr.kernel_info(), flush=True)
+            g, loss, _ = plr.loss_grad(th)
+            assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
+            loss_ref = oracle.calc_loss_sum(X, y, th)
+            assert abs(loss - loss_ref) <= LOSS_TOL * abs(loss_ref)
+            l2, _ = plr.calc_loss(th)
+            assert abs(l2 - loss_ref) <= LOSS_TOL * abs(loss_ref)
+            assert np.max(np.abs(plr.predict(th) - oracle.predict(X, th))) <= 1e-14
+    X2 = X.copy()
+    X2[:, d - 1] += 1.0
+    plr.set_data(X2, y)
+    g2, _, _ = plr.loss_grad(np.zeros(d))
+    assert rel(g2, X2.T @ (0.5 - y)) <= GRAD_TOL
+
+
 @pytest.mark.parametrize("n,d", [(1000, 100), (2051, 1000), (333, 257), (70, 8193), (37, 16385)])
 def test_dgd_delta_matches_oracle(plr, oracle, gen, n, d):
     X, y, th = make(gen, n, d)
