@@ -57,6 +57,13 @@ struct Variant {
 // flight, stream fastest; any variant that spills registers loses a third of
 // the bandwidth or more.  From 65 chunks on theta lives in LDS and a variant
 // covers every per-wave count up to its NCH.
+// several waves side by side, exactly WCOL*NCH full chunks plus a tail stage
+// on the last wave (the 2^k + 1 widths of wide rows)
+#define PLR_VARIANT_TAIL(NCH, R, WCOL, MINW, THL, TL)                                            \
+  {NCH, R, WCOL, 1, THL, TL,                                                                     \
+   {{nullptr, plr::shard_pass<NCH, R, WCOL, 1, MINW, false, true, THL, plr::kPassFused, TL>},    \
+    {nullptr, plr::shard_pass<NCH, R, WCOL, 1, MINW, true, true, THL, plr::kPassFused, TL>}}}
+
 const Variant kVariants[] = {
     // one wave per row, exact chunk counts
     PLR_ROW(1, 16, 4, 2, 0),
@@ -116,6 +123,9 @@ const Variant kVariants[] = {
     PLR_ROW(14, 2, 4, 1, 1),   // 64
     PLR_ROW(15, 2, 4, 1, 1),   // 64
     PLR_ROW(16, 2, 4, 1, 1),   // 64
+    PLR_VARIANT_TAIL(4, 4, 8, 2, false, 1),   // 4096 + 32
+    PLR_VARIANT_TAIL(8, 2, 8, 2, true, 1),    // 8192 + 64
+    PLR_VARIANT_TAIL(16, 1, 8, 2, true, 1),   // 16384 + 128
     // 3 chunks per wave: 17..24
     PLR_VARIANT(3, 8, 6, 1, 2, false),
     PLR_VARIANT(3, 8, 7, 1, 2, false),
@@ -138,7 +148,7 @@ const Variant kVariants[] = {
     PLR_VARIANT(17, 1, 8, 1, 2, true),    // ..136
     PLR_VARIANT(19, 1, 8, 1, 2, true),    // ..152 (152 KiB of theta in LDS)
 };
-constexpr int kMaxTailChunks = 16;  // widest row with a tail-stage variant
+constexpr int kAlwaysOneWave = 16;  // up to here no several-waves variant is considered
 constexpr int kMaxRowChunks = 32;   // widest one-wave row
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int64_t kMaxFusedCols = 19456;
@@ -357,11 +367,11 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   // a few columns past a chunk boundary: the tail-stage variant with the
   // smallest capacity that holds them
   const int64_t full = pitch / plr::kChunkCols, rem = pitch % plr::kChunkCols;
-  if (rem != 0 && full >= 1 && full <= kMaxTailChunks) {
+  if (rem != 0 && full >= 1) {
     int best_cap = 1 << 30;
     for (int i = 0; i < kNumVariants; ++i) {
       const Variant& k = kVariants[i];
-      if (k.tl == 0 || k.nch != full) continue;
+      if (k.tl == 0 || (int64_t)k.nch * k.wcol != full) continue;
       const int cap = plr::kChunkCols * k.tl / k.R;
       if (cap >= rem && cap < best_cap) {
         v = &k;
@@ -377,7 +387,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
       want_k = (int)ceil_div(chunks, 8);
       want_w = (int)ceil_div(chunks, want_k);
       const bool fills_waves = rem == 0 && chunks == (int64_t)want_k * want_w;
-      if (chunks <= kMaxRowChunks && !(chunks > kMaxTailChunks && fills_waves)) {
+      if (chunks <= kMaxRowChunks && !(chunks > kAlwaysOneWave && fills_waves)) {
         want_w = 1;
         want_k = (int)chunks;
       }
@@ -401,7 +411,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   if (tail) {
     c->nch_rt = v->nch;
     c->allch = true;
-    c->theta_len = (int64_t)(v->nch + 1) * plr::kChunkCols;
+    c->theta_len = (full + 1) * plr::kChunkCols;
   } else {
     c->nch_rt = (int)ceil_div(chunks, v->wcol);  // == v->nch except for the theta-in-LDS variants
     c->allch = (chunks == (int64_t)v->nch * v->wcol);

@@ -208,7 +208,8 @@ struct WaveCtx {
   int my_row;         // row of the tile whose dot product ends up in this lane
   uint32_t lane_off;  // byte offset of this lane inside a chunk
   // tail stage (TL > 0): this lane's place among the leftover columns
-  bool tail_in;       // the lane's column pair exists
+  bool owns_tail;     // this wave handles them (the last one of the workgroup's row)
+  bool tail_in;       // ... and the lane's column pair exists
   int tail_row;       // row, within one tail load, that the lane reads
   int tail_slot;      // lane holding the tail dot of row my_row
   uint32_t tail_off;  // byte offset of the lane's pair from the tile base
@@ -305,6 +306,17 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
           s1[r] = fma(x[r][c].y, t.y, s1[r]);
         }
       }
+      // one tail load per row (TL == R): all 64 lanes of load r belong to row
+      // r, so the leftover columns are simply one more term of the partial
+      if constexpr (TL > 0 && TL == R) {
+        if (w.owns_tail) {  // uniform
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            s0[r] = fma(xt[r].x, tht.x, s0[r]);
+            s1[r] = fma(xt[r].y, tht.y, s1[r]);
+          }
+        }
+      }
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if constexpr (R == 1)
@@ -315,7 +327,7 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
     }
     double z = reduce_rows<R>(p, lane);
 
-    if constexpr (TL > 0) {
+    if (TL > 0 && TL < R && w.owns_tail) {  // uniform
       // leftover columns: segment sums, then each row's sum to the lane that
       // holds the row
       constexpr int kRpl = TailGeo<R, TL>::kRowsPerLoad;
@@ -366,8 +378,14 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
         acc[c].x = fma(rr, x[r][c].x, acc[c].x);
         acc[c].y = fma(rr, x[r][c].y, acc[c].y);
       }
+      if constexpr (TL > 0 && TL == R) {
+        if (w.owns_tail) {  // uniform
+          acct.x = fma(rr, xt[r].x, acct.x);
+          acct.y = fma(rr, xt[r].y, acct.y);
+        }
+      }
     }
-    if constexpr (TL > 0) {
+    if (TL > 0 && TL < R && w.owns_tail) {  // uniform
 #pragma unroll
       for (int j = 0; j < TL; ++j) {
         const double rr = __shfl(res, w.tail_src[j], kWave);
@@ -396,16 +414,16 @@ template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD, bool ALLCH, b
 __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a) {
   static_assert(WCOL == 1 || WROW == 1, "column-split workgroups own one row group");
   static_assert((R & (R - 1)) == 0 && R <= kWave, "R must be a power of two");
-  static_assert(TL == 0 || (WCOL == 1 && ALLCH && !THL && MODE == kPassFused && TL <= R &&
-                            TL <= 4 && (TL & (TL - 1)) == 0),
-                "the tail stage goes with one-wave rows of exactly NCH full chunks");
+  static_assert(TL == 0 || (ALLCH && MODE == kPassFused && TL <= R && TL <= 4 &&
+                            (TL & (TL - 1)) == 0),
+                "the tail stage goes with rows of exactly WCOL*NCH full chunks");
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform
   const int wc = (WCOL > 1) ? wave : 0;
   const int wr = (WCOL > 1) ? 0 : wave;
 
-  // with a tail stage the chunks are the NCH full ones
-  const int64_t chunks = (TL > 0) ? NCH : (a.width + kChunkCols - 1) / kChunkCols;
+  // with a tail stage the chunks are the WCOL*NCH full ones
+  const int64_t chunks = (TL > 0) ? NCH * WCOL : (a.width + kChunkCols - 1) / kChunkCols;
   const int64_t slab_c0 = (int64_t)wc * a.nch_rt;          // first chunk of this wave
   int64_t left = chunks - slab_c0;
   const int my_nch = ALLCH ? NCH : (int)(left < 0 ? 0 : (left > a.nch_rt ? a.nch_rt : left));
@@ -429,15 +447,17 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
   constexpr int64_t kBodyCols = (int64_t)NCH * kChunkCols;
   const int tail_pair = lane & (kLpr - 1);
   v2d tht = v2d{0., 0.}, acct = v2d{0., 0.};
+  w.owns_tail = TL > 0 && wc == WCOL - 1;  // the wave next to the leftover columns
   if constexpr (TL > 0) {
-    w.tail_in = 2 * tail_pair < a.tail_cols;
+    w.tail_in = w.owns_tail && 2 * tail_pair < a.tail_cols;
     w.tail_row = lane / kLpr;
     w.tail_slot = (w.my_row % kRpl) * kLpr;
     w.tail_off = (uint32_t)(((int64_t)w.tail_row * a.pitch + kBodyCols + 2 * tail_pair) *
                             sizeof(double));
 #pragma unroll
     for (int j = 0; j < TL; ++j) w.tail_src[j] = lane_of_row<R>(j * kRpl + w.tail_row);
-    if (w.tail_in) tht = *reinterpret_cast<const v2d*>(a.theta + kBodyCols + 2 * tail_pair);
+    if (w.tail_in)
+      tht = *reinterpret_cast<const v2d*>(a.theta + slab_col0 + kBodyCols + 2 * tail_pair);
   }
 
   // theta slab -> registers, or -> this wave's private LDS slab (theta is
@@ -524,7 +544,7 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
         acct.x += __shfl_xor(acct.x, m, kWave);
         acct.y += __shfl_xor(acct.y, m, kWave);
       }
-      emit(acct, lane < kLpr && w.tail_in, out + kBodyCols + 2 * tail_pair);
+      emit(acct, lane < kLpr && w.tail_in, out + slab_col0 + kBodyCols + 2 * tail_pair);
     }
   }
   if constexpr (MODE == kPassFused) {  // the sweeps of a blocked row carry no loss

@@ -66,7 +66,8 @@ TAIL_CASES = [(k, t) for k in (1, 2) for t in (1, 2, 7, 8, 9, 16, 17, 31, 32, 33
              [(k, t) for k in (3, 4) for t in (1, 15, 16, 17, 32)] + \
              [(k, t) for k in (6, 7, 9, 10, 11) for t in (1, 32)] + \
              [(8, t) for t in (1, 31, 32, 33, 64)] + \
-             [(k, t) for k in (12, 13, 14, 15, 16) for t in (1, 64)]
+             [(k, t) for k in (12, 13, 14, 15, 16) for t in (1, 64)] + \
+             [(32, 1), (32, 32), (64, 1), (64, 17), (64, 64), (128, 1), (128, 100)]
 
 
 @pytest.mark.parametrize("k,t", TAIL_CASES)
@@ -74,12 +75,14 @@ def test_rows_just_past_a_chunk_boundary(plr, oracle, gen, k, t):
     d = 128 * k + t
     for n in (1, 3, 77, 1543):
         print("case n=%d d=%d" % (n, d), flush=True)
+        if d > 4096 and n > 100:
+            n = 131
         X, y, th = make(gen, n, d, seed=0x7A11 + d)
         plr.set_data(X, y)
         if n == 1:
             print(plr.kernel_info(), flush=True)
-            if d < 2048:
-                assert "tail=%d" % (t + (t & 1)) in plr.kernel_info()
+            pitch = d + (d & 1) if d < 2048 else (d + 15) // 16 * 16
+            assert "tail=%d " % (pitch - 128 * k) in plr.kernel_info()
         g, loss, n_out = plr.loss_grad(th)
         assert n_out == n
         assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
