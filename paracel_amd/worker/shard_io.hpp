@@ -128,13 +128,73 @@ struct ParsedShard {
   std::vector<double> X, y;      // X: n x d row-major
 };
 
+// std::stod's value for one field, without the library call for the common
+// spelling: [-]digits[.digits][e[+-]digits] with at most 15 significant
+// digits and a decimal exponent within +-22.  Then the digits are an exact
+// double, 10^|e| is an exact double, and the one multiplication or division
+// rounds once -- the correctly rounded result, which is what strtod returns
+// (Clinger's fast path).  Every other spelling (more digits, hex floats, inf,
+// nan, leading blanks or '+', trailing garbage) and every error goes through
+// std::stod itself, so the exceptions are the reference's too.
+inline double parse_field(const char* p, size_t len) {
+  static const double kPow10[23] = {1e0,  1e1,  1e2,  1e3,  1e4,  1e5,  1e6,  1e7,
+                                    1e8,  1e9,  1e10, 1e11, 1e12, 1e13, 1e14, 1e15,
+                                    1e16, 1e17, 1e18, 1e19, 1e20, 1e21, 1e22};
+  const char* q = p;
+  const char* const end = p + len;
+  bool neg = false;
+  if (q < end && *q == '-') {
+    neg = true;
+    ++q;
+  }
+  uint64_t m = 0;
+  int sig = 0, ndig = 0, frac = 0;
+  for (; q < end && *q >= '0' && *q <= '9'; ++q, ++ndig) {
+    m = m * 10 + (uint64_t)(*q - '0');
+    if (m) ++sig;
+    if (sig > 15) goto slow;
+  }
+  if (q < end && *q == '.') {
+    ++q;
+    for (; q < end && *q >= '0' && *q <= '9'; ++q, ++ndig, ++frac) {
+      m = m * 10 + (uint64_t)(*q - '0');
+      if (m) ++sig;
+      if (sig > 15) goto slow;
+    }
+  }
+  if (ndig == 0) goto slow;
+  {
+    int e10 = 0;
+    if (q < end && (*q == 'e' || *q == 'E')) {
+      ++q;
+      bool eneg = false;
+      if (q < end && (*q == '+' || *q == '-')) eneg = (*q++ == '-');
+      int ed = 0;
+      for (; q < end && *q >= '0' && *q <= '9'; ++q, ++ed) {
+        e10 = e10 * 10 + (*q - '0');
+        if (e10 > 9999) goto slow;
+      }
+      if (ed == 0) goto slow;
+      if (eneg) e10 = -e10;
+    }
+    if (q != end) goto slow;
+    e10 -= frac;
+    if (e10 < -22 || e10 > 22) goto slow;
+    double v = (double)m;
+    v = (e10 < 0) ? v / kPow10[-e10] : v * kPow10[e10];
+    return neg ? -v : v;
+  }
+slow:
+  return std::stod(std::string(p, len));  // throws like the reference
+}
+
 inline void parse_one_line(const std::string& line, char sep, std::vector<double>& fields) {
   fields.clear();
   size_t st = 0;
   for (;;) {
     const size_t en = line.find(sep, st);
     const size_t len = (en == std::string::npos ? line.size() : en) - st;
-    if (len) fields.push_back(std::stod(line.substr(st, len)));  // throws like the reference
+    if (len) fields.push_back(parse_field(line.data() + st, len));
     if (en == std::string::npos) break;
     st = en + 1;
   }

@@ -2,11 +2,71 @@
 //   plr_shard_tool parse <input.csv> <rank> <np>   parse this rank's lines and write the cache
 //   plr_shard_tool info  <input.csv> <rank> <np>   validate the cache; print n d
 //   plr_shard_tool lines <input.csv> <rank> <np>   print the lines this rank owns
+//   plr_shard_tool selftest <count> <seed> 0       parse_field against std::stod on <count>
+//                                                  random field spellings, bit for bit
 #include <iostream>
+#include <random>
 
 #include "shard_io.hpp"
 
+// A random field: mostly decimal spellings around the limits of the fast path
+// (digit counts 1..20, exponents around +-22, zeros, signs), some spellings
+// only std::stod understands, some it rejects.
+static std::string random_field(std::mt19937_64& rng) {
+  auto pick = [&](int n) { return (int)(rng() % (uint64_t)n); };
+  static const char* odd[] = {"inf", "-inf", "nan", "0x1.8p3", " 1.5", "+2.5", "1.5abc", "abc",
+                              "-", ".", "e5", "1e", "1e+", "1e400", "1e-400", "4.9e-324", "-0",
+                              "0.0", "-0.0e7", "00012.500", "1.", ".5", "-.5e-3", "1E5", "2.5E-7"};
+  if (pick(16) == 0) return odd[pick((int)(sizeof odd / sizeof *odd))];
+  std::string s;
+  if (pick(2)) s += '-';
+  const int ni = pick(12), nf = pick(12);
+  for (int i = 0; i < ni; ++i) s += (char)('0' + (pick(4) == 0 ? 0 : pick(10)));
+  if (nf || pick(3) == 0) {
+    s += '.';
+    for (int i = 0; i < nf; ++i) s += (char)('0' + (pick(4) == 0 ? 0 : pick(10)));
+  }
+  if (pick(2)) {
+    s += pick(2) ? 'e' : 'E';
+    const int k = pick(3);
+    if (k == 0) s += '-';
+    if (k == 1) s += '+';
+    s += std::to_string(pick(3) == 0 ? pick(400) : pick(30));
+  }
+  return s;
+}
+
+static int selftest(long count, unsigned long long seed) {
+  std::mt19937_64 rng(seed);
+  long fast_or_equal = 0, threw = 0;
+  for (long i = 0; i < count; ++i) {
+    const std::string f = random_field(rng);
+    double want = 0., got = 0.;
+    bool want_throw = false, got_throw = false;
+    try {
+      want = std::stod(f);
+    } catch (const std::exception&) {
+      want_throw = true;
+    }
+    try {
+      got = plr_ps::parse_field(f.data(), f.size());
+    } catch (const std::exception&) {
+      got_throw = true;
+    }
+    if (want_throw != got_throw || (!want_throw && memcmp(&want, &got, sizeof want) != 0)) {
+      std::cout << "MISMATCH '" << f << "'\n";
+      return 1;
+    }
+    threw += want_throw;
+    ++fast_or_equal;
+  }
+  std::cout << "ok " << fast_or_equal << " fields, " << threw << " rejected by both\n";
+  return 0;
+}
+
 int main(int argc, char** argv) {
+  if (argc == 5 && std::string(argv[1]) == "selftest")
+    return selftest(atol(argv[2]), strtoull(argv[3], nullptr, 0));
   if (argc != 5) {
     std::cerr << "usage: plr_shard_tool parse|info|lines <input> <rank> <np>\n";
     return 2;

@@ -121,3 +121,31 @@ def test_parser_errors(tmp_path):
     f.write_text("3,,7,1\n")                            # empty field dropped (str_split)
     assert run("parse", f, 0, 1).stdout.split() == ["1", "3"]
     assert run("parse", tmp_path / "missing.csv", 0, 1).returncode == 1
+
+
+def test_field_parser_equals_stod_bit_for_bit():
+    # the short-decimal fast path against std::stod itself on random spellings:
+    # digit counts around 15, exponents around +-22, zeros, signs, hex floats,
+    # inf/nan, blanks, garbage -- values and exceptions must agree
+    for seed in (1, 0xBEEF):
+        out = run("selftest", 1500000, seed, 0)
+        assert out.returncode == 0, out.stdout + out.stderr
+        assert out.stdout.startswith("ok 1500000 fields")
+
+
+def test_parser_against_python_float(tmp_path):
+    # python's float() is correctly rounded, like strtod: fields written with few
+    # digits (fast path) and with 17 (library path) in one file
+    rng = np.random.default_rng(11)
+    vals = rng.normal(size=(200, 6)) * 10.0 ** rng.integers(-30, 30, size=(200, 6))
+    lines = []
+    for i, row in enumerate(vals):
+        fmt = ["%.3f", "%.17g", "%.14e", "%r"][i % 4]
+        lines.append(",".join((fmt % v) if fmt != "%r" else repr(float(v)) for v in row) + ",1")
+    f = tmp_path / "p.csv"
+    f.write_text("\n".join(lines) + "\n")
+    assert run("parse", f, 0, 1).returncode == 0
+    raw = np.fromfile(str(f) + ".plrshard.0of1", dtype=np.uint8)
+    X = np.frombuffer(raw[48:48 + 8 * 200 * 7].tobytes(), dtype=np.float64).reshape(200, 7)
+    want = np.array([[float(t) for t in l.split(",")[:-1]] for l in lines])
+    assert X[:, 1:].tobytes() == want.tobytes()
