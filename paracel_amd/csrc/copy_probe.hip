@@ -1,6 +1,9 @@
 // Counter calibration for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: launches a
 // plain copy kernel that reads exactly N bytes and writes exactly N bytes, so
 // that what the counters report for it fixes their scale on this device.
+// It then times the runtime's own device-to-device copy of the same buffers
+// (hipMemcpyAsync, 5 repetitions after a warm-up): the copy ceiling that the
+// streaming pass's read rate is quoted next to.
 //   usage: copy_probe [MiB = 1024] [launches = 3]
 #include <hip/hip_runtime.h>
 #include <stdio.h>
@@ -50,6 +53,18 @@ int main(int argc, char** argv) {
   printf("plain_copy: %d launches, each reads %zu bytes and writes %zu bytes; %.3f ms avg, "
          "%.1f GB/s read+write\n", launches, bytes, bytes, total / launches,
          2.0 * bytes / (total / launches) * 1e-6);
+  const int reps = 5;
+  CK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, 0));
+  CK(hipDeviceSynchronize());
+  CK(hipEventRecord(e0, 0));
+  for (int i = 0; i < reps; ++i) CK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, 0));
+  CK(hipEventRecord(e1, 0));
+  CK(hipDeviceSynchronize());
+  float ms = 0.f;
+  CK(hipEventElapsedTime(&ms, e0, e1));
+  printf("hipMemcpy device-to-device: %d copies of %zu bytes; %.3f ms avg, %.1f GB/s read+write "
+         "(%.1f GB/s each way)\n", reps, bytes, ms / reps, 2.0 * bytes / (ms / reps) * 1e-6,
+         1.0 * bytes / (ms / reps) * 1e-6);
   CK(hipFree(src));
   CK(hipFree(dst));
   return 0;
