@@ -32,12 +32,12 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # known size; None until measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
     # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000) KiB per shard_pass dispatch; see profiles/
-    "c2_headline_1m_x_1000": 8055607504,
-    "c3_tall_10m_x_256": 20560472309,
-    "c4_wide_200k_x_16384": 26261494739,
-    "c4b_wide_200k_x_16385": 26466443874,
-    "c5_e2e_2m_x_512": 8210210591,
-    "x_bias_10m_x_257": 21202464437,
+    "c2_headline_1m_x_1000": 8056281406,
+    "c3_tall_10m_x_256": 20560480416,
+    "c4_wide_200k_x_16384": 26261496415,
+    "c4b_wide_200k_x_16385": 26287132305,
+    "c5_e2e_2m_x_512": 8210208784,
+    "x_bias_10m_x_257": 21175219596,
 }
 
 
