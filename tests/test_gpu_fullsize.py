@@ -43,7 +43,7 @@ def stream_and_reference(plr, cfg, theta, slab_rows=0):
 
 
 FULL = ["c2_headline_1m_x_1000", "c3_tall_10m_x_256", "c4_wide_200k_x_16384",
-        "c4b_wide_200k_x_16385", "c5_e2e_2m_x_512"]
+        "c4b_wide_200k_x_16385", "c5_e2e_2m_x_512", "x_bias_10m_x_257"]
 
 
 @pytest.mark.parametrize("name", FULL)
@@ -78,3 +78,38 @@ def test_full_size_shard(plr, oracle, gen, name):
     assert rel(gs, oracle.gsum(Xs, ys, theta)) <= 1e-10
     want = oracle.calc_loss_sum(Xs, ys, theta)
     assert abs(ls - want) <= 1e-9 * want
+
+
+def test_shard_of_160_gb_repeats_a_block(plr):
+    # more than half of the 288 GB of HBM in one shard (byte offsets past 2^37): the same
+    # 250 000-row block uploaded 80 times plus a ragged remainder, so additivity gives the
+    # answer from the block alone
+    from paracel_amd import Plr, PlrError
+
+    n, d, rows = 20_000_123, 1000, 250_000
+    rng = np.random.default_rng(5)
+    blk = rng.normal(size=(rows, d)) / np.sqrt(d)
+    yb = (rng.random(rows) < 0.5) * 1.0
+    th = rng.normal(size=d)
+    print("case n=%d d=%d (%.0f GB)" % (n, d, 8e-9 * n * d), flush=True)
+    try:
+        plr.alloc_data(n, d)
+    except PlrError as e:
+        if e.code == -3:
+            pytest.skip("device memory does not hold a 160 GB shard")
+        raise
+    for r0 in range(0, n, rows):
+        m = min(rows, n - r0)
+        plr.set_data_chunk(r0, blk[:m], yb[:m])
+    g, loss, n_out = plr.loss_grad(th)
+    assert n_out == n
+    with Plr(0) as one:
+        one.set_data(blk, yb)
+        gb, lb, _ = one.loss_grad(th)
+        rem = n % rows
+        one.set_data(blk[:rem], yb[:rem])
+        gr, lr, _ = one.loss_grad(th)
+    want = gb * (n // rows) + gr
+    assert rel(g, want) <= 1e-12
+    assert abs(loss - (lb * (n // rows) + lr)) <= 1e-12 * loss
+    plr.set_data(blk[:8], yb[:8])   # release the 160 GB before the next test
