@@ -467,6 +467,27 @@ def test_device_resident_training_matches_oracle_and_per_round_path(plr, oracle,
     np.testing.assert_array_equal(plr.train_dgd(np.zeros(cfg.d), alpha, beta, 100), theta)
 
 
+@pytest.mark.parametrize("n,d", [(3000, 16), (2000, 257), (1500, 1025), (500, 2500), (300, 4097),
+                                 (200, 16385), (120, 20001)])
+def test_device_resident_training_in_every_kernel_family(plr, oracle, gen, n, d):
+    # packed rows, tail stage, one wave per row, several waves + tail, column blocks:
+    # device-resident rounds give the bits of the host-driven loop, and the oracle's theta
+    X, y, _ = make(gen, n, d, seed=0x7EA + d)
+    alpha, beta = 0.1 / n, 0.005
+    plr.set_data(X, y)
+    print(plr.kernel_info(), flush=True)
+    theta, curve = plr.train_dgd(np.zeros(d), alpha, beta, 6, want_curve=True)
+    th = np.zeros(d)
+    losses = []
+    for _ in range(6):
+        delta, l = plr.dgd_delta(th, alpha, beta)
+        losses.append(l)
+        th = th + delta
+    np.testing.assert_array_equal(theta, th)
+    np.testing.assert_array_equal(curve, np.array(losses))
+    assert rel(theta, oracle.train_dgd(X, y, np.zeros(d), alpha, beta, 6)) <= 1e-8
+
+
 def _random_shapes(count, seed):
     rng = np.random.default_rng(seed)
     out = []
