@@ -17,7 +17,7 @@
 //     row's partial, log2(64/R) plain butterfly steps finish it.  So the
 //     exp/log of a row is evaluated once per tile by the lane that holds
 //     it, not 64 times, and R-1+log2(64/R) lane exchanges replace 6R.
-//   * Rows of more than 16 chunks: WCOL waves of a workgroup split the
+//   * Wide rows (more than 32 chunks): WCOL waves of a workgroup split the
 //     columns; their partial dots meet in LDS (double-buffered, one barrier
 //     per tile) and are summed in wave order.
 //   * A row that ends a few columns past a chunk boundary (the file path
@@ -25,7 +25,8 @@
 //     not get a nearly empty chunk of its own: the TL > 0 variants cover the
 //     leftover columns of ALL rows of a tile with TL loads, 64*TL/R lanes per
 //     row, reduce them inside those lane segments and fold them into the
-//     row's dot product and the gradient separately.
+//     row's dot product and the gradient separately (on the last wave of the
+//     row when several waves share it).
 //   * Rows are spread over the grid tile-interleaved (tile t goes to row
 //     group t mod G), so at any moment the grid streams one contiguous window
 //     of X.
@@ -408,7 +409,7 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
 //        wide rows, where theta + accumulators + tile would not fit
 // MODE : kPassFused, or one of the two sweeps of a column-blocked row
 // TL   : 0, or the number of loads per tile that cover the columns past the
-//        NCH full chunks (a.tail_cols of them, at most 128*TL/R)
+//        WCOL*NCH full chunks (a.tail_cols of them, at most 128*TL/R)
 template <int NCH, int R, int WCOL, int WROW, int MINW, bool GRAD, bool ALLCH, bool THL,
           int MODE = kPassFused, int TL = 0>
 __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a) {
