@@ -372,6 +372,32 @@ def test_labels_other_than_one_are_class_zero(plr, oracle, gen):
     assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
 
 
+def test_non_finite_inputs_propagate_like_the_reference(plr, oracle, gen):
+    # the reference does no input checking: a NaN or an infinity in a sample poisons
+    # exactly the entries IEEE arithmetic says it should, on the device as on the host
+    X, y, th = make(gen, 200, 300)
+    for kind, val in (("nan", np.nan), ("inf", np.inf), ("-inf", -np.inf)):
+        Xb = X.copy()
+        Xb[17, 5] = val
+        plr.set_data(Xb, y)
+        g, loss, _ = plr.loss_grad(th)
+        g_ref = oracle.gsum(Xb, y, th)
+        with np.errstate(invalid="ignore", over="ignore", divide="ignore"):
+            loss_ref = oracle.calc_loss_sum(Xb, y, th)
+        np.testing.assert_array_equal(np.isnan(g), np.isnan(g_ref), err_msg=kind)
+        np.testing.assert_array_equal(np.isinf(g), np.isinf(g_ref), err_msg=kind)
+        ok = np.isfinite(g_ref)
+        assert rel(g[ok], g_ref[ok]) <= GRAD_TOL
+        assert (np.isnan(loss) and np.isnan(loss_ref)) or loss == loss_ref or \
+            abs(loss - loss_ref) <= 1e-9 * abs(loss_ref)
+    # a NaN label poisons every column its row touches
+    yb = y.copy()
+    yb[3] = np.nan
+    plr.set_data(X, yb)
+    g, _, _ = plr.loss_grad(th)
+    np.testing.assert_array_equal(np.isnan(g), np.isnan(oracle.gsum(X, yb, th)))
+
+
 def test_empty_shard(plr):
     plr.set_data(np.zeros((0, 10)), np.zeros(0))
     g, loss, n = plr.loss_grad(np.ones(10))
