@@ -33,6 +33,7 @@ SYMBOLS = [
     ("plr_predict", C.c_int, [_ctx, _dp, _dp]),
     ("plr_predict_linear", C.c_int, [_ctx, _dp, _dp]),
     ("plr_synchronize", C.c_int, [_ctx]),
+    ("plr_set_timing", C.c_int, [_ctx, C.c_int]),
     ("plr_get_shape", C.c_int, [_ctx, _i64p, _i64p]),
     ("plr_get_timing", C.c_int, [_ctx, _dp, _dp, _i64p]),
     ("plr_reset_timing", C.c_int, [_ctx]),
@@ -204,6 +205,10 @@ class Plr:
 
     def reset_timing(self):
         self._check(self._lib.plr_reset_timing(self._h))
+
+    def set_timing(self, enabled):
+        """Timing events on (default) or off (saves 6-8 us per call)."""
+        self._check(self._lib.plr_set_timing(self._h, 1 if enabled else 0))
 
     def probe_read_bandwidth(self, reps=10):
         """GB/s a pure streaming read of the resident shard sustains."""

@@ -231,6 +231,7 @@ struct plr_ctx {
 
   double last_ms = 0., sum_ms = 0.;
   int64_t launches = 0;
+  bool timing = true;           // record the two events around the streaming kernels
 
   std::string err;
   std::string info;
@@ -596,7 +597,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   pa.z_accumulate = 0;
   pa.res_in = nullptr;
 
-  PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
+  if (c->timing) PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
   if (c->packed) {
     hipLaunchKernelGGL(c->packed->fn[grad ? 1 : 0], dim3(grid), dim3(threads), 0, c->stream, pa);
     PLR_HIP(c, hipGetLastError());
@@ -649,7 +650,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
       PLR_HIP(c, hipMemsetAsync(c->d_part_g, 0, (size_t)grid * c->pitch * sizeof(double),
                                 c->stream));
   }
-  PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
+  if (c->timing) PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
 
   if (!predict) {
     FinishArgs fa;
@@ -687,6 +688,7 @@ int stage_theta_from_host(plr_ctx* c, const double* theta) {
 }
 
 int account_timing(plr_ctx* c) {
+  if (!c->timing) return PLR_OK;
   float ms = 0.f;
   PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
   c->last_ms = ms;
@@ -922,6 +924,12 @@ int plr_get_timing(const plr_ctx* c, double* last_ms, double* sum_ms, int64_t* l
   if (last_ms) *last_ms = c->last_ms;
   if (sum_ms) *sum_ms = c->sum_ms;
   if (launches) *launches = c->launches;
+  return PLR_OK;
+}
+
+int plr_set_timing(plr_ctx* c, int enabled) {
+  if (!c) return PLR_ERR_INVALID;
+  c->timing = enabled != 0;
   return PLR_OK;
 }
 

@@ -398,6 +398,23 @@ def test_non_finite_inputs_propagate_like_the_reference(plr, oracle, gen):
     np.testing.assert_array_equal(np.isnan(g), np.isnan(oracle.gsum(X, yb, th)))
 
 
+def test_timing_switch(plr, gen):
+    X, y, th = make(gen, 500, 130)
+    plr.set_data(X, y)
+    plr.reset_timing()
+    g1, l1, _ = plr.loss_grad(th)
+    assert plr.timing()[2] == 1 and plr.timing()[0] > 0
+    plr.set_timing(False)
+    g2, l2, _ = plr.loss_grad(th)
+    d2, _ = plr.dgd_delta(th, 1e-3, 1e-2)
+    assert plr.timing()[2] == 1               # nothing recorded while off
+    np.testing.assert_array_equal(g1, g2)
+    assert l1 == l2
+    plr.set_timing(True)
+    plr.loss_grad(th)
+    assert plr.timing()[2] == 2
+
+
 def test_empty_shard(plr):
     plr.set_data(np.zeros((0, 10)), np.zeros(0))
     g, loss, n = plr.loss_grad(np.ones(10))
