@@ -331,6 +331,7 @@ def main():
     kern_ms = kern_ms_sum / launches
 
     read_ceiling = ctx.probe_read_bandwidth(10)
+    copy_ceiling = ctx.probe_copy_bandwidth(2 << 30, 5)   # read + written, runtime D2D copy
     bytes_step = cfg.algorithmic_bytes()
     achieved = bytes_step / (kern_ms * 1e-3) / 1e9
     traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name)
@@ -357,7 +358,8 @@ def main():
                      "kernel_ms": kern_ms, "algorithmic_bytes": bytes_step,
                      "whole_step_gbs": bytes_step / (elapsed / a.steps) / 1e9,
                      "read_ceiling_gbs": read_ceiling,
-                     "frac_of_read_ceiling": achieved / read_ceiling},
+                     "frac_of_read_ceiling": achieved / read_ceiling,
+                     "copy_ceiling_gbs": copy_ceiling},
         "cpu_baseline": None,
         "loss_mean": loss / n,
     }

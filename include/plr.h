@@ -138,6 +138,13 @@ int plr_set_timing(plr_ctx* ctx, int enabled);
  * sustains. */
 int plr_probe_read_bandwidth(plr_ctx* ctx, int reps, double* gb_per_s);
 
+/* Copy ceiling of this device: the runtime's device-to-device copy of `bytes`
+ * bytes between two temporary buffers (allocated and freed inside the call),
+ * `reps` times after one warm-up; reports GB/s of bytes read plus bytes
+ * written.  No counterpart in the reference; benchmarks quote it next to the
+ * read ceiling. */
+int plr_probe_copy_bandwidth(plr_ctx* ctx, int64_t bytes, int reps, double* gb_per_s);
+
 /* Human-readable description of the kernel variant chosen for the resident
  * shape (tile shape, grid), for logs.  Context-owned, never freed. */
 const char* plr_kernel_info(const plr_ctx* ctx);

@@ -34,6 +34,7 @@ SYMBOLS = [
     ("plr_predict_linear", C.c_int, [_ctx, _dp, _dp]),
     ("plr_synchronize", C.c_int, [_ctx]),
     ("plr_set_timing", C.c_int, [_ctx, C.c_int]),
+    ("plr_probe_copy_bandwidth", C.c_int, [_ctx, C.c_int64, C.c_int, C.POINTER(C.c_double)]),
     ("plr_get_shape", C.c_int, [_ctx, _i64p, _i64p]),
     ("plr_get_timing", C.c_int, [_ctx, _dp, _dp, _i64p]),
     ("plr_reset_timing", C.c_int, [_ctx]),
@@ -209,6 +210,12 @@ class Plr:
     def set_timing(self, enabled):
         """Timing events on (default) or off (saves 6-8 us per call)."""
         self._check(self._lib.plr_set_timing(self._h, 1 if enabled else 0))
+
+    def probe_copy_bandwidth(self, nbytes=1 << 30, reps=5):
+        """GB/s (read + written) of the runtime's device-to-device copy of nbytes."""
+        gbs = C.c_double()
+        self._check(self._lib.plr_probe_copy_bandwidth(self._h, nbytes, reps, C.byref(gbs)))
+        return gbs.value
 
     def probe_read_bandwidth(self, reps=10):
         """GB/s a pure streaming read of the resident shard sustains."""

@@ -904,6 +904,34 @@ int plr_probe_read_bandwidth(plr_ctx* c, int reps, double* gb_per_s) {
   return PLR_OK;
 }
 
+int plr_probe_copy_bandwidth(plr_ctx* c, int64_t bytes, int reps, double* gb_per_s) {
+  if (!c) return PLR_ERR_INVALID;
+  if (!gb_per_s || reps < 1 || bytes < 1)
+    return fail(c, PLR_ERR_INVALID, "need bytes >= 1, reps >= 1 and an output");
+  PLR_HIP(c, hipSetDevice(c->device));
+  void *src = nullptr, *dst = nullptr;
+  hipError_t e = hipMalloc(&src, (size_t)bytes);
+  if (e == hipSuccess) e = hipMalloc(&dst, (size_t)bytes);
+  if (e == hipSuccess) e = hipMemsetAsync(src, 1, (size_t)bytes, c->stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyDeviceToDevice, c->stream);
+  if (e == hipSuccess) e = hipEventRecord(c->ev0, c->stream);
+  for (int i = 0; i < reps && e == hipSuccess; ++i)
+    e = hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyDeviceToDevice, c->stream);
+  if (e == hipSuccess) e = hipEventRecord(c->ev1, c->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+  float ms = 0.f;
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, c->ev0, c->ev1);
+  if (src) (void)hipFree(src);
+  if (dst) (void)hipFree(dst);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(c, e == hipErrorOutOfMemory ? PLR_ERR_NOMEM : PLR_ERR_HIP,
+                std::string("copy probe failed: ") + hipGetErrorString(e));
+  }
+  *gb_per_s = 2.0 * (double)bytes * reps / (ms * 1e-3) / 1e9;
+  return PLR_OK;
+}
+
 int plr_synchronize(plr_ctx* c) {
   if (!c) return PLR_ERR_INVALID;
   PLR_HIP(c, hipSetDevice(c->device));

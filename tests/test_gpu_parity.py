@@ -415,6 +415,13 @@ def test_timing_switch(plr, gen):
     assert plr.timing()[2] == 2
 
 
+def test_bandwidth_probes(plr, gen):
+    X, y, _ = make(gen, 4096, 512)
+    plr.set_data(X, y)
+    assert plr.probe_read_bandwidth(2) > 100.0       # GB/s; a 16 MB shard sits in cache
+    assert plr.probe_copy_bandwidth(64 << 20, 2) > 100.0
+
+
 def test_empty_shard(plr):
     plr.set_data(np.zeros((0, 10)), np.zeros(0))
     g, loss, n = plr.loss_grad(np.ones(10))
