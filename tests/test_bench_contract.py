@@ -1,0 +1,59 @@
+"""bench.py's command-line contract: what can be checked without a GPU, and
+(marked gpu) that the default-shaped run prints one JSON line with the fields
+the harness reads."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BENCH = os.path.join(ROOT, "bench.py")
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, BENCH, "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_unknown_workload_is_refused():
+    r = subprocess.run([sys.executable, BENCH, "--workload", "nope"], capture_output=True, text=True)
+    assert r.returncode != 0 and "unknown workload" in r.stderr
+
+
+def test_parameter_server_round_trip_mode_runs_on_the_host():
+    r = subprocess.run([sys.executable, BENCH, "--ps-roundtrip"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["metric"] == "ps_round_trip_us"
+    for d in ("100", "512", "1001", "16385"):
+        for mode in ("dense", "packed"):
+            assert out["widths"][d][mode]["read_us"] > 0
+            assert out["widths"][d][mode]["bupdate_us"] > 0
+
+
+@pytest.mark.gpu
+def test_one_json_line_with_roofline_and_cpu_baseline():
+    r = subprocess.run([sys.executable, BENCH, "--workload", "c2_headline_1m_x_1000", "--rows",
+                        "200000", "--steps", "5", "--warmup", "1", "--cpu-sample-rows", "20000"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    out = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config",
+                "roofline", "cpu_baseline"):
+        assert key in out
+    assert out["n_gpus"] == 1 and out["steps"] == 5 and out["dtype"] == "f64"
+    assert out["vs_baseline"] is None and out["data"] == "synthetic"
+    assert "workload" in out["config"] and "model" not in out["config"]
+    rf = out["roofline"]
+    assert rf["bound"] == "hbm" and rf["peak"] == 8000.0 and rf["unit"] == "GB/s"
+    assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-12
+    assert 0.3 < rf["frac"] < 1.0
+    cb = out["cpu_baseline"]
+    assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
