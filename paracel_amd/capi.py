@@ -129,9 +129,11 @@ class Plr:
             X = np.ascontiguousarray(X)
             ldx = d
         y = _vec(y, n, "y")
+        self._shape = None
         self._check(self._lib.plr_set_data(self._h, _p(X), n, d, ldx, _p(y)))
 
     def alloc_data(self, n, d):
+        self._shape = None
         self._check(self._lib.plr_alloc_data(self._h, n, d))
 
     def set_data_chunk(self, row0, X, y):
@@ -142,9 +144,14 @@ class Plr:
 
     @property
     def shape(self):
-        n, d = C.c_int64(), C.c_int64()
-        self._check(self._lib.plr_get_shape(self._h, C.byref(n), C.byref(d)))
-        return n.value, d.value
+        # asked of the library once per resident shard (the per-step calls use it)
+        if getattr(self, "_shape", None) is None:
+            n, d = C.c_int64(), C.c_int64()
+            self._check(self._lib.plr_get_shape(self._h, C.byref(n), C.byref(d)))
+            if n.value == 0 and d.value == 0:
+                return 0, 0
+            self._shape = (n.value, d.value)
+        return self._shape
 
     # -- compute ----------------------------------------------------------
     def loss_grad(self, theta, flags=PLR_LOSS_REFERENCE):
