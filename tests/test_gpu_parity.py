@@ -538,6 +538,28 @@ def test_device_resident_training_in_every_kernel_family(plr, oracle, gen, n, d)
     assert rel(theta, oracle.train_dgd(X, y, np.zeros(d), alpha, beta, 6)) <= 1e-8
 
 
+def test_every_width_up_to_4400_against_numpy(plr):
+    # variant selection has a case per chunk count, tail capacity and pitch rule: walk
+    # every width (small shards, so this is about indexing, not bandwidth) against a
+    # library-routine reference -- numpy GEMV + scipy expit / logaddexp in fp64
+    from scipy.special import expit
+
+    rng = np.random.default_rng(123)
+    widths = list(range(1, 4400)) + list(range(4400, 20600, 97)) + [19455, 19456, 19457]
+    for d in widths:
+        n = 23 if d < 4400 else 11
+        X = rng.normal(size=(n, d)) / np.sqrt(d)
+        y = (rng.random(n) < 0.5) * 1.0
+        th = rng.normal(size=d)
+        plr.set_data(X, y)
+        g, loss, n_out = plr.loss_grad(th, 1)
+        z = X @ th
+        g_ref = X.T @ (expit(z) - y)
+        l_ref = np.sum(np.logaddexp(0.0, np.where(y == 1.0, -z, z)))
+        ok = n_out == n and rel(g, g_ref) <= 1e-11 and abs(loss - l_ref) <= 1e-11 * l_ref
+        assert ok, "d=%d: %s" % (d, plr.kernel_info())
+
+
 def _random_shapes(count, seed):
     rng = np.random.default_rng(seed)
     out = []
