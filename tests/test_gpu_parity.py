@@ -560,6 +560,29 @@ def test_every_width_up_to_4400_against_numpy(plr):
         assert ok, "d=%d: %s" % (d, plr.kernel_info())
 
 
+@pytest.mark.parametrize("d", [3, 16, 64, 100, 130, 257, 1000, 1025, 2500, 4097, 16385, 20001])
+def test_every_row_count_around_the_tile_sizes(plr, d):
+    # partial tiles, partial tail loads, fewer rows than row groups: n = 0..139 in every family
+    from scipy.special import expit
+
+    rng = np.random.default_rng(d)
+    Xall = rng.normal(size=(139, d)) / np.sqrt(d)
+    yall = (rng.random(139) < 0.5) * 1.0
+    th = rng.normal(size=d)
+    for n in range(0, 140):
+        X, y = Xall[:n], yall[:n]
+        plr.set_data(X, y)
+        g, loss, n_out = plr.loss_grad(th, 1)
+        z = X @ th
+        g_ref = X.T @ (expit(z) - y)
+        l_ref = np.sum(np.logaddexp(0.0, np.where(y == 1.0, -z, z)))
+        assert n_out == n
+        assert np.linalg.norm(g - g_ref) <= 1e-11 * max(np.linalg.norm(g_ref), 1e-300), (n, d)
+        assert abs(loss - l_ref) <= 1e-11 * max(l_ref, 1e-300), (n, d)
+        h = plr.predict(th)
+        assert h.shape == (n,) and (n == 0 or np.max(np.abs(h - expit(z))) <= 1e-14)
+
+
 def _random_shapes(count, seed):
     rng = np.random.default_rng(seed)
     out = []
