@@ -146,7 +146,16 @@ void logistic_regression_gpu::dump_result() {
     paracel_dump_vector(theta, "lr_theta_", "|");
     if (debug) paracel_dump_vector(loss_error, "lr_loss_error_", "\n");
   }
-  if (!pred_h.empty()) paracel_dump_vector(pred_h, "pred_v_", "\n");
+  // lr.cpp:346: (sample, h) pairs, one "x0,...,xk:h" line each (ps.hpp:1312-1319)
+  if (!pred_h.empty()) {
+    std::vector<std::pair<std::vector<double>, double> > predv;
+    predv.reserve(pred_h.size());
+    for (size_t i = 0; i < pred_h.size(); ++i)
+      predv.emplace_back(std::vector<double>(pred_samples.begin() + i * pred_dim,
+                                             pred_samples.begin() + (i + 1) * pred_dim),
+                         pred_h[i]);
+    paracel_dump_vector(predv, "pred_v_", "\n");
+  }
 }
 
 void logistic_regression_gpu::test(const std::string& test_fn) {
@@ -181,6 +190,8 @@ void logistic_regression_gpu::predict(const std::string& pred_fn) {
     ++n_local;
   }
   data_dim = kdim + 1;
+  pred_samples = flat;  // kept for dump_result, as the reference keeps pred_samples
+  pred_dim = data_dim;
   upload();
   pred_h.assign(n_local, 0.);
   check(plr_predict(gpu, theta.data(), pred_h.data()), "plr_predict");

@@ -63,6 +63,8 @@ class logistic_regression_gpu : public paralg {
   std::vector<double> theta, theta0;
   std::vector<double> loss_error;     // one entry per round when debug
   std::vector<double> pred_h;
+  std::vector<double> pred_samples;   // flattened prediction rows (lr.hpp: pred_samples)
+  int64_t pred_dim = 0;
   plr_ctx* gpu = nullptr;
   double round_sec = 0.;
 };

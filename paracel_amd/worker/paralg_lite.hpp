@@ -20,6 +20,7 @@
 #include <memory>
 #include <stdexcept>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "msgpack_lite.hpp"
@@ -232,13 +233,26 @@ class paralg {
   template <class T>
   void allreduce(T&) const {}                  // comm.hpp:629-636 MPI_SUM over 1 worker
 
-  // ps.hpp:983-1017 / :1308: "<output><prefix><rank>", std::to_string
+  // ps.hpp:983-1017 / :1308: "<output><prefix><rank>" (truncated, not
+  // appended, as with the reference's default append_flag), std::to_string
   // (6 decimals) joined by sep
   void paracel_dump_vector(const std::vector<double>& v, const std::string& prefix,
                            const std::string& sep) {
-    std::ofstream os(todir(output) + prefix + std::to_string(rank_), std::ios_base::app);
+    std::ofstream os(todir(output) + prefix + std::to_string(rank_));
     for (size_t i = 0; i + 1 < v.size(); ++i) os << std::to_string(v[i]) << sep;
     if (!v.empty()) os << std::to_string(v.back()) << '\n';
+  }
+  // the (sample, value) form of predictions, ps.hpp:1312-1319:
+  // "x0,x1,...,xk:value" per entry
+  void paracel_dump_vector(const std::vector<std::pair<std::vector<double>, double> >& v,
+                           const std::string& prefix, const std::string& sep) {
+    std::ofstream os(todir(output) + prefix + std::to_string(rank_));
+    for (size_t i = 0; i < v.size(); ++i) {
+      const std::vector<double>& x = v[i].first;
+      for (size_t j = 0; j + 1 < x.size(); ++j) os << std::to_string(x[j]) << ',';
+      if (!x.empty()) os << std::to_string(x.back());
+      os << ':' << std::to_string(v[i].second) << (i + 1 < v.size() ? sep : std::string("\n"));
+    }
   }
 
  protected:

@@ -86,8 +86,13 @@ def test_csv_driver_follows_the_reference_call_order(server_info, oracle, tmp_pa
     loss_line = [ln for ln in r.stdout.splitlines() if ln.startswith("final loss:")][0]
     assert abs(float(loss_line.split(":")[1]) - oracle.calc_loss(X, y, theta_ref)) <= 1e-10
     assert "loss in test dataset is:" in r.stdout
-    pred = np.array([float(t) for t in (outdir / "pred_v_0").read_text().split()])
+    # pred_v_<rank>: "x0,x1,...,xk:h" per sample (lr.cpp:346, ps.hpp:1312-1319)
+    plines = (outdir / "pred_v_0").read_text().splitlines()
+    assert len(plines) == n
+    pred = np.array([float(l.split(":")[1]) for l in plines])
     np.testing.assert_allclose(pred, oracle.predict(X, theta_ref), atol=5.1e-7, rtol=0)
+    xs = np.array([[float(t) for t in l.split(":")[0].split(",")] for l in plines])
+    np.testing.assert_allclose(xs, X, atol=5.1e-7, rtol=0)
     # debug: one loss per round, at the theta read at the start of that round
     curve = np.array([float(t) for t in (outdir / "lr_loss_error_0").read_text().split()])
     assert curve.shape == (20,) and abs(curve[0] - np.log(2)) < 1e-6 and curve[-1] < curve[0]
