@@ -108,8 +108,7 @@ void logistic_regression_gpu::dgd_learning() {
     paracel_sync();
     paracel_bupdate("theta", delta);
     paracel_sync();
-    if (debug || rounds <= 10)
-      std::cout << "worker" << get_worker_id() << " finished round: " << rd << std::endl;
+    std::cout << "worker" << get_worker_id() << " finished round: " << rd << std::endl;
   }
   round_sec += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
   theta = paracel_read<std::vector<double> >("theta");  // last pull
