@@ -70,6 +70,12 @@ def main():
         case("n40_d7_odd_labels", 40, 7, 6, special="odd_labels"),
         case("n25_d9_large_z", 25, 9, 7, xs=4.0, ts=2.0),
         case("n50_d3_readme_knobs", 50, 3, 8, alpha=0.001, beta=0.01),
+        # rows wider than 64 columns reach the other device kernels: one ragged chunk,
+        # chunk + tail stage, two chunks + wide tail, eight chunks + tail
+        case("n6_d70", 6, 70, 9, xs=0.5),
+        case("n7_d130_tail", 7, 130, 10, xs=0.5),
+        case("n4_d300_tail", 4, 300, 11, xs=0.25),
+        case("n2_d1030_tail", 2, 1030, 12, xs=0.125),
     ]
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lr_small.json")
     with open(out, "w") as f:
