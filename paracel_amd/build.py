@@ -51,6 +51,14 @@ def build_copy_probe():
     return out
 
 
+def build_plan_check():
+    """Host-only check of the width -> kernel-variant choice -> paracel_amd/plr_plan_check"""
+    out = os.path.join(_HERE, "plr_plan_check")
+    _run(["g++", "-O2", "-std=c++17", "-Wall", "-Wextra", "-o", out,
+          os.path.join(_HERE, "csrc", "plr_plan_check.cpp")])
+    return out
+
+
 def build_worker():
     """Host side of the worker path (g++): parameter-server process, reducer
     plugin, GPU LR worker, shard tool ->
@@ -61,4 +69,5 @@ def build_worker():
 
 
 def build_all():
-    return [build_libplr(), build_libplr_gen(), build_copy_probe()] + build_worker()
+    return [build_libplr(), build_libplr_gen(), build_copy_probe(), build_plan_check()] + \
+        build_worker()

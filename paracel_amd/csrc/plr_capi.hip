@@ -12,6 +12,7 @@
 #include <string>
 
 #include "plr_kernels.hpp"
+#include "plr_plan.hpp"
 
 namespace {
 
@@ -20,144 +21,43 @@ using plr::PassArgs;
 
 typedef void (*pass_fn)(PassArgs);
 
-struct Variant {
-  int nch, R, wcol, wrow;
-  bool thl;
-  int tl;  // tail loads per tile (0: the row ends inside or at the end of a chunk)
-  // [grad][allch]; one-wave rows always match their variant exactly, so they
-  // carry only the allch instances
+// The shapes and the width -> variant choice live in plr_plan.hpp (host-only,
+// checked on a CPU for every width); here the kernel instances, in the same
+// order.  [grad][allch]: rows handled by one wave and the tail-stage variants
+// always match their variant exactly, so they carry only the allch instances.
+using plr_plan::Shape;
+using plr_plan::kShapes;
+using plr_plan::kNumShapes;
+using plr_plan::kBlkNch;
+using plr_plan::kBlkWcol;
+using plr_plan::kBlockCols;
+
+struct VariantFns {
   pass_fn fn[2][2];
 };
 
-// several waves side by side over the columns
-#define PLR_VARIANT(NCH, R, WCOL, WROW, MINW, THL)                         \
-  {NCH, R, WCOL, WROW, THL, 0,                                             \
-   {{plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, false, THL>,         \
-     plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, true, THL>},         \
-    {plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, false, THL>,          \
-     plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, true, THL>}}}
-// one wave per row: NCH full chunks (the last may be ragged when TL == 0),
-// plus, with TL > 0, up to 128*TL/R leftover columns
-#define PLR_ROW(NCH, R, WROW, MINW, TL)                                                      \
-  {NCH, R, 1, WROW, false, TL,                                                               \
-   {{nullptr, plr::shard_pass<NCH, R, 1, WROW, MINW, false, true, false, plr::kPassFused, TL>}, \
-    {nullptr, plr::shard_pass<NCH, R, 1, WROW, MINW, true, true, false, plr::kPassFused, TL>}}}
+template <int NCH, int R, int WCOL, int WROW, int MINW, bool THL, int TL>
+VariantFns make_fns() {
+  VariantFns f = {{{nullptr, nullptr}, {nullptr, nullptr}}};
+  f.fn[0][1] = plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, true, THL, plr::kPassFused, TL>;
+  f.fn[1][1] = plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, true, THL, plr::kPassFused, TL>;
+  if constexpr (WCOL > 1 && TL == 0) {
+    f.fn[0][0] = plr::shard_pass<NCH, R, WCOL, WROW, MINW, false, false, THL>;
+    f.fn[1][0] = plr::shard_pass<NCH, R, WCOL, WROW, MINW, true, false, THL>;
+  }
+  return f;
+}
 
-// A row of C chunks (128 columns each) is handled by one wave up to C = 32
-// (one exact variant per C; the last chunk may be ragged), then by ceil(C/8)
-// chunks per wave on as many waves side by side as that takes (<= 8), so at
-// most one wave of the workgroup is partly idle.  Between 17 and 32 chunks
-// the several-waves variants are 1-2 % faster when the row fills them exactly
-// (18, 21, 24, 28, 32 whole chunks) and up to 10 % slower otherwise, so only
-// those widths take them.  A row of up to 16 chunks that ends 32-64 columns
-// past a chunk boundary takes the variant with that many full chunks and a
-// tail stage.  Tile heights and register budgets
-// (MINW = waves per SIMD the allocation leaves room for) come from sweeps on
-// MI355X: one or two resident waves per SIMD, each with 16-48 KiB of loads in
-// flight, stream fastest; any variant that spills registers loses a third of
-// the bandwidth or more.  From 65 chunks on theta lives in LDS and a variant
-// covers every per-wave count up to its NCH.
-// several waves side by side, exactly WCOL*NCH full chunks plus a tail stage
-// on the last wave (the 2^k + 1 widths of wide rows)
-#define PLR_VARIANT_TAIL(NCH, R, WCOL, MINW, THL, TL)                                            \
-  {NCH, R, WCOL, 1, THL, TL,                                                                     \
-   {{nullptr, plr::shard_pass<NCH, R, WCOL, 1, MINW, false, true, THL, plr::kPassFused, TL>},    \
-    {nullptr, plr::shard_pass<NCH, R, WCOL, 1, MINW, true, true, THL, plr::kPassFused, TL>}}}
-
-const Variant kVariants[] = {
-    // one wave per row, exact chunk counts
-    PLR_ROW(1, 16, 4, 2, 0),
-    PLR_ROW(2, 32, 4, 1, 0),
-    PLR_ROW(3, 16, 2, 1, 0),
-    PLR_ROW(4, 16, 2, 1, 0),
-    PLR_ROW(5, 8, 2, 1, 0),
-    PLR_ROW(6, 8, 2, 1, 0),
-    PLR_ROW(7, 4, 4, 1, 0),
-    PLR_ROW(8, 4, 4, 1, 0),
-    PLR_ROW(9, 4, 4, 1, 0),
-    PLR_ROW(10, 4, 4, 1, 0),
-    PLR_ROW(11, 4, 4, 1, 0),
-    PLR_ROW(12, 2, 4, 1, 0),
-    PLR_ROW(13, 4, 4, 1, 0),
-    PLR_ROW(14, 4, 4, 1, 0),
-    PLR_ROW(15, 2, 4, 1, 0),
-    PLR_ROW(16, 2, 4, 1, 0),
-    PLR_ROW(17, 1, 4, 1, 0),
-    PLR_ROW(18, 1, 4, 1, 0),
-    PLR_ROW(19, 1, 4, 1, 0),
-    PLR_ROW(20, 1, 4, 1, 0),
-    PLR_ROW(21, 1, 4, 1, 0),
-    PLR_ROW(22, 1, 4, 1, 0),
-    PLR_ROW(23, 1, 4, 1, 0),
-    PLR_ROW(24, 1, 4, 1, 0),
-    PLR_ROW(25, 1, 4, 1, 0),
-    PLR_ROW(26, 1, 4, 1, 0),
-    PLR_ROW(27, 1, 4, 1, 0),
-    PLR_ROW(28, 1, 4, 1, 0),
-    PLR_ROW(29, 1, 4, 1, 0),
-    PLR_ROW(30, 1, 4, 1, 0),
-    PLR_ROW(31, 1, 4, 1, 0),
-    PLR_ROW(32, 1, 4, 1, 0),
-    // one wave per row with a tail stage (capacity 128*TL/R columns)
-    PLR_ROW(1, 32, 4, 1, 2),   // 8
-    PLR_ROW(1, 32, 4, 1, 4),   // 16
-    PLR_ROW(1, 16, 4, 2, 4),   // 32
-    PLR_ROW(1, 8, 4, 2, 4),    // 64
-    PLR_ROW(2, 16, 4, 1, 1),   // 8
-    PLR_ROW(2, 16, 4, 1, 2),   // 16
-    PLR_ROW(2, 16, 4, 1, 4),   // 32
-    PLR_ROW(2, 8, 4, 2, 4),    // 64
-    PLR_ROW(3, 8, 4, 1, 1),    // 16
-    PLR_ROW(3, 8, 4, 1, 2),    // 32
-    PLR_ROW(4, 8, 4, 1, 1),    // 16
-    PLR_ROW(4, 8, 4, 1, 2),    // 32
-    PLR_ROW(6, 4, 4, 1, 1),    // 32
-    PLR_ROW(7, 4, 4, 1, 1),    // 32
-    PLR_ROW(8, 4, 4, 1, 1),    // 32
-    PLR_ROW(8, 4, 4, 1, 2),    // 64
-    PLR_ROW(9, 4, 4, 1, 1),    // 32
-    PLR_ROW(10, 4, 4, 1, 1),   // 32
-    PLR_ROW(11, 4, 4, 1, 1),   // 32
-    PLR_ROW(12, 2, 4, 1, 1),   // 64
-    PLR_ROW(13, 2, 4, 1, 1),   // 64
-    PLR_ROW(14, 2, 4, 1, 1),   // 64
-    PLR_ROW(15, 2, 4, 1, 1),   // 64
-    PLR_ROW(16, 2, 4, 1, 1),   // 64
-    PLR_VARIANT_TAIL(4, 4, 8, 2, false, 1),   // 4096 + 32
-    PLR_VARIANT_TAIL(8, 2, 8, 2, true, 1),    // 8192 + 64
-    PLR_VARIANT_TAIL(16, 1, 8, 2, true, 1),   // 16384 + 128
-    // 3 chunks per wave: 17..24
-    PLR_VARIANT(3, 8, 6, 1, 2, false),
-    PLR_VARIANT(3, 8, 7, 1, 2, false),
-    PLR_VARIANT(3, 8, 8, 1, 2, false),
-    // 4..7 chunks per wave: 25..56
-    PLR_VARIANT(4, 4, 7, 1, 2, false),
-    PLR_VARIANT(4, 4, 8, 1, 2, false),
-    PLR_VARIANT(5, 4, 7, 1, 2, false),
-    PLR_VARIANT(5, 4, 8, 1, 2, false),
-    PLR_VARIANT(6, 4, 7, 1, 2, false),
-    PLR_VARIANT(6, 4, 8, 1, 2, false),
-    PLR_VARIANT(7, 4, 7, 1, 2, false),
-    PLR_VARIANT(7, 4, 8, 1, 2, false),
-    // 8 chunks per wave and up: theta in LDS
-    PLR_VARIANT(8, 4, 8, 1, 2, true),     // 57..64
-    PLR_VARIANT(10, 2, 8, 1, 2, true),    // ..80
-    PLR_VARIANT(12, 2, 8, 1, 2, true),    // ..96
-    PLR_VARIANT(14, 1, 8, 1, 2, true),    // ..112
-    PLR_VARIANT(16, 1, 8, 1, 2, true),    // ..128
-    PLR_VARIANT(17, 1, 8, 1, 2, true),    // ..136
-    PLR_VARIANT(19, 1, 8, 1, 2, true),    // ..152 (152 KiB of theta in LDS)
+const VariantFns kFns[] = {
+#define PLR_V(NCH, R, WCOL, WROW, MINW, THL, TL) make_fns<NCH, R, WCOL, WROW, MINW, THL, TL>(),
+#include "plr_variants.def"
+#undef PLR_V
 };
-constexpr int kAlwaysOneWave = 16;  // up to here no several-waves variant is considered
-constexpr int kMaxRowChunks = 32;   // widest one-wave row
-constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
-constexpr int64_t kMaxFusedCols = 19456;
+static_assert(sizeof(kFns) / sizeof(kFns[0]) == (size_t)kNumShapes, "one kernel set per shape");
 
-// Rows wider than that are processed in column blocks of 16384, in two sweeps
-// over X (dot products of all blocks, then residuals, then the rank-1
-// updates of all blocks): X is read twice, but any width works.
-constexpr int kBlkNch = 16, kBlkWcol = 8;
-constexpr int64_t kBlockCols = (int64_t)kBlkNch * kBlkWcol * plr::kChunkCols;  // 16384
+// Rows wider than the widest fused variant are processed in column blocks of
+// 16384, in two sweeps over X (dot products of all blocks, then residuals,
+// then the rank-1 updates of all blocks): X is read twice, but any width works.
 // [allch]
 const pass_fn kBlockDot[2] = {
     plr::shard_pass<kBlkNch, 1, kBlkWcol, 1, 2, false, false, true, plr::kPassDot>,
@@ -183,9 +83,9 @@ const PackedVariant kPacked[] = {
     PLR_PACKED(5, 2, 2, 1),  // pitch 32
     PLR_PACKED(6, 1, 2, 1),  // pitch 64
 };
-constexpr int64_t kMaxPackedCols = 64;
 
-const Variant kBlockVariant = {kBlkNch, 1, kBlkWcol, 1, true, 0, {{nullptr, nullptr}, {nullptr, nullptr}}};
+// the column-blocked path's shape: 8 waves x 16 chunks, one row per tile, theta in LDS
+const Shape kBlockShape = {kBlkNch, 1, kBlkWcol, 1, 2, true, 0};
 
 std::string g_create_error;
 
@@ -204,7 +104,8 @@ struct plr_ctx {
   bool have_data = false;
 
   // per-shape workspace
-  const Variant* var = nullptr;
+  const Shape* var = nullptr;       // shape of the shard_pass variant in use
+  const VariantFns* fns = nullptr;  // its kernel instances (fused path)
   int nch_rt = 0;
   int grid = 0, grid_nograd = 0;
   bool allch = false;
@@ -291,24 +192,29 @@ void free_shape(plr_ctx* c) {
   c->packed = nullptr;
   c->tail_cols = 0;
   c->var = nullptr;
+  c->fns = nullptr;
   c->info.clear();
 }
 
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-// Pick the kernel variant and persistent grid for an n x d shard.
+// Pick the kernel variant (plr_plan.hpp) and the persistent grid for an
+// n x d shard.
 int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
-  if (d <= kMaxPackedCols) {
-    int logp = 1;
-    while ((int64_t(1) << logp) < d) ++logp;
-    const PackedVariant* pv = &kPacked[logp - 1];
+  plr_plan::Plan pl;
+  if (!plr_plan::plan_width(d, pl))
+    return fail(c, PLR_ERR_UNSUPPORTED, "no kernel variant covers this width");
+  c->pitch = pl.pitch;
+  c->theta_len = pl.theta_len;
+  c->nch_rt = pl.nch_rt;
+  c->allch = pl.allch;
+  c->tail_cols = pl.tail_cols;
+  if (pl.path == plr_plan::kPathPacked) {
+    const PackedVariant* pv = &kPacked[pl.logp - 1];
     const int threads = plr::kWave * pv->wrow;
     c->packed = pv;
-    c->var = &kBlockVariant;  // unused by the packed path, kept non-null
-    c->pitch = int64_t(1) << logp;
+    c->var = &kBlockShape;  // unused by the packed path, kept non-null
     c->nch_rt = 1;
-    c->allch = false;
-    c->theta_len = plr::kChunkCols;
     int occ = 0, occ2 = 0;
     PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
                    &occ, reinterpret_cast<const void*>(pv->fn[1]), threads, 0));
@@ -329,16 +235,10 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
     c->info = b;
     return PLR_OK;
   }
-  if (d > kMaxFusedCols) {
-    const int64_t pitch = (d + 15) & ~int64_t(15);
+  if (pl.path == plr_plan::kPathBlocked) {
     const int threads = plr::kWave * kBlkWcol;
-    c->var = &kBlockVariant;
+    c->var = &kBlockShape;
     c->blocked = true;
-    c->pitch = pitch;
-    c->nch_rt = kBlkNch;
-    c->allch = false;
-    // theta padded so that the last (narrower) block still reads whole slabs
-    c->theta_len = ceil_div(pitch, kBlockCols) * kBlockCols;
     int occ = 0, occ2 = 0;
     PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
                    &occ, reinterpret_cast<const void*>(kBlockAxpy[0]), threads, 0));
@@ -354,80 +254,25 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
     snprintf(b, sizeof b,
              "column-blocked shard_pass<NCH=%d,R=1,WCOL=%d> two sweeps over %lld blocks of %lld "
              "columns, pitch=%lld grid=%d x %d threads",
-             kBlkNch, kBlkWcol, (long long)ceil_div(pitch, kBlockCols), (long long)kBlockCols,
-             (long long)pitch, c->grid, threads);
+             kBlkNch, kBlkWcol, (long long)ceil_div(c->pitch, kBlockCols), (long long)kBlockCols,
+             (long long)c->pitch, c->grid, threads);
     c->info = b;
     return PLR_OK;
   }
-  // even pitch so that every row start is 16-byte aligned; wide rows are
-  // aligned to 128 B (<= 0.7 % more bytes, +3 % bandwidth when d is odd)
-  const int64_t pitch = (d >= 2048) ? ((d + 15) & ~int64_t(15)) : ((d + 1) & ~int64_t(1));
-  const int64_t chunks = ceil_div(pitch, plr::kChunkCols);
-  const Variant* v = nullptr;
-  int tail = 0;
-  // a few columns past a chunk boundary: the tail-stage variant with the
-  // smallest capacity that holds them
-  const int64_t full = pitch / plr::kChunkCols, rem = pitch % plr::kChunkCols;
-  if (rem != 0 && full >= 1) {
-    int best_cap = 1 << 30;
-    for (int i = 0; i < kNumVariants; ++i) {
-      const Variant& k = kVariants[i];
-      if (k.tl == 0 || (int64_t)k.nch * k.wcol != full) continue;
-      const int cap = plr::kChunkCols * k.tl / k.R;
-      if (cap >= rem && cap < best_cap) {
-        v = &k;
-        best_cap = cap;
-      }
-    }
-    if (v) tail = (int)rem;
-  }
-  if (!v) {
-    // (waves, chunks per wave) for this width, then the variant that has them
-    int want_w = 8, want_k = (int)ceil_div(chunks, 8);  // beyond 64 chunks: theta in LDS
-    if (chunks <= 64) {
-      want_k = (int)ceil_div(chunks, 8);
-      want_w = (int)ceil_div(chunks, want_k);
-      const bool fills_waves = rem == 0 && chunks == (int64_t)want_k * want_w;
-      if (chunks <= kMaxRowChunks && !(chunks > kAlwaysOneWave && fills_waves)) {
-        want_w = 1;
-        want_k = (int)chunks;
-      }
-    }
-    for (int i = 0; i < kNumVariants; ++i) {
-      const Variant& k = kVariants[i];
-      if (k.tl != 0) continue;
-      const bool fits = (want_k >= 8 && want_w == 8)
-                            ? (k.thl && k.wcol == 8 && k.nch >= want_k)
-                            : (!k.thl && k.wcol == want_w && k.nch == want_k);
-      if (fits) {
-        v = &k;
-        break;
-      }
-    }
-  }
-  if (!v) return fail(c, PLR_ERR_UNSUPPORTED, "no kernel variant covers this width");
+  const Shape* v = &kShapes[pl.variant];
+  const VariantFns* f = &kFns[pl.variant];
   c->var = v;
-  c->pitch = pitch;
-  c->tail_cols = tail;
-  if (tail) {
-    c->nch_rt = v->nch;
-    c->allch = true;
-    c->theta_len = (full + 1) * plr::kChunkCols;
-  } else {
-    c->nch_rt = (int)ceil_div(chunks, v->wcol);  // == v->nch except for the theta-in-LDS variants
-    c->allch = (chunks == (int64_t)v->nch * v->wcol);
-    c->theta_len = (int64_t)v->wcol * c->nch_rt * plr::kChunkCols;
-  }
-  if (!v->fn[1][c->allch] || !v->fn[0][c->allch])
+  c->fns = f;
+  if (!f->fn[1][c->allch] || !f->fn[0][c->allch])
     return fail(c, PLR_ERR_UNSUPPORTED, "kernel variant lacks the instance this width needs");
   const int threads = plr::kWave * v->wcol * v->wrow;
   const int64_t ntiles = ceil_div(n, v->R);
   const int64_t want = ceil_div(ntiles, v->wrow);
   int occ = 0, occ_ng = 0;
   PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                 &occ, reinterpret_cast<const void*>(v->fn[1][c->allch]), threads, 0));
+                 &occ, reinterpret_cast<const void*>(f->fn[1][c->allch]), threads, 0));
   PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                 &occ_ng, reinterpret_cast<const void*>(v->fn[0][c->allch]), threads, 0));
+                 &occ_ng, reinterpret_cast<const void*>(f->fn[0][c->allch]), threads, 0));
   if (occ < 1 || occ_ng < 1)
     return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
   int64_t g = (int64_t)c->num_cu * occ, g2 = (int64_t)c->num_cu * occ_ng;
@@ -441,8 +286,8 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   snprintf(b, sizeof b,
            "shard_pass<NCH=%d,R=%d,WCOL=%d,WROW=%d,ALLCH=%d,TL=%d> nch_rt=%d tail=%d pitch=%lld "
            "grid=%d x %d threads (occupancy %d blocks/CU, %d CUs)",
-           v->nch, v->R, v->wcol, v->wrow, (int)c->allch, v->tl, c->nch_rt, tail,
-           (long long)pitch, c->grid, threads, occ, c->num_cu);
+           v->nch, v->R, v->wcol, v->wrow, (int)c->allch, v->tl, c->nch_rt, c->tail_cols,
+           (long long)c->pitch, c->grid, threads, occ, c->num_cu);
   c->info = b;
   return PLR_OK;
 }
@@ -571,7 +416,7 @@ enum PassKind { kPassGrad, kPassDelta, kPassLoss, kPassPredict, kPassPredictLine
 // d_curve[train_round].
 int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, double beta,
                  double* out, int train_round) {
-  const Variant* v = c->var;
+  const Shape* v = c->var;
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
   const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
   const int grid = grad ? c->grid : c->grid_nograd;
@@ -602,7 +447,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     hipLaunchKernelGGL(c->packed->fn[grad ? 1 : 0], dim3(grid), dim3(threads), 0, c->stream, pa);
     PLR_HIP(c, hipGetLastError());
   } else if (!c->blocked) {
-    hipLaunchKernelGGL(v->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
+    hipLaunchKernelGGL(c->fns->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
                        c->stream, pa);
     PLR_HIP(c, hipGetLastError());
   } else if (c->n > 0) {

@@ -1,0 +1,110 @@
+// Host-only check of the width -> variant choice (plr_plan.hpp): walks every
+// width and verifies what the kernels and the launch code rely on.
+//   plr_plan_check              check d = 1 .. 70000, report, exit 0/1
+//   plr_plan_check <d>          print the plan for one width
+#include <stdio.h>
+#include <stdlib.h>
+
+#include <vector>
+
+#include "plr_plan.hpp"
+
+using namespace plr_plan;
+
+static int failures = 0;
+#define CHECK(cond, d)                                                        \
+  do {                                                                        \
+    if (!(cond)) {                                                            \
+      if (++failures <= 20) printf("d=%lld: %s\n", (long long)(d), #cond);    \
+    }                                                                         \
+  } while (0)
+
+static void print_plan(int64_t d) {
+  Plan p;
+  if (!plan_width(d, p)) {
+    printf("d=%lld: no variant\n", (long long)d);
+    return;
+  }
+  static const char* names[] = {"packed", "fused", "blocked"};
+  printf("d=%lld path=%s pitch=%lld theta_len=%lld", (long long)d, names[p.path],
+         (long long)p.pitch, (long long)p.theta_len);
+  if (p.path == kPathPacked) printf(" logp=%d", p.logp);
+  if (p.path == kPathFused) {
+    const Shape& s = kShapes[p.variant];
+    printf(" variant=%d NCH=%d R=%d WCOL=%d WROW=%d THL=%d TL=%d chunks=%lld nch_rt=%d allch=%d tail=%d",
+           p.variant, s.nch, s.R, s.wcol, s.wrow, (int)s.thl, s.tl, (long long)p.chunks, p.nch_rt,
+           (int)p.allch, p.tail_cols);
+  }
+  printf("\n");
+}
+
+int main(int argc, char** argv) {
+  if (argc > 1) {
+    print_plan(atoll(argv[1]));
+    return 0;
+  }
+  std::vector<int64_t> used(kNumShapes, 0);
+  const int64_t kMaxD = 70000;
+  for (int64_t d = 1; d <= kMaxD; ++d) {
+    Plan p;
+    if (!plan_width(d, p)) {
+      CHECK(false && "plan_width failed", d);
+      continue;
+    }
+    CHECK(p.pitch >= d && p.pitch % 2 == 0, d);
+    CHECK(p.theta_len >= p.pitch || p.path == kPathPacked, d);
+    if (p.path == kPathPacked) {
+      CHECK(d <= kMaxPackedCols && p.logp >= 1 && p.logp <= 6, d);
+      CHECK(p.pitch == (int64_t(1) << p.logp) && (p.pitch / 2 < d || d == 1), d);
+      CHECK(p.theta_len >= p.pitch, d);
+    } else if (p.path == kPathBlocked) {
+      CHECK(d > kMaxFusedCols && p.pitch % 16 == 0 && p.pitch - d < 16, d);
+      CHECK(p.theta_len % kBlockCols == 0 && p.theta_len >= p.pitch, d);
+    } else {
+      CHECK(d > kMaxPackedCols && d <= kMaxFusedCols, d);
+      CHECK(p.variant >= 0 && p.variant < kNumShapes, d);
+      if (p.variant < 0 || p.variant >= kNumShapes) continue;
+      const Shape& s = kShapes[p.variant];
+      used[p.variant]++;
+      CHECK(p.pitch - d < (d >= 2048 ? 16 : 2), d);
+      CHECK(d < 2048 || p.pitch % 16 == 0, d);
+      CHECK(p.chunks == ceil_div(p.pitch, kChunkCols), d);
+      CHECK(s.wcol == 1 || s.wrow == 1, d);
+      CHECK((s.R & (s.R - 1)) == 0 && s.R <= 64, d);
+      // theta in LDS: one slab per wave, within the 160 KiB of a compute unit
+      CHECK(!s.thl || (int64_t)s.wcol * s.wrow * s.nch * 1024 <= 160 * 1024, d);
+      // the 32-bit lane offsets of a tile (R rows of pitch doubles) cannot wrap
+      CHECK((int64_t)s.R * p.pitch * 8 + 8 * p.pitch < (int64_t(1) << 32), d);
+      if (p.tail_cols) {
+        CHECK(s.tl > 0 && s.tl <= s.R && s.tl <= 4 && (s.tl & (s.tl - 1)) == 0, d);
+        CHECK(p.allch && p.nch_rt == s.nch, d);
+        CHECK((int64_t)s.nch * s.wcol * kChunkCols + p.tail_cols == p.pitch, d);
+        CHECK(p.tail_cols % 2 == 0 && p.tail_cols <= kChunkCols * s.tl / s.R, d);
+        CHECK(p.theta_len >= p.pitch, d);
+      } else {
+        CHECK(s.tl == 0, d);
+        CHECK(p.nch_rt >= 1 && p.nch_rt <= s.nch, d);
+        CHECK((int64_t)s.wcol * p.nch_rt >= p.chunks, d);            // every chunk has a wave
+        CHECK((int64_t)(s.wcol - 1) * p.nch_rt < p.chunks, d);       // no wave without a chunk
+        CHECK(p.allch == (p.chunks == (int64_t)s.nch * s.wcol), d);
+        CHECK(!p.allch || p.nch_rt == s.nch, d);
+        // one-wave rows exist only as exact (allch) instances
+        CHECK(s.wcol > 1 || p.allch, d);
+        CHECK(p.theta_len >= (int64_t)s.wcol * p.nch_rt * kChunkCols, d);
+        // idle chunk slots: fewer than one wave's worth
+        CHECK((int64_t)s.wcol * p.nch_rt - p.chunks < p.nch_rt, d);
+      }
+    }
+  }
+  int dead = 0;
+  for (int i = 0; i < kNumShapes; ++i)
+    if (!used[i]) {
+      const Shape& s = kShapes[i];
+      printf("variant %d (NCH=%d R=%d WCOL=%d WROW=%d THL=%d TL=%d) is never chosen\n", i, s.nch,
+             s.R, s.wcol, s.wrow, (int)s.thl, s.tl);
+      ++dead;
+    }
+  printf("%s: %lld widths, %d variants, %d never chosen, %d failed checks\n",
+         (failures || dead) ? "FAIL" : "ok", (long long)kMaxD, kNumShapes, dead, failures);
+  return (failures || dead) ? 1 : 0;
+}
