@@ -107,6 +107,29 @@ int plr_predict(plr_ctx* ctx, const double* theta, double* h_out);
  * (the linear model's prediction; n doubles out). */
 int plr_predict_linear(plr_ctx* ctx, const double* theta, double* z_out);
 
+/* plr_loss_grad for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * No counterpart in the reference.  It needs no context and calls no
+ * hipMalloc / hipFree: the caller passes every input and output as DEVICE
+ * pointers, and the pass keeps its partial results (the zero-padded copy of
+ * theta, the per-workgroup gradient and loss partials) in one static device
+ * array of 8 MiB + 20 KiB per GPU, which that GPU holds until the process ends.
+ *   dX     n rows at a pitch of ldx doubles; ldx must be a multiple of 128
+ *          with d <= ldx <= 2048 (the limit of the static array; wider rows
+ *          are refused with PLR_ERR_INVALID), columns d..ldx-1 must be zero
+ *   dy     n labels;   dtheta  d doubles
+ *   dout   d + 1 doubles: gsum as plr_loss_grad defines it, then loss_sum
+ *   flags  a PLR_LOSS_* value
+ * The work is enqueued on `hip_stream` (a hipStream_t; NULL = the default
+ * stream) and the call returns without waiting: dout is valid once the stream
+ * has reached that point.  All calls on one GPU share that GPU's static array,
+ * so calls that may overlap on a GPU (different streams, different threads)
+ * race; order them on one stream.  Errors are described by
+ * plr_last_error(NULL). */
+int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX,
+                          const double* dy, int64_t n, int64_t d, int64_t ldx,
+                          const double* dtheta, double* dout, unsigned flags);
+
 /* Block until everything this context (and the device) was asked to do has
  * finished.  The compute entry points already return drained; this is the
  * explicit fence benchmarks put on both sides of a timed region. */
@@ -150,7 +173,8 @@ int plr_probe_copy_bandwidth(plr_ctx* ctx, int64_t bytes, int reps, double* gb_p
 const char* plr_kernel_info(const plr_ctx* ctx);
 
 /* Context-owned message of the last error ("" if none); never freed.
- * plr_last_error(NULL) describes the last plr_create failure. */
+ * plr_last_error(NULL) describes the last failure of a call that takes no
+ * context (plr_create, plr_loss_grad_noalloc). */
 const char* plr_last_error(const plr_ctx* ctx);
 
 const char* plr_version(void);

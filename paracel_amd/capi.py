@@ -32,6 +32,8 @@ SYMBOLS = [
     ("plr_calc_loss", C.c_int, [_ctx, _dp, _dp, _i64p, C.c_uint]),
     ("plr_predict", C.c_int, [_ctx, _dp, _dp]),
     ("plr_predict_linear", C.c_int, [_ctx, _dp, _dp]),
+    ("plr_loss_grad_noalloc", C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                        C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_uint]),
     ("plr_synchronize", C.c_int, [_ctx]),
     ("plr_set_timing", C.c_int, [_ctx, C.c_int]),
     ("plr_probe_copy_bandwidth", C.c_int, [_ctx, C.c_int64, C.c_int, C.POINTER(C.c_double)]),
@@ -86,6 +88,18 @@ def _vec(a, n=None, name="array"):
 
 def _p(a):
     return a.ctypes.data_as(_dp) if a is not None else None
+
+
+def loss_grad_noalloc(dX, dy, n, d, ldx, dtheta, dout, flags=PLR_LOSS_REFERENCE, device=0,
+                      stream=None):
+    """plr_loss_grad_noalloc on raw DEVICE addresses (ints); enqueues on `stream`
+    (a hipStream_t as an int, None = the default stream) and returns at once."""
+    lib = load_library()
+    rc = lib.plr_loss_grad_noalloc(int(device), C.c_void_p(stream), C.c_void_p(dX),
+                                   C.c_void_p(dy), n, d, ldx, C.c_void_p(dtheta),
+                                   C.c_void_p(dout), flags)
+    if rc != 0:
+        raise PlrError(rc, lib.plr_last_error(None).decode())
 
 
 class Plr:

@@ -9,6 +9,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <mutex>
 #include <string>
 
 #include "plr_kernels.hpp"
@@ -87,7 +88,30 @@ const PackedVariant kPacked[] = {
 // the column-blocked path's shape: 8 waves x 16 chunks, one row per tile, theta in LDS
 const Shape kBlockShape = {kBlkNch, 1, kBlkWcol, 1, 2, true, 0};
 
-std::string g_create_error;
+std::string g_create_error;  // last failure of a call that has no context
+
+// ---- static device scratch of plr_loss_grad_noalloc ------------------------
+// Everything that entry point needs beyond the caller's inputs and outputs:
+// the zero-padded copy of theta, the per-workgroup loss partials and the
+// per-workgroup gradient partials.  One array per GPU, held until the process
+// ends; every call on a GPU uses that GPU's copy.
+constexpr int64_t kNaMaxPitch = 2048;  // widest row pitch (doubles) the entry point takes
+constexpr int kNaMaxGrid = 512;        // most workgroups a pass may use
+constexpr size_t kNaThetaOff = 0;
+constexpr size_t kNaLossOff = kNaThetaOff + (size_t)kNaMaxPitch * sizeof(double);
+constexpr size_t kNaPartOff = kNaLossOff + (size_t)kNaMaxGrid * sizeof(double);
+constexpr size_t kNaScratchBytes =
+    kNaPartOff + (size_t)kNaMaxGrid * kNaMaxPitch * sizeof(double);  // 8 MiB + 20 KiB
+static_assert(kNaLossOff % 256 == 0 && kNaPartOff % 256 == 0, "sub-buffers stay aligned");
+
+static __device__ __align__(256) unsigned char scratch[kNaScratchBytes];
+
+// In host code `scratch` is only a handle for the symbol; the device address
+// differs per GPU and is looked up once per device, with that device current.
+constexpr int kNaMaxDevices = 64;
+std::mutex g_na_mutex;
+unsigned char* g_na_ptr[kNaMaxDevices] = {};
+int g_na_num_cu[kNaMaxDevices] = {};
 
 }  // namespace
 
@@ -810,6 +834,139 @@ int plr_reset_timing(plr_ctx* c) {
   if (!c) return PLR_ERR_INVALID;
   c->last_ms = c->sum_ms = 0.;
   c->launches = 0;
+  return PLR_OK;
+}
+
+int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, const double* dy,
+                          int64_t n, int64_t d, int64_t ldx, const double* dtheta,
+                          double* dout, unsigned flags) {
+  auto bad = [](int code, const std::string& msg) {
+    g_create_error = "plr_loss_grad_noalloc: " + msg;
+    return code;
+  };
+  if (device_id < 0 || device_id >= kNaMaxDevices) return bad(PLR_ERR_INVALID, "device_id out of range");
+  if (n < 0 || d < 1) return bad(PLR_ERR_INVALID, "need n >= 0 and d >= 1");
+  if (ldx < plr::kChunkCols || ldx % plr::kChunkCols != 0 || ldx < d)
+    return bad(PLR_ERR_INVALID, "ldx must be a multiple of 128 and >= d");
+  if (ldx > kNaMaxPitch) {
+    char b[160];
+    snprintf(b, sizeof b, "ldx = %lld exceeds the static scratch's limit of %lld columns",
+             (long long)ldx, (long long)kNaMaxPitch);
+    return bad(PLR_ERR_INVALID, b);
+  }
+  if (n > (int64_t)((SIZE_MAX / sizeof(double)) / (size_t)ldx))
+    return bad(PLR_ERR_INVALID, "n * ldx overflows");
+  if ((n > 0 && (!dX || !dy)) || !dtheta || !dout)
+    return bad(PLR_ERR_INVALID, "device pointers must not be NULL");
+  if (flags > plr::kLossSquared) return bad(PLR_ERR_INVALID, "unknown loss flag");
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+
+#define PLR_NA_HIP(call)                                                        \
+  do {                                                                          \
+    hipError_t e_ = (call);                                                     \
+    if (e_ != hipSuccess) {                                                     \
+      (void)hipGetLastError();                                                  \
+      return bad(PLR_ERR_HIP, std::string(#call " failed: ") + hipGetErrorString(e_)); \
+    }                                                                           \
+  } while (0)
+
+  PLR_NA_HIP(hipSetDevice(device_id));
+  unsigned char* base = nullptr;
+  int num_cu = 0;
+  {
+    // first call on this device: the device's own address of the static array
+    std::lock_guard<std::mutex> lock(g_na_mutex);
+    if (!g_na_ptr[device_id]) {
+      hipDeviceProp_t prop;
+      PLR_NA_HIP(hipGetDeviceProperties(&prop, device_id));
+      if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return bad(PLR_ERR_UNSUPPORTED, std::string("device is ") + prop.gcnArchName +
+                                            "; this library carries gfx950 code only");
+      unsigned char* ptr = nullptr;
+      PLR_NA_HIP(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+      if (!ptr) return bad(PLR_ERR_HIP, "hipGetSymbolAddress returned a null address");
+      g_na_num_cu[device_id] = prop.multiProcessorCount;
+      g_na_ptr[device_id] = ptr;
+    }
+    base = g_na_ptr[device_id];
+    num_cu = g_na_num_cu[device_id];
+  }
+  double* s_theta = reinterpret_cast<double*>(base + kNaThetaOff);
+  double* s_loss = reinterpret_cast<double*>(base + kNaLossOff);
+  double* s_part = reinterpret_cast<double*>(base + kNaPartOff);
+
+  // the row pitch is a whole number of chunks, so the variant is the exact
+  // one-wave one for ldx / 128 chunks and no lane reads past a row end
+  plr_plan::Plan pl;
+  if (!plr_plan::plan_width(ldx, pl) || pl.path != plr_plan::kPathFused || pl.pitch != ldx ||
+      !pl.allch || pl.tail_cols != 0 || pl.theta_len > kNaMaxPitch)
+    return bad(PLR_ERR_UNSUPPORTED, "no kernel variant covers this pitch");
+  const Shape* v = &kShapes[pl.variant];
+  const bool grad = true;
+  const pass_fn fn = kFns[pl.variant].fn[grad ? 1 : 0][1];
+  if (!fn || v->wcol != 1) return bad(PLR_ERR_UNSUPPORTED, "kernel variant lacks this instance");
+  const int threads = plr::kWave * v->wcol * v->wrow;
+  int occ = 0;
+  PLR_NA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(fn),
+                                                          threads, 0));
+  if (occ < 1) return bad(PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
+  const int64_t want = ceil_div(ceil_div(n, v->R), v->wrow);
+  int64_t g = std::min<int64_t>((int64_t)num_cu * occ, kNaMaxGrid);
+  if (g > want) g = want;
+  if (g < 1) g = 1;
+  const int grid = (int)g;
+
+  hipLaunchKernelGGL(plr::stage_theta_padded, dim3(2), dim3(256), 0, stream, dtheta, s_theta, d,
+                     pl.theta_len);
+  PLR_NA_HIP(hipGetLastError());
+  if (n > 0) {
+    PassArgs pa;
+    pa.X = dX;
+    pa.y = dy;
+    pa.theta = s_theta;
+    pa.part_g = s_part;
+    pa.part_loss = s_loss;
+    pa.h_out = nullptr;
+    pa.n = n;
+    pa.pitch = ldx;
+    pa.width = ldx;
+    pa.ntiles = ceil_div(n, v->R);
+    pa.nch_rt = pl.nch_rt;
+    pa.tail_cols = 0;
+    pa.loss_mode = flags;
+    pa.identity_link = flags == plr::kLossSquared ? 1 : 0;
+    pa.z_buf = nullptr;
+    pa.z_accumulate = 0;
+    pa.res_in = nullptr;
+    hipLaunchKernelGGL(fn, dim3(grid), dim3(threads), 0, stream, pa);
+    PLR_NA_HIP(hipGetLastError());
+  } else {
+    // empty shard: the one partial the finishing kernel reads starts at zero
+    hipLaunchKernelGGL(plr::fill_zero, dim3(8), dim3(256), 0, stream, s_part, ldx);
+    PLR_NA_HIP(hipGetLastError());
+    hipLaunchKernelGGL(plr::fill_zero, dim3(1), dim3(256), 0, stream, s_loss, (int64_t)1);
+    PLR_NA_HIP(hipGetLastError());
+  }
+  FinishArgs fa;
+  fa.part_g = s_part;
+  fa.part_loss = s_loss;
+  fa.theta = s_theta;
+  fa.out = dout;
+  fa.pitch = ldx;
+  fa.d = d;
+  fa.n = n;
+  fa.nparts = grid;
+  fa.nparts_loss = grid;
+  fa.delta_mode = 0;
+  fa.have_grad = 1;
+  fa.alpha = 0.;
+  fa.coff2 = 0.;
+  fa.theta_rw = nullptr;
+  fa.loss_slot = nullptr;
+  hipLaunchKernelGGL(plr::finish_pass, dim3((int)ceil_div(d, plr::kFinCols)),
+                     dim3(plr::kFinCols * plr::kFinSlices), 0, stream, fa);
+  PLR_NA_HIP(hipGetLastError());
+#undef PLR_NA_HIP
   return PLR_OK;
 }
 

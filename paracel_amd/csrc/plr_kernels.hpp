@@ -772,6 +772,25 @@ __global__ __launch_bounds__(256) void stage_theta(const double* __restrict__ ho
     dev_theta[i] = host_theta[i];
 }
 
+// theta already on the device -> the zero-padded copy the pass reads: entries
+// [d, len) are written as zeros every time, so a buffer that is shared between
+// calls of different widths never leaks an old theta into the pad columns.
+__global__ __launch_bounds__(256) void stage_theta_padded(const double* __restrict__ src,
+                                                          double* __restrict__ dst, int64_t d,
+                                                          int64_t len) {
+  for (int64_t i = threadIdx.x + (int64_t)blockIdx.x * blockDim.x; i < len;
+       i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = i < d ? src[i] : 0.;
+}
+
+// Plain fill with zeros (a kernel, not a memset command: safe inside a
+// captured graph).
+__global__ __launch_bounds__(256) void fill_zero(double* __restrict__ dst, int64_t count) {
+  for (int64_t i = threadIdx.x + (int64_t)blockIdx.x * blockDim.x; i < count;
+       i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = 0.;
+}
+
 struct FinishArgs {
   const double* part_g;   // [nparts][pitch]
   const double* part_loss;  // [nparts]
