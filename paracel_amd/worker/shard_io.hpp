@@ -21,13 +21,15 @@
 //                magic, version, input size and input mtime all match.
 #pragma once
 
+#include <fcntl.h>
 #include <glob.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
+#include <sys/mman.h>
 #include <sys/stat.h>
+#include <unistd.h>
 
-#include <fstream>
 #include <stdexcept>
 #include <string>
 #include <thread>
@@ -70,55 +72,102 @@ inline std::vector<std::string> expand_input(const std::string& name) {
   return out;
 }
 
+// One input file's place in the byte stream formed by all inputs end to end.
+struct FileSpan {
+  std::string path;
+  int64_t begin = 0, end = 0;  // [begin, end) in the stream
+};
+
+inline std::vector<FileSpan> stream_layout(const std::vector<std::string>& files) {
+  std::vector<FileSpan> spans;
+  int64_t pos = 0;
+  for (const std::string& f : files) {
+    struct stat st;
+    if (stat(f.c_str(), &st) != 0 || !S_ISREG(st.st_mode))
+      throw std::runtime_error("cannot open " + f);
+    FileSpan s;
+    s.path = f;
+    s.begin = pos;
+    s.end = pos += (int64_t)st.st_size;
+    spans.push_back(s);
+  }
+  return spans;
+}
+
+// Byte range of the stream that worker `rank` of `np` owns: np equal parts of
+// floor(total / np) bytes, the last one taking the remainder
+// (include/load/partition.hpp:57-86 with one block per worker).
+inline void owned_range(int64_t total, int rank, int np, int64_t& lo, int64_t& hi) {
+  const int64_t part = total / np;
+  lo = (int64_t)rank * part;
+  hi = (rank == np - 1) ? total : lo + part;
+}
+
+// A read-only mapping of one file, released on scope exit.
+class MappedFile {
+ public:
+  explicit MappedFile(const std::string& path, int64_t size) : size_(size) {
+    if (size_ == 0) return;
+    const int fd = open(path.c_str(), O_RDONLY);
+    if (fd < 0) throw std::runtime_error("cannot open " + path);
+    void* p = mmap(nullptr, (size_t)size_, PROT_READ, MAP_PRIVATE, fd, 0);
+    close(fd);
+    if (p == MAP_FAILED) throw std::runtime_error("cannot map " + path);
+    data_ = static_cast<const char*>(p);
+  }
+  ~MappedFile() {
+    if (data_) munmap(const_cast<char*>(data_), (size_t)size_);
+  }
+  MappedFile(const MappedFile&) = delete;
+  MappedFile& operator=(const MappedFile&) = delete;
+  const char* data() const { return data_; }
+
+ private:
+  const char* data_ = nullptr;
+  int64_t size_;
+};
+
+// The lines of one file whose first byte lies in [lo, hi) (file offsets).  A
+// line starts at offset 0 or right after a newline, and runs to the next
+// newline or the end of the file; the one that starts before hi is taken
+// whole even when it runs past hi.  Blank lines are dropped.
+inline void lines_starting_in(const char* text, int64_t size, int64_t lo, int64_t hi,
+                              std::vector<std::string>& out) {
+  if (lo < 0) lo = 0;
+  if (hi > size) hi = size;
+  int64_t pos = lo;
+  if (pos > 0 && text[pos - 1] != '\n') {  // inside a line that belongs to an earlier range
+    const void* nl = memchr(text + pos, '\n', (size_t)(size - pos));
+    if (!nl) return;
+    pos = static_cast<const char*>(nl) - text + 1;
+  }
+  while (pos < hi) {
+    const void* nl = memchr(text + pos, '\n', (size_t)(size - pos));
+    const int64_t stop = nl ? static_cast<const char*>(nl) - text : size;
+    if (stop > pos) out.emplace_back(text + pos, (size_t)(stop - pos));
+    pos = stop + 1;
+  }
+}
+
+// The reference's "linesplit" load (paralg::paracel_load, include/ps.hpp:178-197
+// -> loader::fixload, include/load/loader.hpp:81-96 -> partition.hpp:121-175):
+// worker `rank` gets the lines that start inside its byte range of the stream.
+// Every line of the input goes to exactly one worker, in stream order.  (On
+// input with blank lines the reference stops reading a file at the first one
+// when its range runs on into the next file, and hands them to the parser
+// otherwise; here they are skipped.)
 inline std::vector<std::string> load_lines(const std::string& input, int rank, int np) {
+  if (np < 1 || rank < 0 || rank >= np) throw std::invalid_argument("bad worker rank");
   const std::vector<std::string> files = expand_input(input);
   if (files.empty()) throw std::runtime_error("cannot open " + input);
-  std::vector<long> displs(files.size() + 1, 0);  // byte offset of each file in the union
-  for (size_t i = 0; i < files.size(); ++i) {
-    std::ifstream f(files[i], std::ios::ate);
-    if (!f) throw std::runtime_error("cannot open " + files[i]);
-    displs[i + 1] = displs[i] + (long)f.tellg();
-  }
-  const long sz = displs.back();
-  const long bk = sz / np;
-  const long st = (long)rank * bk;
-  const long en = (rank == np - 1) ? sz : (long)(rank + 1) * bk;
+  const std::vector<FileSpan> spans = stream_layout(files);
+  int64_t lo = 0, hi = 0;
+  owned_range(spans.back().end, rank, np, lo, hi);
   std::vector<std::string> lines;
-  if (st >= en) return lines;
-  size_t fst = 0, fen = 0;  // first and last file the range touches
-  for (size_t i = 0; i < files.size(); ++i) {
-    if (st >= displs[i]) fst = i;
-    if (en > displs[i + 1]) fen = i + 1;
-  }
-  if (fen >= files.size()) fen = files.size() - 1;
-  bool from_file_start = false;
-  for (size_t fi = fst; fi <= fen; ++fi) {
-    long offset = from_file_start ? 0 : st - displs[fi];
-    std::ifstream f(files[fi]);
-    if (offset) {
-      // step back one byte and finish the line in progress: if that byte is
-      // the newline itself, the next line starts exactly at `st` and is ours
-      f.seekg(offset - 1);
-      std::string l;
-      std::getline(f, l);
-      offset += (long)l.size();
-    }
-    if (fi == fen) {
-      while (offset + displs[fi] < en) {
-        std::string l;
-        if (!std::getline(f, l)) break;
-        offset += (long)l.size() + 1;
-        lines.push_back(l);
-      }
-    } else {
-      from_file_start = true;
-      for (;;) {  // to the end of this file (the reference stops at an empty line)
-        std::string l;
-        std::getline(f, l);
-        if (l.empty()) break;
-        lines.push_back(l);
-      }
-    }
+  for (const FileSpan& f : spans) {
+    if (f.end <= lo || f.begin >= hi || f.end == f.begin) continue;  // no byte of it is ours
+    const MappedFile m(f.path, f.end - f.begin);
+    lines_starting_in(m.data(), f.end - f.begin, lo - f.begin, hi - f.begin, lines);
   }
   return lines;
 }

@@ -2,6 +2,8 @@
 //   plr_shard_tool parse <input.csv> <rank> <np>   parse this rank's lines and write the cache
 //   plr_shard_tool info  <input.csv> <rank> <np>   validate the cache; print n d
 //   plr_shard_tool lines <input.csv> <rank> <np>   print the lines this rank owns
+//   plr_shard_tool owners <input> <lo_np> <hi_np>  for every np in [lo_np, hi_np] and every rank:
+//                                                  "np rank line" per owned line
 //   plr_shard_tool selftest <count> <seed> 0       parse_field against std::stod on <count>
 //                                                  random field spellings, bit for bit
 #include <iostream>
@@ -67,6 +69,18 @@ static int selftest(long count, unsigned long long seed) {
 int main(int argc, char** argv) {
   if (argc == 5 && std::string(argv[1]) == "selftest")
     return selftest(atol(argv[2]), strtoull(argv[3], nullptr, 0));
+  if (argc == 5 && std::string(argv[1]) == "owners") {
+    try {
+      for (int np = atoi(argv[3]); np <= atoi(argv[4]); ++np)
+        for (int r = 0; r < np; ++r)
+          for (const std::string& l : plr_ps::load_lines(argv[2], r, np))
+            std::cout << np << " " << r << " " << l << "\n";
+    } catch (const std::exception& e) {
+      std::cerr << e.what() << "\n";
+      return 1;
+    }
+    return 0;
+  }
   if (argc != 5) {
     std::cerr << "usage: plr_shard_tool parse|info|lines <input> <rank> <np>\n";
     return 2;

@@ -82,6 +82,72 @@ def test_directory_and_glob_inputs_are_one_byte_stream(tmp_path, np_):
     assert run("lines", str(d) + "/*.nothing", 0, 1).returncode == 1
 
 
+def _owners_by_definition(blobs, np_):
+    """Brute force of the rule itself: lay the files end to end, cut the stream into np
+    ranges of floor(total/np) bytes (the last takes the rest), and give every non-blank
+    line to the range its FIRST byte falls in.  Lines never span two files."""
+    total = sum(len(b) for b in blobs)
+    part = total // np_
+    owned = [[] for _ in range(np_)]
+    base = 0
+    for b in blobs:
+        pos = 0
+        while pos < len(b):
+            nl = b.find(b"\n", pos)
+            stop = len(b) if nl < 0 else nl
+            if stop > pos:
+                start = base + pos
+                r = np_ - 1 if part == 0 else min(start // part, np_ - 1)
+                owned[r].append(b[pos:stop].decode())
+            pos = stop + 1
+        base += len(b)
+    return owned
+
+
+@pytest.mark.parametrize("case", ["one_file", "three_files", "no_final_newline", "tiny_lines"])
+def test_ownership_rule_by_brute_force_for_np_1_to_99(tmp_path, case):
+    # the reference's own test (test/test_partition.cpp) checks line continuity for
+    # np = 1..99 on one file; here the definition is evaluated directly, byte by byte,
+    # also over several files, files that lack the final newline and one-byte lines
+    rng = np.random.default_rng(len(case))
+    d = tmp_path / "in"
+    d.mkdir()
+
+    def text(n, maxlen):
+        return "".join("".join(rng.choice(list("0123456789.,-e"), size=rng.integers(1, maxlen)))
+                       + "\n" for _ in range(n))
+
+    if case == "one_file":
+        files = {"a.csv": text(300, 40)}
+    elif case == "three_files":
+        files = {"a.csv": text(120, 30), "b.csv": text(5, 200), "c.csv": text(211, 12)}
+    elif case == "no_final_newline":
+        files = {"a.csv": text(50, 25)[:-1], "b.csv": text(70, 25)[:-1], "c.csv": text(3, 9)}
+    else:
+        files = {"a.csv": text(150, 2), "b.csv": "7\n" * 90}
+    for name, t in files.items():
+        (d / name).write_text(t)
+    blobs = [files[k].encode() for k in sorted(files)]   # glob order = sorted names
+    out = run("owners", d, 1, 99)
+    assert out.returncode == 0, out.stderr
+    got = {}
+    for ln in out.stdout.splitlines():
+        a, b, line = ln.split(" ", 2)
+        got.setdefault(int(a), {}).setdefault(int(b), []).append(line)
+    for np_ in range(1, 100):
+        want = _owners_by_definition(blobs, np_)
+        for r in range(np_):
+            assert got.get(np_, {}).get(r, []) == want[r], (case, np_, r)
+
+
+def test_blank_lines_are_dropped(tmp_path):
+    f = tmp_path / "e.csv"
+    f.write_text("1,2,1\n\n3,4,0\n\n\n5,6,1\n")
+    for np_ in (1, 2, 5):
+        got = sum((run("lines", f, r, np_).stdout.splitlines() for r in range(np_)), [])
+        assert got == ["1,2,1", "3,4,0", "5,6,1"]
+
+
 def test_parser_matches_oracle_and_cache_roundtrip(tmp_path, oracle):
     f = tmp_path / "c.csv"
     lines = make_csv(f, 300, 7, 2)
