@@ -6,7 +6,12 @@ synthetic shard that is already resident in HBM: theta goes in from the host,
 the gradient sum and the loss come back to the host.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps 50] [--warmup 5] [--workload NAME]
-                    [--no-cpu-baseline] [--rows N]
+                    [--no-cpu-baseline] [--rows N] [--headline-only]
+
+The line is the headline configuration (1M x 1000).  Unless --workload or
+--headline-only is given, the other configurations (c1, c3, c4, c4b, c5 bare and
+c5 end to end through the parameter server) are timed in the same run, with the
+same steps / warmup, and reported under "per_config".
 
 roofline.achieved = algorithmic bytes per step (X once + y + theta + gradient +
 loss = 8nd + 8n + 16d + 8) / average duration of the streaming kernel, measured
@@ -28,17 +33,54 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 
 # HBM bytes per launch of the streaming kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs, scaled by what the same counters read for a copy kernel of
-# known size; None until measured for that workload.
-MEASURED_TRAFFIC_BYTES = {
-    # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000) KiB per shard_pass dispatch; see profiles/
-    "c2_headline_1m_x_1000": 8056281406,
-    "c3_tall_10m_x_256": 20560480416,
-    "c4_wide_200k_x_16384": 26261496415,
-    "c4b_wide_200k_x_16385": 26287132305,
-    "c5_e2e_2m_x_512": 8210208784,
-    "x_bias_10m_x_257": 21175219596,
+# WRITE_SIZE runs (scaled by what the same counters read for a copy kernel of
+# known size): workload -> (rows, kernel description the figure was measured with,
+# bytes, summary file).  Reported only when rows and kernel match what this run
+# uses, so a changed variant choice yields null instead of a stale figure.
+MEASURED_TRAFFIC = {
+    "c2_headline_1m_x_1000": (
+        1000000, "shard_pass<NCH=8,R=4,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=8 tail=0 pitch=1000 "
+        "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)", 8056281406,
+        "profiles/shard_pass_c2_headline_1m_x_1000.md"),
+    "c3_tall_10m_x_256": (
+        10000000, "shard_pass<NCH=2,R=32,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=2 tail=0 pitch=256 "
+        "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)", 20560480416,
+        "profiles/shard_pass_c3_tall_10m_x_256.md"),
+    "c4_wide_200k_x_16384": (
+        200000, "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=0> nch_rt=16 tail=0 pitch=16384 "
+        "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26261496415,
+        "profiles/shard_pass_c4_wide_200k_x_16384.md"),
+    "c4b_wide_200k_x_16385": (
+        200000, "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=1> nch_rt=16 tail=16 pitch=16400 "
+        "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26287132305,
+        "profiles/shard_pass_c4b_wide_200k_x_16385.md"),
+    "c5_e2e_2m_x_512": (
+        2000000, "shard_pass<NCH=4,R=16,WCOL=1,WROW=2,ALLCH=1,TL=0> nch_rt=4 tail=0 pitch=512 "
+        "grid=512 x 128 threads (occupancy 2 blocks/CU, 256 CUs)", 8210208784,
+        "profiles/shard_pass_c5_e2e_2m_x_512.md"),
+    "x_bias_10m_x_257": (
+        10000000, "shard_pass<NCH=2,R=16,WCOL=1,WROW=4,ALLCH=1,TL=1> nch_rt=2 tail=2 pitch=258 "
+        "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)", 21175219596,
+        "profiles/shard_pass_tail_stage_x_bias_10m_x_257.md"),
 }
+
+# The other configurations a default run times after the headline.
+PER_CONFIG = ["c1_dense_100k_x_100", "c3_tall_10m_x_256", "c4_wide_200k_x_16384",
+              "c4b_wide_200k_x_16385", "c5_e2e_2m_x_512"]
+
+# A one-GPU box gives a job 16 CPUs whatever os.cpu_count() shows there.
+CPU_SHARE = 16
+
+
+def measured_traffic(cfg, kernel_info):
+    ent = MEASURED_TRAFFIC.get(cfg.name)
+    if not ent or ent[0] != cfg.n or ent[1] != kernel_info:
+        return None, None
+    return ent[2], ent[3]
+
+
+def cpu_threads():
+    return max(1, min(CPU_SHARE, os.cpu_count() or 1))
 
 
 def parse_args():
@@ -46,7 +88,11 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=int(os.environ.get("WORLD_SIZE", "1")))
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2_headline_1m_x_1000")
+    ap.add_argument("--workload", default=None,
+                    help="time only this workload (default: the headline c2_headline_1m_x_1000 "
+                         "plus the other configurations under per_config)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="skip the per_config section of a default run")
     ap.add_argument("--rows", type=int, default=0, help="override n (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-rows", type=int, default=0)
@@ -101,37 +147,45 @@ def reference_build_status():
     return "reference dependencies present (reference binary not timed by this script)"
 
 
-def cpu_baseline(cfg, Xs, ys, theta):
+def cpu_model_name():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name"):
+                    return ln.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return ""
+
+
+def cpu_baseline(cfg, Xs, ys, theta, reps1=4, repsp=20):
     """Reference traversal on the host cores: 1 core (tool/lr_serial, prun.py -w 1)
     and P local workers (mpirun -n P bin/lr), on the row sample, scaled to n."""
     from oracle import oracle
 
     m = Xs.shape[0]
-    cores = max(1, min(16, os.cpu_count() or 1))
-    t1, _, tl1, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=1, reps=4)
-    tp, _, tlp, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=cores, reps=20)
+    cores = cpu_threads()
+    t1, _, tl1, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=1, reps=reps1)
+    tp, _, tlp, _ = oracle.baseline_time(Xs, ys, theta, cfg.alpha, cfg.beta, threads=cores,
+                                         reps=repsp)
     scale = cfg.n / float(m)
-    model = ""
-    try:
-        with open("/proc/cpuinfo") as f:
-            for ln in f:
-                if ln.startswith("model name"):
-                    model = ln.split(":", 1)[1].strip()
-                    break
-    except OSError:
-        pass
+    whole = "all %d rows" % m if m == cfg.n else \
+        "first %d of %d rows, time scaled linearly in n" % (m, cfg.n)
     return {
         "value": 1.0 / (tp * scale),
         "unit": "steps/s",
         "cores": cores,
+        "host_cpu_count": os.cpu_count(),
+        "cores_note": "threads used = min(os.cpu_count(), %d): a one-GPU box gives a job a "
+                      "%d-CPU share of its host" % (CPU_SHARE, CPU_SHARE),
         "kind": "port",
-        "sample": "first %d of %d rows (d=%d), gradient traversal lr.cpp:132-138 in the "
-                  "reference's vector<vector<double>> layout, g++ -O3, %d threads as local "
-                  "workers; time scaled linearly in n" % (m, cfg.n, cfg.d, cores),
+        "sample": "%s (d=%d), gradient traversal lr.cpp:132-138 in the reference's "
+                  "vector<vector<double>> layout, g++ -O3, %d threads as local workers"
+                  % (whole, cfg.d, cores),
         "value_1core": 1.0 / (t1 * scale),
         "loss_pass_seconds_1core_scaled": tl1 * scale,
         "loss_pass_seconds_pcore_scaled": tlp * scale,
-        "cpu_model": model,
+        "cpu_model": cpu_model_name(),
         "reference_build": reference_build_status(),
     }
 
@@ -177,13 +231,15 @@ def run_train(a, cfg):
     print(json.dumps(out), flush=True)
 
 
-def run_e2e(a, cfg):
+def run_e2e(a, cfg, rounds=None):
     """steps rounds of read theta -> GPU delta -> bupdate against a real server
     process; final theta against the CPU oracle's multi-worker training."""
     import subprocess
     import tempfile
 
     import numpy as np
+
+    rounds = rounds or a.steps
 
     pkg = os.path.join(ROOT, "paracel_amd")
     if cfg.spec.kind != 0 or cfg.spec.zero_prob != 0.0 or cfg.spec.outlier_mod != 0:
@@ -198,7 +254,7 @@ def run_e2e(a, cfg):
             tout = os.path.join(td, "theta.bin")
             cmd = [os.path.join(pkg, "plr_lr_worker"), "--server_info", info,
                    "--synthetic", "%x,%d,%d,%.17g" % (cfg.seed, cfg.n, cfg.d, cfg.spec.scale),
-                   "--rounds", str(a.steps), "--alpha", "%.17g" % cfg.alpha,
+                   "--rounds", str(rounds), "--alpha", "%.17g" % cfg.alpha,
                    "--beta", "%.17g" % cfg.beta, "--theta0", "zero",
                    "--update_file", os.path.join(pkg, "liblr_update.so"), "--theta_out", tout]
             r = subprocess.run(cmd, capture_output=True, text=True)
@@ -211,7 +267,7 @@ def run_e2e(a, cfg):
         srv.wait()
     out = {
         "metric": "lr_e2e_iters_per_sec", "value": rep["iters_per_sec"], "unit": "iters/s",
-        "n_gpus": 1, "steps": a.steps, "warmup": 0,
+        "n_gpus": 1, "steps": rounds, "warmup": 0,
         "ms_per_step": 1e3 / rep["iters_per_sec"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": {"workload": cfg.name + " via parameter server", "n": cfg.n, "d": cfg.d,
@@ -227,7 +283,7 @@ def run_e2e(a, cfg):
     if not a.no_cpu_baseline:
         from oracle import oracle
 
-        cores = max(1, min(16, os.cpu_count() or 1))
+        cores = cpu_threads()
         X = np.empty((cfg.n, cfg.d))
         y = np.empty(cfg.n)
         step = 262144
@@ -236,15 +292,15 @@ def run_e2e(a, cfg):
             _, y[lo:lo + m] = cfg.rows(lo, m, out=X[lo:lo + m])
         t0 = time.time()
         theta_cpu = oracle.train_dgd_workers(X, y, np.zeros(cfg.d), cfg.alpha, cfg.beta,
-                                             a.steps, cores)
+                                             rounds, cores)
         sec = time.time() - t0
         out["theta_rel_err_vs_cpu"] = float(np.linalg.norm(theta_gpu - theta_cpu) /
                                             np.linalg.norm(theta_cpu))
-        out["cpu_baseline"] = {"value": a.steps / sec, "unit": "iters/s", "cores": cores,
-                               "kind": "port",
+        out["cpu_baseline"] = {"value": rounds / sec, "unit": "iters/s", "cores": cores,
+                               "host_cpu_count": os.cpu_count(), "kind": "port",
                                "sample": "all %d rounds on the full shard, %d local workers "
-                                         "(threads), in-process server add" % (a.steps, cores)}
-    print(json.dumps(out), flush=True)
+                                         "(threads), in-process server add" % (rounds, cores)}
+    return out
 
 
 def run_ps_roundtrip(a):
@@ -275,47 +331,26 @@ def run_ps_roundtrip(a):
     print(json.dumps(out), flush=True)
 
 
-def main():
-    a = parse_args()
-    if a.gpus != 1:
-        print("bench.py measures one GPU's shard: this build has no multi-GPU path "
-              "(run with --gpus 1)", file=sys.stderr)
-        sys.exit(2)
-    if a.ps_roundtrip:
-        run_ps_roundtrip(a)
-        return
-
-    import numpy as np  # noqa: F401
-
+def run_step(a, cfg, with_cpu, full_cpu_sample=False, cpu_reps=(4, 20)):
+    """The bare gradient step on one workload: upload, warm up, time a.steps calls of
+    plr_loss_grad; returns the result record (contract keys + roofline + cpu_baseline)."""
     from paracel_amd import Plr
-    from paracel_amd.datagen import gen
 
-    cfgs = gen.configs()
-    if a.workload not in cfgs:
-        print("unknown workload %s; known: %s" % (a.workload, ", ".join(cfgs)), file=sys.stderr)
-        sys.exit(2)
-    cfg = cfgs[a.workload]
-    if a.rows:
-        cfg = cfg.scaled(a.rows)
-    if a.e2e:
-        run_e2e(a, cfg)
-        return
-    if a.train:
-        run_train(a, cfg)
-        return
     theta = cfg.theta()
-
-    # ~2 GB sample for the CPU leg (bounded: a few seconds per traversal on one core)
     sample_rows = 0
-    if not a.no_cpu_baseline:
-        sample_rows = a.cpu_sample_rows or max(1, min(cfg.n, int(2.0e9 // (8 * cfg.d))))
+    if with_cpu:
+        # bounded CPU leg: ~2 GB of rows (a few seconds per traversal on one core), or
+        # the whole shard where asked (the headline: 8 GB fit the host)
+        sample_rows = a.cpu_sample_rows or (
+            cfg.n if full_cpu_sample else max(1, min(cfg.n, int(2.0e9 // (8 * cfg.d)))))
 
     ctx = Plr(0)
     t0 = time.time()
     Xs, ys = upload(ctx, cfg, keep_rows=sample_rows)
     t_up = time.time() - t0
-    print("# shard %d x %d generated and uploaded in %.1f s; %s" %
-          (cfg.n, cfg.d, t_up, ctx.kernel_info()), file=sys.stderr, flush=True)
+    info = ctx.kernel_info()
+    print("# shard %d x %d generated and uploaded in %.1f s; %s" % (cfg.n, cfg.d, t_up, info),
+          file=sys.stderr, flush=True)
 
     for _ in range(a.warmup):
         ctx.loss_grad(theta)
@@ -334,7 +369,8 @@ def main():
     copy_ceiling = ctx.probe_copy_bandwidth(2 << 30, 5)   # read + written, runtime D2D copy
     bytes_step = cfg.algorithmic_bytes()
     achieved = bytes_step / (kern_ms * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get(cfg.name)
+    whole = bytes_step / (elapsed / a.steps) / 1e9
+    traffic, traffic_src = measured_traffic(cfg, info)
     out = {
         "metric": "lr_gradient_steps_per_sec",
         "value": a.steps / elapsed,
@@ -352,20 +388,90 @@ def main():
                    "step": "plr_loss_grad: theta host->device, fused loss+gradient pass, "
                            "gsum+loss device->host",
                    "lambda": cfg.lam, "alpha": cfg.alpha, "beta": cfg.beta,
-                   "kernel": ctx.kernel_info()},
+                   "kernel": info},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_source": traffic_src,
                      "kernel_ms": kern_ms, "algorithmic_bytes": bytes_step,
-                     "whole_step_gbs": bytes_step / (elapsed / a.steps) / 1e9,
+                     "whole_step_gbs": whole, "whole_step_frac": whole / HBM_PEAK_GBS,
                      "read_ceiling_gbs": read_ceiling,
                      "frac_of_read_ceiling": achieved / read_ceiling,
                      "copy_ceiling_gbs": copy_ceiling},
         "cpu_baseline": None,
         "loss_mean": loss / n,
     }
-    if not a.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, Xs, ys, theta)
+    if with_cpu:
+        out["cpu_baseline"] = cpu_baseline(cfg, Xs, ys, theta, *cpu_reps)
     ctx.close()
+    return out
+
+
+def per_config_entry(rec):
+    """The per_config summary of one bare-step record."""
+    r = rec["roofline"]
+    e = {"steps_per_sec": rec["value"], "ms_per_step": rec["ms_per_step"],
+         "kernel_ms": r["kernel_ms"], "achieved_gbs": r["achieved"], "frac": r["frac"],
+         "whole_step_frac": r["whole_step_frac"], "algorithmic_bytes": r["algorithmic_bytes"],
+         "traffic": r["traffic"], "read_ceiling_gbs": r["read_ceiling_gbs"],
+         "n": rec["config"]["n"], "d": rec["config"]["d"], "kernel_info": rec["config"]["kernel"]}
+    if rec["cpu_baseline"]:
+        c = rec["cpu_baseline"]
+        e["cpu_steps_per_sec"] = c["value"]
+        e["cpu_steps_per_sec_1core"] = c["value_1core"]
+        e["cpu_cores"] = c["cores"]
+        e["cpu_sample"] = c["sample"]
+    return e
+
+
+def main():
+    a = parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU's shard: this build has no multi-GPU path "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if a.ps_roundtrip:
+        run_ps_roundtrip(a)
+        return
+
+    import numpy as np  # noqa: F401
+
+    from paracel_amd.datagen import gen
+
+    cfgs = gen.configs()
+    name = a.workload or "c2_headline_1m_x_1000"
+    if name not in cfgs:
+        print("unknown workload %s; known: %s" % (name, ", ".join(cfgs)), file=sys.stderr)
+        sys.exit(2)
+    cfg = cfgs[name]
+    if a.rows:
+        cfg = cfg.scaled(a.rows)
+    if a.e2e:
+        print(json.dumps(run_e2e(a, cfg)), flush=True)
+        return
+    if a.train:
+        run_train(a, cfg)
+        return
+
+    with_cpu = not a.no_cpu_baseline
+    out = run_step(a, cfg, with_cpu, full_cpu_sample=(a.workload is None and not a.rows))
+    if a.workload is None and not a.headline_only and not a.rows:
+        # the other configurations, same steps / warmup, bounded CPU legs
+        per = {}
+        for other in PER_CONFIG:
+            rec = run_step(a, cfgs[other], with_cpu, cpu_reps=(2, 6))
+            per[other] = per_config_entry(rec)
+        # config 5 as it is defined: 100 rounds through the parameter server
+        e2e = run_e2e(a, cfgs["c5_e2e_2m_x_512"], rounds=100)
+        per["c5_e2e_2m_x_512_via_ps"] = {
+            "iters_per_sec": e2e["value"], "ms_per_iter": e2e["ms_per_step"], "rounds": 100,
+            "gpu_only_iters_per_sec": e2e["gpu_only_iters_per_sec"],
+            "gpu_kernel_ms_per_iter": e2e["gpu_kernel_ms_per_iter"],
+            "theta_rel_err_vs_cpu": e2e["theta_rel_err_vs_cpu"],
+            "final_loss": e2e["final_loss"],
+            "cpu_iters_per_sec": (e2e.get("cpu_baseline") or {}).get("value"),
+            "cpu_cores": (e2e.get("cpu_baseline") or {}).get("cores"),
+            "step": e2e["config"]["step"]}
+        out["per_config"] = per
     print(json.dumps(out), flush=True)
 
 

@@ -85,6 +85,15 @@ const PackedVariant kPacked[] = {
     PLR_PACKED(6, 1, 2, 1),  // pitch 64
 };
 
+// Rows of 65..96 columns: a half-wave per row, G row pairs per tile.
+struct PairVariant {
+  int G, wrow;
+  pass_fn fn[2];  // [grad]
+};
+// 16 rows per tile, two waves per SIMD (sweeps on MI355X: 6.5-7.0 TB/s for
+// every even pitch 66..96; taller tiles and other occupancies lose 5-20 %)
+const PairVariant kPair = {8, 4, {plr::pair_pass<8, 4, 2, false>, plr::pair_pass<8, 4, 2, true>}};
+
 // the column-blocked path's shape: 8 waves x 16 chunks, one row per tile, theta in LDS
 const Shape kBlockShape = {kBlkNch, 1, kBlkWcol, 1, 2, true, 0};
 
@@ -135,6 +144,7 @@ struct plr_ctx {
   bool allch = false;
   int tail_cols = 0;            // columns handled by the variant's tail stage
   const PackedVariant* packed = nullptr;  // d <= 64: packed-row kernel
+  const PairVariant* pair = nullptr;      // 65..96 columns: half-wave rows
   bool blocked = false;         // rows wider than the widest fused variant: column blocks
   double* d_z = nullptr;        // n: blocked rows only, x.theta accumulated over the blocks
   double* d_res = nullptr;      // n: blocked rows only, residual per row
@@ -214,6 +224,7 @@ void free_shape(plr_ctx* c) {
   c->curve_len = 0;
   c->blocked = false;
   c->packed = nullptr;
+  c->pair = nullptr;
   c->tail_cols = 0;
   c->var = nullptr;
   c->fns = nullptr;
@@ -256,6 +267,31 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
              "(occupancy %d blocks/CU, %d CUs)",
              (long long)c->pitch, pv->U, pv->wrow, plr::kWave * pv->U, c->grid, threads, occ,
              c->num_cu);
+    c->info = b;
+    return PLR_OK;
+  }
+  if (pl.path == plr_plan::kPathPair) {
+    const PairVariant* pv = &kPair;
+    const int threads = plr::kWave * pv->wrow;
+    c->pair = pv;
+    c->var = &kBlockShape;  // unused by this path, kept non-null
+    c->nch_rt = 1;
+    int occ = 0, occ2 = 0;
+    PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                   &occ, reinterpret_cast<const void*>(pv->fn[1]), threads, 0));
+    PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                   &occ2, reinterpret_cast<const void*>(pv->fn[0]), threads, 0));
+    if (occ < 1 || occ2 < 1)
+      return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
+    const int64_t ntiles = ceil_div(n, (int64_t)2 * pv->G);
+    const int64_t want = std::max<int64_t>(1, ceil_div(ntiles, pv->wrow));
+    c->grid = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ);
+    c->grid_nograd = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ2);
+    char b[256];
+    snprintf(b, sizeof b,
+             "pair_pass<G=%d,WROW=%d> pitch=%lld, %d rows per tile, grid=%d x %d threads "
+             "(occupancy %d blocks/CU, %d CUs)",
+             pv->G, pv->wrow, (long long)c->pitch, 2 * pv->G, c->grid, threads, occ, c->num_cu);
     c->info = b;
     return PLR_OK;
   }
@@ -444,7 +480,9 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
   const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
   const int grid = grad ? c->grid : c->grid_nograd;
-  const int threads = c->packed ? plr::kWave * c->packed->wrow : plr::kWave * v->wcol * v->wrow;
+  const int threads = c->packed ? plr::kWave * c->packed->wrow
+                      : c->pair ? plr::kWave * c->pair->wrow
+                                : plr::kWave * v->wcol * v->wrow;
 
   PassArgs pa;
   pa.X = c->dX;
@@ -469,6 +507,9 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   if (c->timing) PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
   if (c->packed) {
     hipLaunchKernelGGL(c->packed->fn[grad ? 1 : 0], dim3(grid), dim3(threads), 0, c->stream, pa);
+    PLR_HIP(c, hipGetLastError());
+  } else if (c->pair) {
+    hipLaunchKernelGGL(c->pair->fn[grad ? 1 : 0], dim3(grid), dim3(threads), 0, c->stream, pa);
     PLR_HIP(c, hipGetLastError());
   } else if (!c->blocked) {
     hipLaunchKernelGGL(c->fns->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,

@@ -239,7 +239,10 @@ __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       x[r][c] = v2d{0., 0.};
-      if (rv && (ALLCH || c < w.my_nch))  // uniform
+      // uniform, except that a one-chunk row loads its ragged chunk under the
+      // lane mask: lanes past the row end then request nothing (every load of
+      // the tile sits under the same mask, so the run of loads stays unbroken)
+      if (rv && (ALLCH || c < w.my_nch) && (NCH > 1 || w.ragged_c < 0 || w.lane_in_ragged))
         x[r][c] = load_x(reinterpret_cast<const v2d*>(
             rowp + w.lane_off + (uint32_t)(c * kChunkCols * sizeof(double))));
     }
@@ -697,6 +700,164 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void packed_pass(PassArgs a) {
         s.y += o.y;
       }
       *reinterpret_cast<v2d*>(a.part_g + (int64_t)blockIdx.x * P + 2 * lane) = s;
+    }
+  }
+  {
+    __shared__ double lx[WROW];
+    const double wl = wave_sum(loss_acc);
+    if (lane == 0) lx[wr] = wl;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      double s = 0.;
+#pragma unroll
+      for (int w = 0; w < WROW; ++w) s += lx[w];
+      a.part_loss[blockIdx.x] = s;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Rows of 65..128 columns, two rows per wave instruction.  With one row per
+// load (shard_pass, one chunk) a pass over rows this short is bound by its
+// instruction stream, not by HBM: every load, every multiply-add, every lane
+// exchange and the whole exp/log sequence are issued per row (or per 16 rows
+// with 16 useful lanes) -- about 35 instructions a row, and half of the lanes
+// of most of them past the row end.  Here a half-wave owns a row: lane l works
+// on row 2g + l/32 of pair g and holds the column pairs (2q, 2q+1) and
+// (64+2q, 65+2q), q = l % 32.  A tile is G pairs; the transposing butterfly
+// over the 32 lanes of a half leaves every lane with ONE row of the tile (all
+// 64 lanes evaluate distinct sigmoid / loss terms when G = 32), the residuals
+// travel back inside the half (ds_bpermute) and the rank-1 update runs on the
+// loaded registers.  The second load of a pair fetches columns 64.. of both
+// rows; its lanes past the row end fetch the next row's first bytes (or the
+// slack behind the shard) and take no part in the dot product.
+//
+// Same reference loops as shard_pass (lr.cpp:69-72,132-138,322-330,361-363).
+template <int G, int WROW, int MINW, bool GRAD>
+__global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
+  static_assert((G & (G - 1)) == 0 && G >= 2 && G <= 32, "G pairs per tile, a power of two");
+  constexpr int kHalf = kWave / 2;
+  constexpr int kTileRows = 2 * G;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wr = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int half = lane / kHalf;
+  const int q = lane & (kHalf - 1);
+  const int64_t p = a.pitch;                         // even, 66..128
+  const bool hi_in = kWave + 2 * q < p;              // this lane's second column pair exists
+  const int my_pair = row_of_lane<G>(q & (G - 1));   // pair whose row ends up in this lane
+  const bool owner = q < G;                          // G < 32: lanes q and q + G hold the same row
+
+  const v2d th_lo = *reinterpret_cast<const v2d*>(a.theta + 2 * q);
+  const v2d th_hi = *reinterpret_cast<const v2d*>(a.theta + kWave + 2 * q);  // zero past the row
+  v2d acc_lo = v2d{0., 0.}, acc_hi = v2d{0., 0.};
+  double loss_acc = 0.;
+
+  const int64_t group = (int64_t)blockIdx.x * WROW + wr;
+  const int64_t ngroups = (int64_t)gridDim.x * WROW;
+  const int64_t nfull = a.n / kTileRows;
+  const int64_t ntiles = (a.n + kTileRows - 1) / kTileRows;
+  const uint32_t lane_off = (uint32_t)((half * p + 2 * q) * sizeof(double));
+  const uint32_t pair_bytes = (uint32_t)(2 * p * sizeof(double));
+
+  auto tile_body = [&](int64_t tile, auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
+    const int64_t row0 = tile * kTileRows;
+    const char* base = reinterpret_cast<const char*>(a.X + row0 * p) + lane_off;
+    v2d xl[G], xh[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      xl[g] = xh[g] = v2d{0., 0.};
+      if (FULL || row0 + 2 * g + half < a.n)
+        xl[g] = load_x(reinterpret_cast<const v2d*>(base + g * pair_bytes));
+    }
+    // the second column pair under the lane mask: lanes past the row end
+    // request nothing
+    if (hi_in) {
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+        if (FULL || row0 + 2 * g + half < a.n)
+          xh[g] = load_x(reinterpret_cast<const v2d*>(base + g * pair_bytes + kWave * sizeof(double)));
+    }
+    const int64_t myrow = row0 + 2 * my_pair + half;
+    const bool valid = FULL || myrow < a.n;
+    double yv = 0.;
+    if (valid && a.y) yv = a.y[myrow];
+
+    typename RowVec<G>::type t;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const double lo = fma(xl[g].x, th_lo.x, xl[g].y * th_lo.y);
+      const double hi = fma(xh[g].x, th_hi.x, xh[g].y * th_hi.y);
+      t[g] = lo + hi;  // lanes without a second pair hold zeros there
+    }
+    // transposing butterfly over the 32 lanes of the half
+#pragma unroll
+    for (int s = 0; s < ilog2(G); ++s) {
+      const int cnt = G >> (s + 1);
+      const int m = 1 << s;
+      const bool up = (lane & m) != 0;
+#pragma unroll
+      for (int k = 0; k < cnt; ++k) {
+        const double lo = t[k], hi = t[k + cnt];
+        const double send = up ? lo : hi;
+        const double keep = up ? hi : lo;
+        t[k] = keep + __shfl_xor(send, m, kWave);
+      }
+    }
+    double z = t[0];
+#pragma unroll
+    for (int s = ilog2(G); s < 5; ++s) z += __shfl_xor(z, 1 << s, kWave);
+
+    double h, l;
+    row_terms(z, yv, a.loss_mode, a.identity_link, h, l);
+    const double res = valid ? (h - yv) : 0.;
+    if (a.h_out && valid && owner) a.h_out[myrow] = h;
+    if (valid && owner) loss_acc += l;
+    if (GRAD) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        // the residual of row 2g + half sits in the lane of this half that kept pair g
+        const double rr = __shfl(res, (lane & kHalf) | lane_of_row<G>(g), kWave);
+        acc_lo.x = fma(rr, xl[g].x, acc_lo.x);
+        acc_lo.y = fma(rr, xl[g].y, acc_lo.y);
+        acc_hi.x = fma(rr, xh[g].x, acc_hi.x);
+        acc_hi.y = fma(rr, xh[g].y, acc_hi.y);
+      }
+    }
+  };
+
+  int64_t tile = group;
+#pragma clang loop unroll(disable)
+  for (; tile < nfull; tile += ngroups) tile_body(tile, std::true_type{});
+  if (tile < ntiles) tile_body(tile, std::false_type{});
+
+  if (GRAD) {
+    // the two halves worked on different rows of the same columns
+    acc_lo.x += __shfl_xor(acc_lo.x, kHalf, kWave);
+    acc_lo.y += __shfl_xor(acc_lo.y, kHalf, kWave);
+    acc_hi.x += __shfl_xor(acc_hi.x, kHalf, kWave);
+    acc_hi.y += __shfl_xor(acc_hi.y, kHalf, kWave);
+    __shared__ v2d gx[(WROW > 1) ? (WROW - 1) * kWave : 1];
+    if (WROW > 1) {
+      if (wr > 0 && half == 0) {
+        gx[(wr - 1) * kWave + q] = acc_lo;
+        gx[(wr - 1) * kWave + kHalf + q] = acc_hi;
+      }
+      __syncthreads();
+    }
+    if (wr == 0 && half == 0) {
+      v2d lo = acc_lo, hi = acc_hi;
+#pragma unroll
+      for (int k = 1; k < WROW; ++k) {
+        const v2d ol = gx[(k - 1) * kWave + q], oh = gx[(k - 1) * kWave + kHalf + q];
+        lo.x += ol.x;
+        lo.y += ol.y;
+        hi.x += oh.x;
+        hi.y += oh.y;
+      }
+      double* out = a.part_g + (int64_t)blockIdx.x * p;
+      *reinterpret_cast<v2d*>(out + 2 * q) = lo;
+      if (hi_in) *reinterpret_cast<v2d*>(out + kWave + 2 * q) = hi;
     }
   }
   {

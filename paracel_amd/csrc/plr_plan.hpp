@@ -11,6 +11,7 @@ namespace plr_plan {
 
 constexpr int kChunkCols = 128;          // columns per chunk (a double2 per lane)
 constexpr int64_t kMaxPackedCols = 64;   // up to here: packed rows, power-of-two pitch
+constexpr int64_t kMaxPairPitch = 96;    // up to this pitch: a half-wave per row (pair_pass)
 constexpr int64_t kMaxFusedCols = 19456; // beyond: column blocks, two sweeps over X
 constexpr int kBlkNch = 16, kBlkWcol = 8;
 constexpr int64_t kBlockCols = (int64_t)kBlkNch * kBlkWcol * kChunkCols;  // 16384
@@ -30,7 +31,7 @@ static const Shape kShapes[] = {
 };
 constexpr int kNumShapes = (int)(sizeof(kShapes) / sizeof(kShapes[0]));
 
-enum Path { kPathPacked = 0, kPathFused = 1, kPathBlocked = 2 };
+enum Path { kPathPacked = 0, kPathFused = 1, kPathBlocked = 2, kPathPair = 3 };
 
 struct Plan {
   Path path;
@@ -59,6 +60,13 @@ inline bool plan_width(int64_t d, Plan& p) {
     p.path = kPathPacked;
     p.logp = logp;
     p.pitch = int64_t(1) << logp;
+    p.theta_len = kChunkCols;
+    return true;
+  }
+  if (((d + 1) & ~int64_t(1)) <= kMaxPairPitch) {
+    // 65..96 columns: two rows per wave instruction, even pitch
+    p.path = kPathPair;
+    p.pitch = (d + 1) & ~int64_t(1);
     p.theta_len = kChunkCols;
     return true;
   }

@@ -25,7 +25,7 @@ static void print_plan(int64_t d) {
     printf("d=%lld: no variant\n", (long long)d);
     return;
   }
-  static const char* names[] = {"packed", "fused", "blocked"};
+  static const char* names[] = {"packed", "fused", "blocked", "pair"};
   printf("d=%lld path=%s pitch=%lld theta_len=%lld", (long long)d, names[p.path],
          (long long)p.pitch, (long long)p.theta_len);
   if (p.path == kPathPacked) printf(" logp=%d", p.logp);
@@ -53,10 +53,14 @@ int main(int argc, char** argv) {
     }
     CHECK(p.pitch >= d && p.pitch % 2 == 0, d);
     CHECK(p.theta_len >= p.pitch || p.path == kPathPacked, d);
+    CHECK(p.path != kPathFused || p.pitch > kMaxPairPitch, d);
     if (p.path == kPathPacked) {
       CHECK(d <= kMaxPackedCols && p.logp >= 1 && p.logp <= 6, d);
       CHECK(p.pitch == (int64_t(1) << p.logp) && (p.pitch / 2 < d || d == 1), d);
       CHECK(p.theta_len >= p.pitch, d);
+    } else if (p.path == kPathPair) {
+      CHECK(d > kMaxPackedCols && p.pitch <= kMaxPairPitch && p.pitch - d < 2, d);
+      CHECK(p.theta_len >= kChunkCols, d);  // both column pairs of every lane read theta
     } else if (p.path == kPathBlocked) {
       CHECK(d > kMaxFusedCols && p.pitch % 16 == 0 && p.pitch - d < 16, d);
       CHECK(p.theta_len % kBlockCols == 0 && p.theta_len >= p.pitch, d);

@@ -154,6 +154,14 @@ def configs():
         "x_bias_10m_x_257": Config("x_bias_10m_x_257", 10_000_000, 257, 0x5EED0008, UNIFORM, 1.0,
                                    lam=0.001, outlier_mod=100, outlier_scale=100.0,
                                    theta_scale=0.1),
+        # rows of 65..96 columns at HBM-resident size: the half-wave-per-row kernel
+        "x_short_30m_x_66": Config("x_short_30m_x_66", 30_000_000, 66, 0x5EED0009, NORMAL,
+                                   1.0 / np.sqrt(66), lam=0.01),
+        "x_short_30m_x_72": Config("x_short_30m_x_72", 30_000_000, 72, 0x5EED000A, NORMAL,
+                                   1.0 / np.sqrt(72), lam=0.01),
+        # config 1's shape (the reference tutorial's 100 features) at HBM-resident size
+        "x_c1shape_20m_x_100": Config("x_c1shape_20m_x_100", 20_000_000, 100, 0x5EED000B, NORMAL,
+                                      1.0, lam=0.01, theta0_zero=True),
         # narrow rows: the packed-row kernel (several whole rows per 128-double chunk)
         "x_narrow_30m_x_16": Config("x_narrow_30m_x_16", 30_000_000, 16, 0x5EED0007, NORMAL, 0.25,
                                     lam=0.01),

@@ -35,6 +35,25 @@ def test_parameter_server_round_trip_mode_runs_on_the_host():
             assert out["widths"][d][mode]["bupdate_us"] > 0
 
 
+def test_traffic_table_names_known_workloads_and_committed_summaries():
+    sys.path.insert(0, ROOT)
+    import bench
+    from paracel_amd.datagen import gen
+
+    cfgs = gen.configs()
+    for name, (rows, kernel, nbytes, src) in bench.MEASURED_TRAFFIC.items():
+        assert name in cfgs and cfgs[name].n == rows
+        assert os.path.exists(os.path.join(ROOT, src)), src
+        # counter traffic can only exceed the algorithmic bytes, and not by much
+        assert 1.0 <= nbytes / cfgs[name].algorithmic_bytes() < 1.1
+        # a figure measured with another kernel or another shard size is not reported
+        assert bench.measured_traffic(cfgs[name], kernel) == (nbytes, src)
+        assert bench.measured_traffic(cfgs[name], kernel + " ") == (None, None)
+        assert bench.measured_traffic(cfgs[name].scaled(rows // 2), kernel) == (None, None)
+    for name in bench.PER_CONFIG:
+        assert name in cfgs
+
+
 @pytest.mark.gpu
 def test_one_json_line_with_roofline_and_cpu_baseline():
     r = subprocess.run([sys.executable, BENCH, "--workload", "c2_headline_1m_x_1000", "--rows",
@@ -55,5 +74,8 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert rf["bound"] == "hbm" and rf["peak"] == 8000.0 and rf["unit"] == "GB/s"
     assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-12
     assert 0.3 < rf["frac"] < 1.0
+    assert rf["traffic"] is None          # 200 000 rows: not the shard the counters were read on
+    assert abs(rf["whole_step_frac"] - rf["whole_step_gbs"] / rf["peak"]) < 1e-12
     cb = out["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
+    assert cb["cores"] <= cb["host_cpu_count"] and cb["cores"] <= 16

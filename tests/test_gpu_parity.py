@@ -39,6 +39,8 @@ SHAPES = [
     # several tiles per row group and a partial last tile, for every tile height
     (40003, 256), (20005, 512), (9001, 1000), (6149, 2047), (3077, 4097), (2053, 8193),
     (8195, 100), (515, 16384),
+    # 65..96 columns: a half-wave per row (pair_pass), 16 rows per tile
+    (1, 65), (15, 66), (16, 67), (17, 72), (1000, 80), (4099, 95), (40003, 96), (300, 97),
 ]
 
 
@@ -126,7 +128,8 @@ def test_rows_of_17_to_32_chunks(plr, oracle, gen, chunks):
     assert rel(g2, X2.T @ (0.5 - y)) <= GRAD_TOL
 
 
-@pytest.mark.parametrize("n,d", [(1000, 100), (2051, 1000), (333, 257), (70, 8193), (37, 16385)])
+@pytest.mark.parametrize("n,d", [(1000, 100), (2051, 1000), (333, 257), (70, 8193), (37, 16385),
+                                 (1500, 70)])
 def test_dgd_delta_matches_oracle(plr, oracle, gen, n, d):
     X, y, th = make(gen, n, d)
     plr.set_data(X, y)
@@ -144,7 +147,7 @@ def test_dgd_delta_matches_oracle(plr, oracle, gen, n, d):
     assert rel(delta2, oracle.dgd_delta(X, y, th, 0.001, 0.01)) <= GRAD_TOL
 
 
-@pytest.mark.parametrize("n,d", [(999, 100), (2051, 1000), (130, 4097)])
+@pytest.mark.parametrize("n,d", [(999, 100), (2051, 1000), (130, 4097), (999, 72)])
 def test_calc_loss_and_predict(plr, oracle, gen, n, d):
     X, y, th = make(gen, n, d)
     plr.set_data(X, y)
@@ -160,7 +163,7 @@ def test_calc_loss_and_predict(plr, oracle, gen, n, d):
     assert abs(loss2 - loss) <= 1e-12 * abs(loss)
 
 
-@pytest.mark.parametrize("n,d", [(999, 100), (2051, 1000), (70, 8193)])
+@pytest.mark.parametrize("n,d", [(999, 100), (2051, 1000), (70, 8193), (999, 90)])
 def test_linear_model_pieces(plr, oracle, gen, n, d):
     # the ridge worker's loss and prediction (alg/regression/ridge/ridge.hpp:103-109,130-139)
     # and the least-squares gradient, on the same streaming pass with the identity link
@@ -372,10 +375,11 @@ def test_labels_other_than_one_are_class_zero(plr, oracle, gen):
     assert rel(g, oracle.gsum(X, y, th)) <= GRAD_TOL
 
 
-def test_non_finite_inputs_propagate_like_the_reference(plr, oracle, gen):
+@pytest.mark.parametrize("d", [300, 80, 40])
+def test_non_finite_inputs_propagate_like_the_reference(plr, oracle, gen, d):
     # the reference does no input checking: a NaN or an infinity in a sample poisons
     # exactly the entries IEEE arithmetic says it should, on the device as on the host
-    X, y, th = make(gen, 200, 300)
+    X, y, th = make(gen, 200, d)
     for kind, val in (("nan", np.nan), ("inf", np.inf), ("-inf", -np.inf)):
         Xb = X.copy()
         Xb[17, 5] = val
@@ -517,8 +521,8 @@ def test_device_resident_training_matches_oracle_and_per_round_path(plr, oracle,
     np.testing.assert_array_equal(plr.train_dgd(np.zeros(cfg.d), alpha, beta, 100), theta)
 
 
-@pytest.mark.parametrize("n,d", [(3000, 16), (2000, 257), (1500, 1025), (500, 2500), (300, 4097),
-                                 (200, 16385), (120, 20001)])
+@pytest.mark.parametrize("n,d", [(3000, 16), (2500, 81), (2000, 257), (1500, 1025), (500, 2500),
+                                 (300, 4097), (200, 16385), (120, 20001)])
 def test_device_resident_training_in_every_kernel_family(plr, oracle, gen, n, d):
     # packed rows, tail stage, one wave per row, several waves + tail, column blocks:
     # device-resident rounds give the bits of the host-driven loop, and the oracle's theta
@@ -560,7 +564,8 @@ def test_every_width_up_to_4400_against_numpy(plr):
         assert ok, "d=%d: %s" % (d, plr.kernel_info())
 
 
-@pytest.mark.parametrize("d", [3, 16, 64, 100, 130, 257, 1000, 1025, 2500, 4097, 16385, 20001])
+@pytest.mark.parametrize("d", [3, 16, 64, 66, 95, 100, 130, 257, 1000, 1025, 2500, 4097, 16385,
+                               20001])
 def test_every_row_count_around_the_tile_sizes(plr, d):
     # partial tiles, partial tail loads, fewer rows than row groups: n = 0..139 in every family
     from scipy.special import expit
