@@ -154,6 +154,19 @@ int plr_reset_timing(plr_ctx* ctx);
  * reference. */
 int plr_set_timing(plr_ctx* ctx, int enabled);
 
+/* Tuning and diagnostic switches of a context; no counterpart in the
+ * reference.  Keys:
+ *   "column_blocks_two_sweeps"  value != 0: rows wider than 19456 columns are
+ *        processed in two sweeps over X (dot products, then updates) instead
+ *        of once by cooperating workgroups; applies from the next
+ *        plr_set_data / plr_alloc_data.  Default 0.
+ *   "team_spin_limit"  how many times a workgroup of the one-read wide-row
+ *        pass polls for a partner's partial dot product before it gives up
+ *        (the call then fails with PLR_ERR_HIP instead of hanging).  Default
+ *        4194304; 0 makes every wait give up at once (used to test the
+ *        failure path). */
+int plr_set_option(plr_ctx* ctx, const char* key, int64_t value);
+
 /* Read ceiling of this device, measured on the resident shard: a kernel that
  * only streams X (same access pattern as the fused pass, no arithmetic) is
  * launched `reps` times; reports GB/s.  No counterpart in the reference; used

@@ -36,6 +36,7 @@ SYMBOLS = [
                                         C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_uint]),
     ("plr_synchronize", C.c_int, [_ctx]),
     ("plr_set_timing", C.c_int, [_ctx, C.c_int]),
+    ("plr_set_option", C.c_int, [_ctx, C.c_char_p, C.c_int64]),
     ("plr_probe_copy_bandwidth", C.c_int, [_ctx, C.c_int64, C.c_int, C.POINTER(C.c_double)]),
     ("plr_get_shape", C.c_int, [_ctx, _i64p, _i64p]),
     ("plr_get_timing", C.c_int, [_ctx, _dp, _dp, _i64p]),
@@ -231,6 +232,10 @@ class Plr:
     def set_timing(self, enabled):
         """Timing events on (default) or off (saves 6-8 us per call)."""
         self._check(self._lib.plr_set_timing(self._h, 1 if enabled else 0))
+
+    def set_option(self, key, value):
+        """plr_set_option: "column_blocks_two_sweeps", "team_spin_limit"."""
+        self._check(self._lib.plr_set_option(self._h, key.encode(), int(value)))
 
     def probe_copy_bandwidth(self, nbytes=1 << 30, reps=5):
         """GB/s (read + written) of the runtime's device-to-device copy of nbytes."""

@@ -66,6 +66,22 @@ const pass_fn kBlockDot[2] = {
 const pass_fn kBlockAxpy[2] = {
     plr::shard_pass<kBlkNch, 1, kBlkWcol, 1, 2, true, false, true, plr::kPassAxpy>,
     plr::shard_pass<kBlkNch, 1, kBlkWcol, 1, 2, true, true, true, plr::kPassAxpy>};
+// ... or, when the row fits a team of at most 16 workgroups, read once: each
+// workgroup of a team owns one column block and the partial dot products are
+// exchanged per row.  [grad]
+typedef void (*team_fn)(plr::TeamArgs);
+// three row buffers per wave: the deepest pipeline that leaves the register file unspilled
+#define PLR_TEAM(GRAD, LM) plr::team_pass<plr_plan::kTeamNch, GRAD, plr::LM>
+// [grad][link / loss formula]
+const team_fn kTeam[2][5] = {
+    {PLR_TEAM(false, kTeamLmReference), PLR_TEAM(false, kTeamLmStable),
+     PLR_TEAM(false, kTeamLmNone), PLR_TEAM(false, kTeamLmSquared),
+     PLR_TEAM(false, kTeamLmLinearNone)},
+    {PLR_TEAM(true, kTeamLmReference), PLR_TEAM(true, kTeamLmStable),
+     PLR_TEAM(true, kTeamLmNone), PLR_TEAM(true, kTeamLmSquared),
+     PLR_TEAM(true, kTeamLmLinearNone)}};
+constexpr unsigned kTeamSpinLimit = 1u << 22;  // polls before a wait for a partner gives up
+
 // Narrow rows (d <= 64): power-of-two pitch, several whole rows per chunk.
 struct PackedVariant {
   int logp, U, wrow;
@@ -146,6 +162,14 @@ struct plr_ctx {
   const PackedVariant* packed = nullptr;  // d <= 64: packed-row kernel
   const PairVariant* pair = nullptr;      // 65..96 columns: half-wave rows
   bool blocked = false;         // rows wider than the widest fused variant: column blocks
+  // ... read once by teams of workgroups (team_blocks > 0), else in two sweeps
+  int team_blocks = 0, team_blk_chunks = 0, nteams = 0;
+  unsigned long long* d_zx = nullptr;  // [nteams][4][team_blocks][2] exchange slots, then the
+                                       // status word of the pass
+  int64_t zx_words = 0;
+  unsigned team_spin_limit = kTeamSpinLimit;
+  bool opt_two_sweeps = false;  // plr_set_option("column_blocks_two_sweeps")
+  bool team_check = false;      // a team pass ran since the status word was last read
   double* d_z = nullptr;        // n: blocked rows only, x.theta accumulated over the blocks
   double* d_res = nullptr;      // n: blocked rows only, residual per row
   int64_t theta_len = 0;
@@ -212,6 +236,11 @@ void free_shape(plr_ctx* c) {
   if (c->d_part_loss) (void)hipFree(c->d_part_loss);
   if (c->d_h) (void)hipFree(c->d_h);
   if (c->d_curve) (void)hipFree(c->d_curve);
+  if (c->d_zx) (void)hipFree(c->d_zx);
+  c->d_zx = nullptr;
+  c->team_blocks = c->team_blk_chunks = c->nteams = 0;
+  c->zx_words = 0;
+  c->team_check = false;
   if (c->d_z) (void)hipFree(c->d_z);
   if (c->d_res) (void)hipFree(c->d_res);
   if (c->d_train_out) (void)hipFree(c->d_train_out);
@@ -299,6 +328,33 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
     const int threads = plr::kWave * kBlkWcol;
     c->var = &kBlockShape;
     c->blocked = true;
+    if (pl.team_blocks > 0 && !c->opt_two_sweeps) {
+      // one read of X: teams of team_blocks workgroups, all resident at once;
+      // partners share an XCD, so the grid is a whole number of teams per XCD
+      int tocc = 0, tocc2 = 0;
+      PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                     &tocc, reinterpret_cast<const void*>(kTeam[1][0]), threads, 0));
+      PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                     &tocc2, reinterpret_cast<const void*>(kTeam[0][0]), threads, 0));
+      if (tocc2 < tocc) tocc = tocc2;
+      const int per_xcd = tocc * c->num_cu / plr::kXcds;  // workgroups resident on one XCD
+      const int teams_per_xcd = per_xcd / pl.team_blocks;
+      if (teams_per_xcd >= 1) {
+        c->team_blocks = pl.team_blocks;
+        c->team_blk_chunks = pl.team_blk_chunks;
+        c->nteams = teams_per_xcd * plr::kXcds;
+        c->grid = c->grid_nograd = c->nteams * c->team_blocks;
+        c->zx_words = (int64_t)c->nteams * plr::kTeamSlots * c->team_blocks * 2;
+        char b[256];
+        snprintf(b, sizeof b,
+                 "team_pass<NCH=%d> %d column blocks of %d chunks, %d teams, pitch=%lld "
+                 "grid=%d x %d threads (occupancy %d blocks/CU, %d CUs)",
+                 plr_plan::kTeamNch, c->team_blocks, c->team_blk_chunks, c->nteams,
+                 (long long)c->pitch, c->grid, threads, tocc, c->num_cu);
+        c->info = b;
+        return PLR_OK;
+      }
+    }
     int occ = 0, occ2 = 0;
     PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
                    &occ, reinterpret_cast<const void*>(kBlockAxpy[0]), threads, 0));
@@ -369,7 +425,9 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d) {
   PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)c->theta_len * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_g, (size_t)c->grid * c->pitch * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_loss, (size_t)gmax * sizeof(double)));
-  if (c->blocked && n > 0) {
+  if (c->team_blocks > 0) {
+    PLR_HIP(c, hipMalloc(&c->d_zx, (size_t)(c->zx_words + 1) * sizeof(unsigned long long)));
+  } else if (c->blocked && n > 0) {
     PLR_HIP(c, hipMalloc(&c->d_z, (size_t)n * sizeof(double)));
     PLR_HIP(c, hipMalloc(&c->d_res, (size_t)n * sizeof(double)));
   }
@@ -515,6 +573,34 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     hipLaunchKernelGGL(c->fns->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
                        c->stream, pa);
     PLR_HIP(c, hipGetLastError());
+  } else if (c->team_blocks > 0) {
+    // exchange slots and the status word start at zero (sequence number 0 = empty)
+    hipLaunchKernelGGL(plr::fill_zero, dim3(16), dim3(256), 0, c->stream,
+                       reinterpret_cast<double*>(c->d_zx), c->zx_words + 1);
+    PLR_HIP(c, hipGetLastError());
+    plr::TeamArgs ta;
+    ta.X = c->dX;
+    ta.y = pa.y;
+    ta.theta = c->d_theta;
+    ta.part_g = c->d_part_g;
+    ta.part_loss = c->d_part_loss;
+    ta.h_out = pa.h_out;
+    ta.n = c->n;
+    ta.pitch = c->pitch;
+    ta.nblk = c->team_blocks;
+    ta.nteams = c->nteams;
+    ta.blk_chunks = c->team_blk_chunks;
+    ta.nch_rt = c->team_blk_chunks / plr::kTeamWaves;
+    ta.zeros = c->d_theta + c->theta_len - plr::kChunkCols;  // the padding never changes
+    ta.zx = c->d_zx;
+    ta.status = reinterpret_cast<unsigned*>(c->d_zx + c->zx_words);
+    ta.spin_limit = c->team_spin_limit;
+    const int lm = pa.identity_link ? (pa.loss_mode == plr::kLossSquared ? plr::kTeamLmSquared
+                                                                         : plr::kTeamLmLinearNone)
+                                    : (int)pa.loss_mode;  // kLossReference/Stable/None = 0/1/2
+    hipLaunchKernelGGL(kTeam[grad ? 1 : 0][lm], dim3(grid), dim3(threads), 0, c->stream, ta);
+    PLR_HIP(c, hipGetLastError());
+    c->team_check = true;
   } else if (c->n > 0) {
     // sweep 1: z = x.theta, one launch per column block, accumulated in d_z
     pa.z_buf = c->d_z;
@@ -571,8 +657,8 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     fa.pitch = c->pitch;
     fa.d = c->d;
     fa.n = c->n;
-    fa.nparts = grid;
-    fa.nparts_loss = grid;
+    fa.nparts = c->team_blocks > 0 ? c->nteams : grid;  // a team shares one row of partials
+    fa.nparts_loss = fa.nparts;
     fa.delta_mode = (kind == kPassDelta) ? (train_round >= 0 ? 2 : 1) : 0;
     fa.have_grad = grad ? 1 : 0;
     fa.alpha = alpha;
@@ -607,6 +693,20 @@ int account_timing(plr_ctx* c) {
   return PLR_OK;
 }
 
+// After the stream has drained: did a workgroup of a team pass give up waiting
+// for a partner?  Then the results of that pass are not the shard's.
+int check_team_status(plr_ctx* c) {
+  if (!c->team_check) return PLR_OK;
+  c->team_check = false;
+  unsigned long long st = 0;
+  PLR_HIP(c, hipMemcpy(&st, c->d_zx + c->zx_words, sizeof st, hipMemcpyDeviceToHost));
+  if ((unsigned)st != 0u)
+    return fail(c, PLR_ERR_HIP,
+                "team pass: a workgroup gave up waiting for its partners' partial dot products "
+                "(are all workgroups of the grid resident?); results discarded");
+  return PLR_OK;
+}
+
 // One synchronous pass: theta in, kernels, results in the mapped host buffer.
 int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
              double alpha, double beta) {
@@ -623,6 +723,8 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
   if (rc != PLR_OK) return rc;
   // (measured: hipStreamSynchronize returns ~7 us sooner than a hipStreamQuery poll loop)
   PLR_HIP(c, hipStreamSynchronize(c->stream));
+  rc = check_team_status(c);
+  if (rc != PLR_OK) return rc;
   return account_timing(c);
 }
 
@@ -751,6 +853,8 @@ int plr_train_dgd(plr_ctx* c, double* theta, double alpha, double beta, int roun
   PLR_HIP(c, hipMemcpyAsync(c->h_theta, c->d_theta, (size_t)c->d * sizeof(double),
                             hipMemcpyDeviceToHost, c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
+  rc = check_team_status(c);
+  if (rc != PLR_OK) return rc;
   memcpy(theta, c->h_theta, (size_t)c->d * sizeof(double));
   if (loss_curve)
     PLR_HIP(c, hipMemcpy(loss_curve, c->d_curve, (size_t)rounds * sizeof(double),
@@ -863,6 +967,21 @@ int plr_get_timing(const plr_ctx* c, double* last_ms, double* sum_ms, int64_t* l
   if (sum_ms) *sum_ms = c->sum_ms;
   if (launches) *launches = c->launches;
   return PLR_OK;
+}
+
+int plr_set_option(plr_ctx* c, const char* key, int64_t value) {
+  if (!c) return PLR_ERR_INVALID;
+  if (!key) return fail(c, PLR_ERR_INVALID, "key must not be NULL");
+  if (strcmp(key, "team_spin_limit") == 0) {
+    if (value < 0 || value > 0xffffffffLL) return fail(c, PLR_ERR_INVALID, "spin limit out of range");
+    c->team_spin_limit = (unsigned)value;
+    return PLR_OK;
+  }
+  if (strcmp(key, "column_blocks_two_sweeps") == 0) {
+    c->opt_two_sweeps = value != 0;  // takes effect at the next plr_set_data / plr_alloc_data
+    return PLR_OK;
+  }
+  return fail(c, PLR_ERR_INVALID, std::string("unknown option ") + key);
 }
 
 int plr_set_timing(plr_ctx* c, int enabled) {

@@ -874,6 +874,256 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Rows wider than the fused variants hold (19456 columns), read ONCE.  A team
+// of B workgroups shares every row it processes: workgroup b of the team owns
+// column block b -- 8 waves side by side, theta of the block in LDS, the
+// block's gradient accumulators in registers, one row per step.  What a row
+// needs from the other blocks is one number, its partial dot product.  Each
+// workgroup publishes its partial in global memory and picks up the others';
+// all B workgroups add the B partials in block order, so they arrive at the
+// same bits and the team behaves like one very wide workgroup.
+//
+// Software pipeline, per workgroup, at step t:
+//     look for the partners' partials of row t - 1 (published a step ago, so
+//       the first look nearly always finds them)
+//     request row t + 1 into the buffer row t - 2 has left
+//     dot product of row t (requested a whole step ago), publish it
+//     residual of row t - 1, rank-1 update from the registers that still hold it
+// so neither the exchange nor HBM latency stalls the stream: three row
+// buffers of NCH chunks per wave rotate.
+//
+// The exchange needs no fence: a partial travels as two 64-bit words, each
+// carrying 32 bits of the double and the 32-bit sequence number of its row
+// (never 0; the slots are zeroed before every launch), written and read with
+// relaxed device-scope atomics -- a word is valid exactly when its sequence
+// number is the expected one.  Four slots per team rotate: a workgroup that
+// has just published row t + 1 cannot be more than three rows ahead of what a
+// partner still has to read (to get there it needed the partner's row t - 1,
+// which that partner published only after reading row t - 2).  All workgroups
+// of the grid must be resident at once (the host sizes the grid to the
+// device); should a partner never show up, the wait gives up after spin_limit
+// polls, raises status[0], and every workgroup then runs to its end without
+// waiting -- the host reports the pass as failed.
+//
+// Same reference loops as shard_pass (lr.cpp:69-72,132-138,322-330,361-363).
+constexpr int kXcds = 8;        // workgroups are dealt to the XCDs round-robin
+constexpr int kTeamWaves = 8;
+constexpr int kTeamSlots = 4;
+constexpr int kTeamMaxBlocks = 16;
+
+struct TeamArgs {
+  const double* X;
+  const double* y;
+  const double* theta;       // zero-padded to nblk * blk_chunks * 128 entries
+  const double* zeros;       // 128 doubles of zeros (what an unowned chunk slot reads)
+  double* part_g;            // [nteams][pitch]
+  double* part_loss;         // [nteams]
+  double* h_out;             // n, or nullptr
+  int64_t n, pitch;
+  int nblk;                  // B: column blocks = workgroups per team (<= kTeamMaxBlocks)
+  int nteams;                // grid = nteams * nblk, nteams a multiple of kXcds
+  int blk_chunks;            // 128-column chunks per block (a multiple of 8)
+  int nch_rt;                // chunks per wave = blk_chunks / 8  (<= NCH)
+  unsigned long long* zx;    // [nteams][kTeamSlots][nblk][2] exchange slots
+  unsigned* status;          // [0]: set when a wait gave up
+  unsigned spin_limit;
+};
+
+// the link / loss formula as a compile-time constant: the loop then carries
+// the polynomial coefficients of one formula instead of all of them (they are
+// hoisted into registers, two per coefficient)
+enum : int {
+  kTeamLmReference = 0,   // sigmoid, -log h / -log(1-h)
+  kTeamLmStable = 1,      // sigmoid, log1p(exp(-|z|)) form
+  kTeamLmNone = 2,        // sigmoid, no loss
+  kTeamLmSquared = 3,     // identity link, (z - y)^2
+  kTeamLmLinearNone = 4,  // identity link, no loss
+};
+
+template <int NCH, bool GRAD, int LM>
+__global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
+  constexpr int D = 3;  // row buffers: rows t - 1, t and t + 1
+  constexpr unsigned kLoss = LM == kTeamLmReference ? kLossReference
+                             : LM == kTeamLmStable  ? kLossStable
+                             : LM == kTeamLmSquared ? kLossSquared
+                                                    : kLossNone;
+  constexpr int kIdentity = (LM == kTeamLmSquared || LM == kTeamLmLinearNone) ? 1 : 0;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  // partners share an XCD (and with it an L2): consecutive workgroup ids go
+  // to consecutive XCDs, so the team's members are kXcds apart
+  const int xcd = blockIdx.x % kXcds, k = blockIdx.x / kXcds;
+  const int blk = k % a.nblk;
+  const int team = (k / a.nblk) * kXcds + xcd;
+
+  const int64_t total_chunks = (a.pitch + kChunkCols - 1) / kChunkCols;
+  const int64_t c0 = (int64_t)blk * a.blk_chunks + (int64_t)wave * a.nch_rt;  // my first chunk
+  int64_t blk_end = (int64_t)(blk + 1) * a.blk_chunks;
+  if (blk_end > total_chunks) blk_end = total_chunks;
+  int64_t left = blk_end - c0;
+  const int my_nch = (int)(left < 0 ? 0 : (left > a.nch_rt ? a.nch_rt : left));
+  // the row's last chunk may be ragged (the pitch is a multiple of 16, not of 128)
+  const int rag_cols = (int)(a.pitch % kChunkCols);
+  const int ragged_c =
+      (rag_cols != 0 && my_nch > 0 && c0 + my_nch == total_chunks) ? my_nch - 1 : -1;
+  const bool lane_in_ragged = 2 * lane < rag_cols;
+
+  __shared__ v2d th_lds[kTeamWaves * NCH * kWave];
+  __shared__ double zw[2][kTeamWaves];        // per-wave partial dots, double-buffered
+  __shared__ double zp[2][kTeamMaxBlocks];    // the team's partials of a row, double-buffered
+  v2d* thl = th_lds + wave * NCH * kWave + lane;
+  v2d acc[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    acc[c] = v2d{0., 0.};
+    // (a slot beyond nch_rt reads the page of zeros: a scalar select, no branch)
+    const double* tp = (c < a.nch_rt) ? a.theta + (c0 + c) * kChunkCols : a.zeros;
+    thl[c * kWave] = *reinterpret_cast<const v2d*>(tp + 2 * lane);
+  }
+  double loss_acc = 0.;
+  bool gave_up = false;
+
+  // Uniform base + 32-bit lane offset: no address registers per chunk.  A chunk
+  // slot this wave does not own (c >= my_nch: the last block of an uneven
+  // split) reads a page of zeros instead -- a scalar select of the base, so the
+  // loop body has no branch per chunk.  The ragged chunk is loaded whole; its
+  // lanes past the row end (the next row's bytes) are dropped in the dot
+  // product and never stored.
+  const char* xwave = reinterpret_cast<const char*>(a.X + c0 * kChunkCols);
+  const char* zeros = reinterpret_cast<const char*>(a.zeros);
+  const uint32_t lane_off = (uint32_t)(lane * sizeof(v2d));
+  const int64_t row_bytes = a.pitch * (int64_t)sizeof(double);
+  const int64_t myrows = a.n > team ? (a.n - team + a.nteams - 1) / a.nteams : 0;
+
+  v2d X[D][NCH];
+  auto request = [&](int64_t i, v2d (&buf)[NCH]) {  // row i of this team -> buf
+    const char* rp = xwave + (team + i * a.nteams) * row_bytes;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const char* base = (c < my_nch) ? rp + c * (int)(kChunkCols * sizeof(double)) : zeros;
+      buf[c] = load_x(reinterpret_cast<const v2d*>(base + lane_off));
+    }
+  };
+
+  auto step = [&](int64_t t, auto phase_tag) {
+    constexpr int PH = decltype(phase_tag)::value;      // t mod 3
+    constexpr int PREV = (PH + 2) % 3;                  // buffer of row t - 1
+    constexpr int NEXT = (PH + 1) % 3;                  // buffer of row t - 2: refilled with t + 1
+    const int par = (int)(t & 1);
+    const bool have_row = t < myrows;                   // uniform
+    const bool have_prev = t >= 1;                      // uniform
+
+    // Wave 0 collects the partials of row t - 1 (its own included: one code
+    // path) with vector loads, and vector loads return in issue order: the
+    // first look is requested BEFORE the next row, so it is not queued behind
+    // X; any further look comes after it, at the pace rows arrive.
+    const bool poller = have_prev && wave == 0 && lane < a.nblk;
+    const unsigned seq = (unsigned)t;  // sequence number of row t - 1
+    const unsigned long long* pslot =
+        a.zx + ((int64_t)(team * kTeamSlots + (int)((t + kTeamSlots - 1) % kTeamSlots)) * a.nblk +
+                (poller ? lane : 0)) * 2;
+    unsigned long long w0 = 0, w1 = 0;
+    if (poller) {
+      w0 = __hip_atomic_load(pslot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      w1 = __hip_atomic_load(pslot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("" ::: "memory");
+    if (t + 1 < myrows) request(t + 1, X[NEXT]);
+    asm volatile("" ::: "memory");
+
+    if (have_row) {
+      double s0 = 0., s1 = 0.;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const v2d th = thl[c * kWave];
+        const bool drop = (c == ragged_c) && !lane_in_ragged;
+        s0 = fma(drop ? 0. : X[PH][c].x, th.x, s0);
+        s1 = fma(drop ? 0. : X[PH][c].y, th.y, s1);
+      }
+      const double wsum = wave_sum(s0 + s1);
+      if (lane == 0) zw[par][wave] = wsum;
+    }
+    __syncthreads();
+    if (have_row && threadIdx.x == 0) {
+      double zb = 0.;
+#pragma unroll
+      for (int w = 0; w < kTeamWaves; ++w) zb += zw[par][w];
+      unsigned long long* slot =
+          a.zx + ((int64_t)(team * kTeamSlots + (int)(t % kTeamSlots)) * a.nblk + blk) * 2;
+      const unsigned long long bits = (unsigned long long)__double_as_longlong(zb);
+      const unsigned long long tag = (unsigned long long)(unsigned)(t + 1) << 32;
+      __hip_atomic_store(slot, tag | (bits & 0xffffffffull), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(slot + 1, tag | (bits >> 32), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (poller) {
+      unsigned spins = 0;
+      while ((unsigned)(w0 >> 32) != seq || (unsigned)(w1 >> 32) != seq) {
+        if (gave_up || spins >= a.spin_limit ||
+            ((spins & 63u) == 63u &&
+             __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
+          gave_up = true;
+          __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        ++spins;
+        __builtin_amdgcn_s_sleep(2);
+        w0 = __hip_atomic_load(pslot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        w1 = __hip_atomic_load(pslot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      zp[par][lane] = __longlong_as_double((long long)((w0 & 0xffffffffull) | (w1 << 32)));
+    }
+    __syncthreads();
+    if (have_prev) {
+      const int64_t row = team + (t - 1) * a.nteams;
+      const double yv = a.y ? a.y[row] : 0.;
+      double z = 0.;
+      for (int b = 0; b < a.nblk; ++b) z += zp[par][b];
+      double h, l;
+      row_terms(z, yv, kLoss, kIdentity, h, l);
+      const double res = h - yv;
+      if (blk == 0 && threadIdx.x == 0) {
+        loss_acc += l;
+        if (a.h_out) a.h_out[row] = h;
+      }
+      if (GRAD) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+          acc[c].x = fma(res, X[PREV][c].x, acc[c].x);
+          acc[c].y = fma(res, X[PREV][c].y, acc[c].y);
+        }
+      }
+    }
+  };
+
+  // Row 0 is requested up front; step t requests row t + 1 first thing.
+  // Steps 0 .. myrows: the last one only finishes row myrows - 1.
+  if (myrows > 0) {
+    request(0, X[0]);
+    const int64_t nsteps = myrows + 1;
+    int64_t t = 0;
+#pragma clang loop unroll(disable)
+    for (; t + 3 <= nsteps; t += 3) {
+      step(t, std::integral_constant<int, 0>{});
+      step(t + 1, std::integral_constant<int, 1>{});
+      step(t + 2, std::integral_constant<int, 2>{});
+    }
+    if (t < nsteps) step(t++, std::integral_constant<int, 0>{});
+    if (t < nsteps) step(t++, std::integral_constant<int, 1>{});
+  }
+
+  if (GRAD) {
+    double* out = a.part_g + (int64_t)team * a.pitch + c0 * kChunkCols + 2 * lane;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+      if (c < my_nch && (c != ragged_c || lane_in_ragged))
+        *reinterpret_cast<v2d*>(out + (int64_t)c * kChunkCols) = acc[c];
+  }
+  if (blk == 0 && threadIdx.x == 0) a.part_loss[team] = loss_acc;
+}
+
 // Pure streaming read of a buffer with shard_pass's access pattern (a wave
 // takes contiguous 8 KiB tiles, interleaved over the grid) and next to no
 // arithmetic: what it sustains is the read ceiling the fused pass is up

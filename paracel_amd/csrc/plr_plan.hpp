@@ -15,6 +15,8 @@ constexpr int64_t kMaxPairPitch = 96;    // up to this pitch: a half-wave per ro
 constexpr int64_t kMaxFusedCols = 19456; // beyond: column blocks, two sweeps over X
 constexpr int kBlkNch = 16, kBlkWcol = 8;
 constexpr int64_t kBlockCols = (int64_t)kBlkNch * kBlkWcol * kChunkCols;  // 16384
+constexpr int kMaxTeamBlocks = 16;       // column blocks a team of workgroups may span
+constexpr int kTeamNch = 8;              // chunks per wave the team kernel is built for
 constexpr int kAlwaysOneWave = 16;       // up to here no several-waves variant is considered
 constexpr int kMaxRowChunks = 32;        // widest one-wave row
 
@@ -45,6 +47,10 @@ struct Plan {
   int nch_rt;         // chunks per wave actually used (<= the variant's NCH)
   bool allch;         // every wave of the row uses exactly NCH chunks
   int tail_cols;      // columns handled by the variant's tail stage (0: none)
+  // column-blocked path, one read of X: a team of team_blocks workgroups per
+  // row, each owning team_blk_chunks chunks (0 blocks: too wide, two sweeps)
+  int team_blocks;
+  int team_blk_chunks;
 };
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -76,6 +82,18 @@ inline bool plan_width(int64_t d, Plan& p) {
     p.nch_rt = kBlkNch;
     // theta padded so that the last (narrower) block still reads whole slabs
     p.theta_len = ceil_div(p.pitch, kBlockCols) * kBlockCols;
+    // the row's chunks dealt evenly to the fewest workgroups that can hold
+    // them, each block a whole number of chunks per wave
+    const int64_t chunks = ceil_div(p.pitch, kChunkCols);
+    const int64_t blocks = ceil_div(chunks, (int64_t)kBlkWcol * kTeamNch);
+    if (blocks <= kMaxTeamBlocks) {
+      p.team_blocks = (int)blocks;
+      p.team_blk_chunks = (int)(ceil_div(ceil_div(chunks, blocks), kBlkWcol) * kBlkWcol);
+      const int64_t need = blocks * p.team_blk_chunks * kChunkCols;
+      if (need > p.theta_len) p.theta_len = need;
+    }
+    // one more chunk of padding: the page of zeros an unowned chunk slot reads
+    p.theta_len += kChunkCols;
     return true;
   }
   p.path = kPathFused;

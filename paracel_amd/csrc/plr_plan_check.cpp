@@ -44,7 +44,7 @@ int main(int argc, char** argv) {
     return 0;
   }
   std::vector<int64_t> used(kNumShapes, 0);
-  const int64_t kMaxD = 70000;
+  const int64_t kMaxD = 140000;
   for (int64_t d = 1; d <= kMaxD; ++d) {
     Plan p;
     if (!plan_width(d, p)) {
@@ -63,7 +63,18 @@ int main(int argc, char** argv) {
       CHECK(p.theta_len >= kChunkCols, d);  // both column pairs of every lane read theta
     } else if (p.path == kPathBlocked) {
       CHECK(d > kMaxFusedCols && p.pitch % 16 == 0 && p.pitch - d < 16, d);
-      CHECK(p.theta_len % kBlockCols == 0 && p.theta_len >= p.pitch, d);
+      CHECK(p.theta_len >= p.pitch + kChunkCols, d);  // a whole chunk of zeros behind theta
+      if (p.team_blocks) {
+        const int64_t chunks = ceil_div(p.pitch, kChunkCols);
+        CHECK(p.team_blocks >= 2 && p.team_blocks <= kMaxTeamBlocks, d);
+        CHECK(p.team_blk_chunks % kBlkWcol == 0 && p.team_blk_chunks / kBlkWcol <= kTeamNch, d);
+        CHECK((int64_t)p.team_blocks * p.team_blk_chunks >= chunks, d);            // covers the row
+        CHECK((int64_t)(p.team_blocks - 1) * p.team_blk_chunks < chunks, d);       // no empty block
+        CHECK(p.theta_len >=
+                  (int64_t)p.team_blocks * p.team_blk_chunks * kChunkCols + kChunkCols, d);
+      } else {
+        CHECK(ceil_div(p.pitch, kChunkCols) > (int64_t)kMaxTeamBlocks * kBlkWcol * kTeamNch, d);
+      }
     } else {
       CHECK(d > kMaxPackedCols && d <= kMaxFusedCols, d);
       CHECK(p.variant >= 0 && p.variant < kNumShapes, d);

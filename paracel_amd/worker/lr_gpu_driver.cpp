@@ -58,6 +58,7 @@ static std::map<std::string, std::string> parse_flat_json(const std::string& pat
     if (i >= s.size() || s[i] != ':') throw std::invalid_argument("cfg: expected ':'");
     ++i;
     skip();
+    if (i >= s.size()) throw std::invalid_argument("cfg: value missing");
     if (s[i] == '"') {
       kv[key] = str();
     } else {

@@ -213,6 +213,9 @@ inline void dec(Reader& r, std::vector<double>& v) {
   else if (t == 0xdc) n = r.be(2);
   else if (t == 0xdd) n = r.be(4);
   else throw std::runtime_error("msgpack: not an array");
+  // every element takes at least one byte: a length the field cannot hold is
+  // refused before anything is allocated for it
+  if ((size_t)(r.end - r.p) < n) throw std::runtime_error("msgpack: array longer than its field");
   v.resize(n);
   // all-float64 arrays (what a packed vector<double> always is) in one pass;
   // anything else (integers or float32 among the elements) element by element

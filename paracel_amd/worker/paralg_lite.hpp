@@ -5,14 +5,24 @@
 // process, one thread; REQ sockets are created lazily per op family and
 // strictly alternate send/recv like kvclt's (client.hpp:541-561).
 //
-// Worker-to-worker collectives are MPI in the reference (ps.hpp:890-899);
-// this build runs one worker per GPU box, so paracel_sync() is a no-op and
-// the all-reduces over workers are identities.  A multi-worker build links
-// the reference's own Comm instead.
+// Worker-to-worker collectives are MPI in the reference (paracel_sync =
+// MPI_Barrier, ps.hpp:890-892; Comm::allreduce = MPI_Allreduce(SUM),
+// utils/comm.hpp:629-636).  Here the workers are plain processes (one shard
+// each, sharing the GPU of the box), so the same two collectives run over what
+// every worker already has a connection to -- server 0's tables:
+//   barrier    every worker adds 1 to the integer "plr_sync_<k>" (incr_int on
+//              the ssp port) and waits until it reads worker_sz (pull_int);
+//              k counts this worker's barriers, and all workers call them in
+//              the same order, as MPI requires too
+//   allreduce  every worker pushes its value under "plr_ar_<k>_<rank>",
+//              barrier, then pulls all worker_sz values and adds them in rank
+//              order -- the same bits on every worker
+// With one worker both are no-ops.
 #pragma once
 
 #include <stdio.h>
 #include <sys/stat.h>
+#include <unistd.h>
 #include <zmq.h>
 
 #include <fstream>
@@ -105,6 +115,15 @@ class kvclt {
     bool stat = true;
     const bool r = req(4, paste({pack<std::string>("push_int"), pack(key), pack(v)}), stat);
     return r && stat;
+  }
+  // client.hpp:469-480, :495-501
+  bool incr_int(const std::string& key, int delta) {
+    bool stat = false;
+    const bool r = req(4, paste({pack<std::string>("incr_int"), pack(key), pack(delta)}), stat);
+    return r && stat;
+  }
+  bool pull_int(const std::string& key, int& val) {
+    return req(4, paste({pack<std::string>("pull_int"), pack(key)}), val);
   }
   bool contains(const std::string& key) {
     bool v = false;
@@ -227,11 +246,40 @@ class paralg {
   bool paracel_bupdate(const std::string& key, const std::vector<double>& delta) {
     return srv(key).bupdate_drop(key, delta);
   }
-  void paracel_sync() {}                       // ps.hpp:890-892 (MPI_Barrier; 1 worker)
+  // ps.hpp:890-892 (MPI_Barrier there): returns once every worker has arrived
+  void paracel_sync() {
+    if (nworker_ <= 1) return;
+    const std::string key = "plr_sync_" + std::to_string(sync_count_++);
+    if (!kvm_[0]->incr_int(key, 1)) throw std::runtime_error("paracel_sync: incr_int failed");
+    int arrived = 0;
+    for (unsigned spins = 0;; ++spins) {
+      if (kvm_[0]->pull_int(key, arrived) && arrived >= nworker_) break;
+      usleep(spins < 64 ? 20 : 200);
+    }
+  }
   size_t get_worker_id() const { return rank_; }
   size_t get_worker_size() const { return nworker_; }
-  template <class T>
-  void allreduce(T&) const {}                  // comm.hpp:629-636 MPI_SUM over 1 worker
+  // comm.hpp:629-636 (MPI_Allreduce, MPI_SUM): v becomes the sum over all workers
+  void allreduce(double& v) {
+    if (nworker_ <= 1) return;
+    const std::string base = "plr_ar_" + std::to_string(reduce_count_++) + "_";
+    if (!kvm_[0]->push(base + std::to_string(rank_), v))
+      throw std::runtime_error("allreduce: push failed");
+    paracel_sync();
+    double sum = 0.;
+    for (int r = 0; r < nworker_; ++r) {
+      double part = 0.;
+      if (!kvm_[0]->pull(base + std::to_string(r), part))
+        throw std::runtime_error("allreduce: a worker's value is missing");
+      sum += part;
+    }
+    v = sum;
+  }
+  void allreduce(int& v) {
+    double d = (double)v;  // exact: counts of rows
+    allreduce(d);
+    v = (int)d;
+  }
 
   // ps.hpp:983-1017 / :1308: "<output><prefix><rank>" (truncated, not
   // appended, as with the reference's default append_flag), std::to_string
@@ -267,6 +315,7 @@ class paralg {
     return *kvm_[kvm_.size() == 1 ? 0 : std::hash<std::string>()(key) % kvm_.size()];
   }
   int rank_, nworker_;
+  long sync_count_ = 0, reduce_count_ = 0;
   void* zctx_ = nullptr;
   std::vector<std::unique_ptr<kvclt> > kvm_;
 };

@@ -181,12 +181,19 @@ def test_linear_model_pieces(plr, oracle, gen, n, d):
     assert abs(loss2 - want) <= 1e-12 * want
 
 
-@pytest.mark.parametrize("n,d", [(19, 19457), (300, 33000), (1030, 20001), (64, 65536)])
-def test_rows_wider_than_the_fused_kernels(plr, oracle, gen, n, d):
-    # past 19456 columns the row is processed in column blocks, two sweeps over X
-    print("case n=%d d=%d" % (n, d), flush=True)
+@pytest.mark.parametrize("two_sweeps", [0, 1])
+@pytest.mark.parametrize("n,d", [(19, 19457), (300, 33000), (1030, 20001), (64, 65536),
+                                 (700, 32768), (515, 24577), (40, 131072), (12, 140000),
+                                 (3, 20000), (2100, 20016)])
+def test_rows_wider_than_the_fused_kernels(plr, oracle, gen, n, d, two_sweeps):
+    # past 19456 columns the row is processed in column blocks: by teams of workgroups that
+    # exchange partial dot products (X read once; up to 16 blocks of 8192 columns), or in two
+    # sweeps over X
+    print("case n=%d d=%d two_sweeps=%d" % (n, d, two_sweeps), flush=True)
     X, y, th = make(gen, n, d)
+    plr.set_option("column_blocks_two_sweeps", two_sweeps)
     plr.set_data(X, y)
+    assert ("team_pass" in plr.kernel_info()) == (not two_sweeps and d <= 131072)
     print(plr.kernel_info(), flush=True)
     g, loss, n_out = plr.loss_grad(th)
     assert n_out == n
@@ -203,6 +210,32 @@ def test_rows_wider_than_the_fused_kernels(plr, oracle, gen, n, d):
     assert np.max(np.abs(plr.predict(th) - oracle.predict(X, th))) <= 1e-14
     t5 = plr.train_dgd(np.zeros(d), 0.1 / n, 0.005, 5)
     assert rel(t5, oracle.train_dgd(X, y, np.zeros(d), 0.1 / n, 0.005, 5)) <= 1e-10
+
+
+def test_wide_row_exchange_gives_up_instead_of_hanging(plr, oracle, gen):
+    # a workgroup that never hears from its partners must not spin for ever: with the poll
+    # limit at 0 every wait that does not find its partial at the first look gives up, the
+    # kernel runs to its end and the call reports the failure (a pass in which every first
+    # look happens to succeed is correct and also accepted)
+    from paracel_amd import PlrError
+
+    X, y, th = make(gen, 600, 20001)
+    plr.set_data(X, y)
+    assert "team_pass" in plr.kernel_info()
+    g_ref = oracle.gsum(X, y, th)
+    plr.set_option("team_spin_limit", 0)
+    try:
+        g, _, _ = plr.loss_grad(th)
+        assert rel(g, g_ref) <= GRAD_TOL
+        print("every first look succeeded", flush=True)
+    except PlrError as e:
+        assert e.code == -2 and "gave up waiting" in str(e)
+    # the context is usable again once the limit is back
+    plr.set_option("team_spin_limit", 1 << 22)
+    g, _, _ = plr.loss_grad(th)
+    assert rel(g, g_ref) <= GRAD_TOL
+    with pytest.raises(PlrError):
+        plr.set_option("no_such_option", 1)
 
 
 NARROW = [(n, d) for d in (1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 48, 63, 64)
