@@ -85,6 +85,18 @@ int plr_loss_grad(plr_ctx* ctx, const double* theta, double* gsum,
 int plr_dgd_delta(plr_ctx* ctx, const double* theta, double alpha, double beta,
                   double* delta, double* loss_sum);
 
+/* The same round for the linear model (identity link instead of the sigmoid):
+ * delta = alpha*X^T(y - X theta) - 2*alpha*beta*n*theta, i.e. the update
+ * expression of the ridge worker, alg/regression/ridge/ridge.hpp:79-84
+ * (coff1 = alpha*(y - x.theta); t = coff1*x[i] - coff2*theta[i]), summed over
+ * the shard at a FIXED theta.  The reference's ridge trainer applies that
+ * expression sample by sample, changing theta inside the row loop
+ * (ridge.hpp:78-86); this is its full-batch form, as lr.cpp:132-138 is for
+ * logistic regression.  loss_sum (nullable) receives sum_i (x_i.theta - y_i)^2
+ * (ridge.hpp:103-109). */
+int plr_dgd_delta_linear(plr_ctx* ctx, const double* theta, double alpha, double beta,
+                         double* delta, double* loss_sum);
+
 /* `rounds` full-batch rounds with theta kept on the device: each round is
  * lr.cpp:125-138 (delta at the current theta) followed by the reducer's
  * theta += delta (update.cpp:26-32) -- the single-process training loop of

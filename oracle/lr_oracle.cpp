@@ -214,6 +214,37 @@ void oracle_lsq_gsum(const double* X, int64_t n, int64_t d, int64_t ldx,
   }
 }
 
+void oracle_ridge_delta(const double* X, int64_t n, int64_t d, int64_t ldx,
+                        const double* y, const double* theta, double alpha,
+                        double beta, double* delta) {
+  const double coff2 = 2. * beta * alpha;
+  for (int64_t i = 0; i < d; ++i) delta[i] = 0.;
+  for (int64_t k = 0; k < n; ++k) {
+    const double* x = X + k * ldx;
+    const double coff1 = alpha * (y[k] - dot_seq(x, theta, d));
+    for (int64_t i = 0; i < d; ++i) {
+      double t = coff1 * x[i] - coff2 * theta[i];
+      delta[i] += t;
+    }
+  }
+}
+
+void oracle_ridge_train_workers(const double* X, int64_t n, int64_t d, int64_t ldx,
+                                const double* y, double* theta, double alpha,
+                                double beta, int rounds, int workers) {
+  if (workers < 1) workers = 1;
+  vector<vector<double> > delta(workers, vector<double>(d));
+  for (int rd = 0; rd < rounds; ++rd) {
+    for (int w = 0; w < workers; ++w) {
+      const int64_t lo = n * w / workers, hi = n * (w + 1) / workers;
+      oracle_ridge_delta(X + lo * ldx, hi - lo, d, ldx, y + lo, theta, alpha, beta,
+                         delta[w].data());
+    }
+    for (int w = 0; w < workers; ++w)
+      for (int64_t i = 0; i < d; ++i) theta[i] = theta[i] + delta[w][i];
+  }
+}
+
 void oracle_gsum_hp(const double* X, int64_t n, int64_t d, int64_t ldx,
                     const double* y, const double* theta, double* gsum) {
   vector<long double> acc(d, 0.L);

@@ -108,6 +108,22 @@ void oracle_predict_linear(const double* X, int64_t n, int64_t d, int64_t ldx,
 void oracle_lsq_gsum(const double* X, int64_t n, int64_t d, int64_t ldx,
                      const double* y, const double* theta, double* gsum);
 
+/* The ridge worker's update expression (ridge.hpp:79-84: coff1 = alpha*(y -
+ * x.theta); t = coff1*x[i] - coff2*theta[i], coff2 = 2*beta*alpha) summed over
+ * the rows at a FIXED theta: delta[i] += t, row order, from 0.0.  This is the
+ * full-batch form of that expression (what lr.cpp:132-138 is for logistic
+ * regression); the reference's own ridge trainer instead adds t to theta
+ * inside the row loop (ridge.hpp:78-86) and is not restated here. */
+void oracle_ridge_delta(const double* X, int64_t n, int64_t d, int64_t ldx,
+                        const double* y, const double* theta, double alpha,
+                        double beta, double* delta);
+/* `rounds` rounds of that batch delta with P workers over contiguous row
+ * shards and the server-side add of update.cpp:26-32 (ridge's update.cpp is
+ * the same element-wise sum), in worker order. */
+void oracle_ridge_train_workers(const double* X, int64_t n, int64_t d, int64_t ldx,
+                                const double* y, double* theta, double alpha,
+                                double beta, int rounds, int workers);
+
 /* long-double arbiters: same formulas, every sum and exp/log in 80-bit. */
 void oracle_gsum_hp(const double* X, int64_t n, int64_t d, int64_t ldx,
                     const double* y, const double* theta, double* gsum);

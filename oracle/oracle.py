@@ -44,6 +44,11 @@ def load():
         L.oracle_train_dgd.argtypes = shp + [_dp, _dp, C.c_double, C.c_double, C.c_int]
         L.oracle_train_dgd_workers.restype = None
         L.oracle_train_dgd_workers.argtypes = shp + [_dp, _dp, C.c_double, C.c_double, C.c_int, C.c_int]
+        L.oracle_ridge_delta.restype = None
+        L.oracle_ridge_delta.argtypes = shp + [_dp, _dp, C.c_double, C.c_double, _dp]
+        L.oracle_ridge_train_workers.restype = None
+        L.oracle_ridge_train_workers.argtypes = shp + [_dp, _dp, C.c_double, C.c_double, C.c_int,
+                                                       C.c_int]
         L.oracle_dgd_delta_hp.restype = None
         L.oracle_dgd_delta_hp.argtypes = shp + [_dp, _dp, C.c_double, C.c_double, _dp]
         L.oracle_local_parser.restype = C.c_int64
@@ -141,6 +146,23 @@ def lsq_gsum(X, y, theta):
     out = np.empty(d)
     load().oracle_lsq_gsum(_p(X), n, d, d, _p(y), _p(theta), _p(out))
     return out
+
+
+def ridge_delta(X, y, theta, alpha, beta):
+    X, n, d = _shape(X)
+    y, theta = _c(y), _c(theta)
+    out = np.empty(d)
+    load().oracle_ridge_delta(_p(X), n, d, d, _p(y), _p(theta), alpha, beta, _p(out))
+    return out
+
+
+def ridge_train_workers(X, y, theta0, alpha, beta, rounds, workers=1):
+    X, n, d = _shape(X)
+    y = _c(y)
+    theta = np.array(theta0, dtype=np.float64, copy=True)
+    load().oracle_ridge_train_workers(_p(X), n, d, d, _p(y), _p(theta), alpha, beta, rounds,
+                                      workers)
+    return theta
 
 
 def theta_update(a, b):

@@ -62,10 +62,12 @@ def build_plan_check():
 def build_worker():
     """Host side of the worker path (g++): parameter-server process, reducer
     plugin, GPU LR worker, shard tool ->
-    paracel_amd/{plr_ps_server,liblr_update.so,plr_lr_worker,plr_shard_tool,plr_ps_roundtrip}"""
+    paracel_amd/{plr_ps_server,liblr_update.so,plr_lr_worker,plr_ridge_worker,plr_shard_tool,
+    plr_ps_roundtrip,plr_comm_check}"""
     _run(["make", "-B", "-C", os.path.join(_HERE, "worker")])
     return [os.path.join(_HERE, f) for f in ("plr_ps_server", "liblr_update.so", "plr_lr_worker",
-                                             "plr_shard_tool", "plr_ps_roundtrip")]
+                                             "plr_ridge_worker", "plr_shard_tool",
+                                             "plr_ps_roundtrip", "plr_comm_check")]
 
 
 def build_all():

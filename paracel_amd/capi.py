@@ -28,6 +28,7 @@ SYMBOLS = [
     ("plr_set_data_chunk", C.c_int, [_ctx, C.c_int64, C.c_int64, _dp, C.c_int64, _dp]),
     ("plr_loss_grad", C.c_int, [_ctx, _dp, _dp, _dp, _i64p, C.c_uint]),
     ("plr_dgd_delta", C.c_int, [_ctx, _dp, C.c_double, C.c_double, _dp, _dp]),
+    ("plr_dgd_delta_linear", C.c_int, [_ctx, _dp, C.c_double, C.c_double, _dp, _dp]),
     ("plr_train_dgd", C.c_int, [_ctx, _dp, C.c_double, C.c_double, C.c_int, _dp]),
     ("plr_calc_loss", C.c_int, [_ctx, _dp, _dp, _i64p, C.c_uint]),
     ("plr_predict", C.c_int, [_ctx, _dp, _dp]),
@@ -187,6 +188,16 @@ class Plr:
         self._check(self._lib.plr_dgd_delta(self._h, _p(theta), alpha, beta, _p(delta),
                                             C.byref(loss) if want_loss else None))
         return delta, (loss.value if want_loss else None)
+
+    def dgd_delta_linear(self, theta, alpha, beta):
+        """(delta, squared-loss sum) of the linear model's full-batch round."""
+        d = self.shape[1]
+        theta = _vec(theta, d, "theta")
+        delta = np.empty(d, dtype=np.float64)
+        loss = C.c_double()
+        self._check(self._lib.plr_dgd_delta_linear(self._h, _p(theta), alpha, beta, _p(delta),
+                                                   C.byref(loss)))
+        return delta, loss.value
 
     def train_dgd(self, theta0, alpha, beta, rounds, want_curve=False):
         """theta after `rounds` device-resident rounds (and the per-round loss sums)."""

@@ -827,6 +827,19 @@ int plr_dgd_delta(plr_ctx* c, const double* theta, double alpha, double beta,
   return PLR_OK;
 }
 
+int plr_dgd_delta_linear(plr_ctx* c, const double* theta, double alpha, double beta,
+                         double* delta, double* loss_sum) {
+  if (!c) return PLR_ERR_INVALID;
+  if (!delta) return fail(c, PLR_ERR_INVALID, "delta must not be NULL");
+  // the squared-loss formula selects the identity link; its loss term costs
+  // one multiply per row, so it is always evaluated
+  int rc = run_pass(c, kPassDelta, theta, plr::kLossSquared, alpha, beta);
+  if (rc != PLR_OK) return rc;
+  memcpy(delta, c->h_out, (size_t)c->d * sizeof(double));
+  if (loss_sum) *loss_sum = c->h_out[c->d];
+  return PLR_OK;
+}
+
 int plr_train_dgd(plr_ctx* c, double* theta, double alpha, double beta, int rounds,
                   double* loss_curve) {
   if (!c) return PLR_ERR_INVALID;

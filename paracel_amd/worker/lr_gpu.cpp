@@ -12,8 +12,8 @@ logistic_regression_gpu::logistic_regression_gpu(
     const std::string& hosts_dct_str, const std::string& _input, const std::string& output,
     const std::string& update_file_name, const std::string& update_func_name,
     const std::string& method, int _rounds, double _alpha, double _beta, bool _debug,
-    int device_id)
-    : paralg(hosts_dct_str, output, _rounds),
+    int device_id, int _worker_id, int _worker_sz)
+    : paralg(hosts_dct_str, output, _rounds, _worker_id, _worker_sz),
       input(_input),
       update_file(update_file_name),
       update_func(update_func_name),

@@ -23,7 +23,8 @@ class logistic_regression_gpu : public paralg {
                           const std::string& output, const std::string& update_file_name,
                           const std::string& update_func_name, const std::string& method = "dgd",
                           int _rounds = 1, double _alpha = 0.002, double _beta = 0.1,
-                          bool _debug = false, int device_id = 0);
+                          bool _debug = false, int device_id = 0, int worker_id = 0,
+                          int worker_sz = 1);
   virtual ~logistic_regression_gpu();
 
   // lr.cpp:76-93: "f1,...,fk,label" -> [1.0, f1..fk] and label

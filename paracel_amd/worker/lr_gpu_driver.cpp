@@ -10,6 +10,10 @@
 // file, runs the rounds against the parameter server and prints one JSON line
 // with the end-to-end and GPU-only rates; --theta_out writes the final theta
 // as raw doubles.
+//
+// Where the reference takes rank and size from MPI (lr_driver.cpp:36-37, one
+// process per worker under mpirun), --worker_id R --worker_sz W name this
+// process's place among W plain worker processes that share the server.
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -21,66 +25,17 @@
 #include <sstream>
 
 #include "../datagen/plr_gen.h"
+#include "driver_util.hpp"
 #include "lr_gpu.hpp"
 
 using plr_ps::logistic_regression_gpu;
-
-// Flat JSON object of strings, numbers and booleans (what demo_cfg.json holds).
-static std::map<std::string, std::string> parse_flat_json(const std::string& path) {
-  std::ifstream f(path);
-  if (!f) throw std::invalid_argument("cannot open cfg file " + path);
-  std::stringstream ss;
-  ss << f.rdbuf();
-  const std::string s = ss.str();
-  std::map<std::string, std::string> kv;
-  size_t i = 0;
-  auto skip = [&]() { while (i < s.size() && strchr(" \t\r\n,", s[i])) ++i; };
-  auto str = [&]() {
-    std::string o;
-    ++i;  // opening quote
-    while (i < s.size() && s[i] != '"') {
-      if (s[i] == '\\' && i + 1 < s.size()) ++i;
-      o.push_back(s[i++]);
-    }
-    ++i;
-    return o;
-  };
-  skip();
-  if (i >= s.size() || s[i] != '{') throw std::invalid_argument("cfg: expected '{'");
-  ++i;
-  for (;;) {
-    skip();
-    if (i >= s.size()) throw std::invalid_argument("cfg: unterminated object");
-    if (s[i] == '}') break;
-    if (s[i] != '"') throw std::invalid_argument("cfg: expected a key");
-    const std::string key = str();
-    skip();
-    if (i >= s.size() || s[i] != ':') throw std::invalid_argument("cfg: expected ':'");
-    ++i;
-    skip();
-    if (i >= s.size()) throw std::invalid_argument("cfg: value missing");
-    if (s[i] == '"') {
-      kv[key] = str();
-    } else {
-      size_t j = i;
-      while (j < s.size() && !strchr(",}\r\n \t", s[j])) ++j;
-      kv[key] = s.substr(i, j - i);
-      i = j;
-    }
-  }
-  return kv;
-}
-
-static const std::string& need(const std::map<std::string, std::string>& kv, const char* k) {
-  auto it = kv.find(k);
-  if (it == kv.end()) throw std::invalid_argument(std::string("cfg key missing: ") + k);
-  return it->second;
-}
+using plr_ps::need;
+using plr_ps::parse_flat_json;
 
 int main(int argc, char** argv) {
   std::string server_info, cfg_file, synthetic, theta_out, theta0 = "random", update_file,
                                                            update_func = "lr_theta_update";
-  int rounds = 100, device = 0;
+  int rounds = 100, device = 0, worker_id = 0, worker_sz = 1;
   double alpha = 0.002, beta = 0.1;
   for (int i = 1; i < argc; ++i) {
     std::string a = argv[i], v;
@@ -102,6 +57,8 @@ int main(int argc, char** argv) {
     else if (a == "--update_file") update_file = v;
     else if (a == "--update_func") update_func = v;
     else if (a == "--device") device = atoi(v.c_str());
+    else if (a == "--worker_id") worker_id = atoi(v.c_str());
+    else if (a == "--worker_sz") worker_sz = atoi(v.c_str());
     else {
       std::cerr << "[options]\n\t--server_info\n\t--cfg_file\n";
       return 1;
@@ -115,7 +72,7 @@ int main(int argc, char** argv) {
       if (sscanf(synthetic.c_str(), "%llx,%lld,%lld,%lf", &seed, &n, &d, &scale) != 4)
         throw std::invalid_argument("--synthetic wants SEEDHEX,N,D,SCALE");
       logistic_regression_gpu lr(server_info, "", "", update_file, update_func, "dgd", rounds,
-                                 alpha, beta, false, device);
+                                 alpha, beta, false, device, worker_id, worker_sz);
       {
         plr_gen_spec sp = {seed, PLR_GEN_NORMAL, 0, scale, 0.0, 1.0};
         std::vector<double> X((size_t)n * d), y(n), ts(d);
@@ -143,22 +100,19 @@ int main(int argc, char** argv) {
                                need(kv, "update_file"), need(kv, "update_func"),
                                need(kv, "method"), atoi(need(kv, "rounds").c_str()),
                                atof(need(kv, "alpha").c_str()), atof(need(kv, "beta").c_str()),
-                               need(kv, "debug") == "true", device);
-    if (theta0 == "zero") {
-      // width is known after the parse; solve() asks for theta0 later, so parse here once
-      std::ifstream f(need(kv, "training_input"));
-      std::string first;
-      std::getline(f, first);
-      size_t k = 0;
-      for (char c : first) k += (c == ',');
-      lr.set_theta0(std::vector<double>(k + 1, 0.));
-    }
+                               need(kv, "debug") == "true", device, worker_id, worker_sz);
+    if (theta0 == "zero")
+      lr.set_theta0(std::vector<double>(plr_ps::csv_row_width(need(kv, "training_input")), 0.));
     lr.solve();
     std::cout.precision(17);
     std::cout << "final loss: " << lr.calc_loss() << std::endl;
     if (kv.count("test_input") && !kv["test_input"].empty()) lr.test(kv["test_input"]);
     if (kv.count("predict_input") && !kv["predict_input"].empty()) lr.predict(kv["predict_input"]);
     lr.dump_result();
+    if (!theta_out.empty() && worker_id == 0) {
+      std::ofstream o(theta_out, std::ios::binary);
+      o.write((const char*)lr.get_theta().data(), lr.get_theta().size() * sizeof(double));
+    }
   } catch (const std::exception& e) {
     std::cerr << e.what() << std::endl;
     return 1;

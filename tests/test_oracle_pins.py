@@ -190,6 +190,30 @@ def test_ridge_pieces_against_numpy(oracle):
     assert oracle.ridge_loss_sum(X, oracle.predict_linear(X, th), th) == 0.0
 
 
+def test_ridge_batch_delta_and_training(oracle):
+    # the batch form of ridge.hpp:79-84: delta = alpha X^T(y - X theta) - 2 alpha beta n theta
+    X, _, th = rand_case(400, 13, 21)
+    y = np.random.default_rng(22).normal(size=400)
+    n = 400
+    alpha, beta = 3.0 / n, 0.02
+    want = alpha * (X.T @ (y - X @ th)) - 2 * alpha * beta * n * th
+    assert rel(oracle.ridge_delta(X, y, th, alpha, beta), want) <= 1e-13
+    # X = 0: only the L2 term, n times; theta = 0: only the data term
+    assert rel(oracle.ridge_delta(np.zeros((50, 13)), y[:50], th, alpha, beta),
+               -2 * alpha * beta * 50 * th) <= 1e-14
+    assert rel(oracle.ridge_delta(X, y, np.zeros(13), alpha, beta), alpha * (X.T @ y)) <= 1e-13
+    # a dropped sign or a transposed operand fails this: delta vanishes exactly at the ridge
+    # solution (X^T X + 2 beta n I) theta = X^T y, and training contracts towards it
+    star = np.linalg.solve(X.T @ X + 2 * beta * n * np.eye(13), X.T @ y)
+    assert np.linalg.norm(oracle.ridge_delta(X, y, star, alpha, beta)) <= 1e-13
+    t = oracle.ridge_train_workers(X, y, np.zeros(13), alpha, beta, 400, 1)
+    assert rel(t, star) <= 1e-9
+    # shards add up: W workers give the single worker's theta to rounding
+    for w in (2, 3, 7):
+        assert rel(oracle.ridge_train_workers(X, y, np.zeros(13), alpha, beta, 25, w),
+                   oracle.ridge_train_workers(X, y, np.zeros(13), alpha, beta, 25, 1)) <= 1e-13
+
+
 def test_theta_update_is_elementwise_add(oracle):
     a, b = np.array([1.23, -4.0, 1e300]), np.array([3.21, 4.0, 1e300])
     np.testing.assert_array_equal(oracle.theta_update(a, b), a + b)   # test_proxy.cpp:45-54: 1.23+3.21

@@ -239,3 +239,29 @@ def test_worker_client_round_trips_against_both_servers():
             for b in th.tobytes():
                 h = ((h ^ b) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
             assert l["theta_fnv1a"] == "%016x" % h
+
+
+@pytest.mark.parametrize("W", [1, 2, 3, 5])
+def test_worker_collectives_over_the_server_tables(W):
+    # paracel_sync (MPI_Barrier in the reference, ps.hpp:890-892) and the worker
+    # all-reduce (comm.hpp:629-636) as W plain processes run them: every round a
+    # barrier, a double and an int all-reduce with known sums, and a write that every
+    # other worker must find after the next barrier
+    _need_host_binaries()
+    tool = os.path.join(PKG, "plr_comm_check")
+    if not os.path.exists(tool):
+        subprocess.run(["make", "-C", os.path.join(PKG, "worker"),
+                        os.path.join("..", "plr_comm_check")], check=True)
+    p, info = _start_server(True)
+    try:
+        procs = [subprocess.Popen([tool, "--server_info", info, "--worker_id", str(r),
+                                   "--worker_sz", str(W), "--rounds", "30"],
+                                  stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+                 for r in range(W)]
+        for r, q in enumerate(procs):
+            out, err = q.communicate(timeout=60)
+            assert q.returncode == 0, err
+            assert out.strip() == "ok %d" % r
+    finally:
+        p.kill()
+        p.wait()
