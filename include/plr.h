@@ -61,8 +61,9 @@ void plr_destroy(plr_ctx* ctx);
 int plr_set_data(plr_ctx* ctx, const double* X, int64_t n, int64_t d,
                  int64_t ldx, const double* y);
 
-/* Streaming form of the same: reserve an n x d shard, then fill row ranges
- * in any order (each row exactly once before the first compute call). */
+/* Streaming form of the same: reserve an n x d shard (zero-filled), then fill
+ * row ranges in any order; rows never sent stay zero rows with label 0.
+ * ldx is the caller's row pitch, as in plr_set_data. */
 int plr_alloc_data(plr_ctx* ctx, int64_t n, int64_t d);
 int plr_set_data_chunk(plr_ctx* ctx, int64_t row0, int64_t nrows,
                        const double* X, int64_t ldx, const double* y);

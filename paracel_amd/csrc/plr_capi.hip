@@ -11,6 +11,7 @@
 #include <algorithm>
 #include <mutex>
 #include <string>
+#include <thread>
 
 #include "plr_kernels.hpp"
 #include "plr_plan.hpp"
@@ -80,6 +81,7 @@ const team_fn kTeam[2][5] = {
     {PLR_TEAM(true, kTeamLmReference), PLR_TEAM(true, kTeamLmStable),
      PLR_TEAM(true, kTeamLmNone), PLR_TEAM(true, kTeamLmSquared),
      PLR_TEAM(true, kTeamLmLinearNone)}};
+constexpr int64_t kHostPredictCols = 192;  // from this pitch on predictions go straight to host
 constexpr unsigned kTeamSpinLimit = 1u << 22;  // polls before a wait for a partner gives up
 
 // Narrow rows (d <= 64): power-of-two pitch, several whole rows per chunk.
@@ -177,6 +179,10 @@ struct plr_ctx {
   double* d_part_g = nullptr;   // grid x pitch
   double* d_part_loss = nullptr;  // max(grid, grid_nograd)
   double* d_h = nullptr;        // n (predict), lazily allocated
+  double* h_pred = nullptr;     // n, pinned + device-mapped: where wide shards put predictions
+  double* h_pred_dev = nullptr;
+  void* out_stage = nullptr;    // pinned staging of copy_rows_out, lazily allocated
+  hipStream_t out_stream[4] = {nullptr, nullptr, nullptr, nullptr};
   double* up_stage[2] = {nullptr, nullptr};  // pinned repack buffers for pitched uploads
   hipEvent_t up_done[2] = {nullptr, nullptr};
   size_t up_stage_bytes = 0;
@@ -235,6 +241,8 @@ void free_shape(plr_ctx* c) {
   if (c->d_part_g) (void)hipFree(c->d_part_g);
   if (c->d_part_loss) (void)hipFree(c->d_part_loss);
   if (c->d_h) (void)hipFree(c->d_h);
+  if (c->h_pred) (void)hipHostFree(c->h_pred);
+  c->h_pred = c->h_pred_dev = nullptr;
   if (c->d_curve) (void)hipFree(c->d_curve);
   if (c->d_zx) (void)hipFree(c->d_zx);
   c->d_zx = nullptr;
@@ -408,18 +416,29 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   return PLR_OK;
 }
 
-int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d) {
+int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
   int rc = plan_shape(c, n, d);
   if (rc != PLR_OK) return rc;
+  // sizes are computed in size_t below: a shard whose byte count does not fit
+  // in 64 bits must be refused here, not wrap around to a small allocation
+  // that the kernels would then stream far past
+  const size_t slack_bytes = std::max<size_t>((size_t)c->theta_len * sizeof(double), 64u << 10);
+  if ((uint64_t)n > (UINT64_MAX / sizeof(double) - slack_bytes) / (uint64_t)c->pitch)
+    return fail(c, PLR_ERR_INVALID, "n * pitch * 8 bytes does not fit in 64 bits");
   c->n = n;
   c->d = d;
   // lanes of the chunk that straddles the end of the last row read (and then
   // discard) up to one slab past it: keep that much slack mapped
-  const size_t xbytes = (size_t)n * c->pitch * sizeof(double) +
-                        std::max<size_t>((size_t)c->theta_len * sizeof(double), 64u << 10);
+  const size_t xbytes = (size_t)n * c->pitch * sizeof(double) + slack_bytes;
   if (n > 0) {
     PLR_HIP(c, hipMalloc(&c->dX, xbytes));
     PLR_HIP(c, hipMalloc(&c->dy, (size_t)n * sizeof(double)));
+    if (zero_fill) {
+      // a shard that is filled row range by row range: rows the caller never
+      // sends must read as zeros, not as whatever the memory held
+      PLR_HIP(c, hipMemsetAsync(c->dX, 0, xbytes, c->stream));
+      PLR_HIP(c, hipMemsetAsync(c->dy, 0, (size_t)n * sizeof(double), c->stream));
+    }
   }
   const int gmax = c->grid > c->grid_nograd ? c->grid : c->grid_nograd;
   PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)c->theta_len * sizeof(double)));
@@ -452,12 +471,12 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d) {
 
 // Drop the resident shard (if any) and reserve an n x d one.  On failure the
 // context is left without a shard (shape 0 x 0), never half allocated.
-int alloc_shape(plr_ctx* c, int64_t n, int64_t d) {
+int alloc_shape(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
   if (n < 0 || d < 1)
     return fail(c, PLR_ERR_INVALID, "need n >= 0 and d >= 1");
   PLR_HIP(c, hipSetDevice(c->device));
   free_shape(c);
-  const int rc = alloc_shape_buffers(c, n, d);
+  const int rc = alloc_shape_buffers(c, n, d, zero_fill);
   if (rc != PLR_OK) free_shape(c);  // keeps c->err
   return rc;
 }
@@ -548,7 +567,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   pa.theta = c->d_theta;
   pa.part_g = c->d_part_g;
   pa.part_loss = c->d_part_loss;
-  pa.h_out = predict ? c->d_h : nullptr;
+  pa.h_out = predict ? (c->h_pred_dev ? c->h_pred_dev : c->d_h) : nullptr;
   pa.n = c->n;
   pa.pitch = c->pitch;
   pa.ntiles = ceil_div(c->n, v->R);
@@ -604,6 +623,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   } else if (c->n > 0) {
     // sweep 1: z = x.theta, one launch per column block, accumulated in d_z
     pa.z_buf = c->d_z;
+    double* const pred_out = pa.h_out;  // the residual kernel writes the predictions
     pa.h_out = nullptr;
     for (int64_t col0 = 0; col0 < c->pitch; col0 += kBlockCols) {
       const int64_t w = std::min<int64_t>(kBlockCols, c->pitch - col0);
@@ -620,7 +640,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     // residual, prediction and loss per row
     hipLaunchKernelGGL(plr::residual_pass, dim3(grid), dim3(256), 0, c->stream,
                        (const double*)c->d_z, (const double*)pa.y, grad ? c->d_res : nullptr,
-                       predict ? c->d_h : nullptr, c->d_part_loss, c->n, pa.loss_mode,
+                       pred_out, c->d_part_loss, c->n, pa.loss_mode,
                        pa.identity_link);
     PLR_HIP(c, hipGetLastError());
     // sweep 2: rank-1 updates, block by block
@@ -715,8 +735,21 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
   if (loss_mode > plr::kLossSquared) return fail(c, PLR_ERR_INVALID, "unknown loss flag");
   PLR_HIP(c, hipSetDevice(c->device));
   const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
-  if (predict && !c->d_h && c->n > 0)
-    PLR_HIP(c, hipMalloc(&c->d_h, (size_t)c->n * sizeof(double)));
+  if (predict && !c->d_h && !c->h_pred && c->n > 0) {
+    // Where the predictions go.  A row of kHostPredictCols columns or more
+    // streams slowly enough (8 bytes out per >= 1.5 KiB in) for the host link
+    // to keep up: the kernel then writes straight into pinned host memory --
+    // no HBM write traffic disturbing the read stream, no copy command
+    // afterwards.  Narrower rows produce predictions faster than the link
+    // takes them; they go to device memory and are copied out in a pipeline.
+    if (c->pitch >= kHostPredictCols) {
+      PLR_HIP(c, hipHostMalloc(&c->h_pred, (size_t)c->n * sizeof(double),
+                               hipHostMallocMapped | hipHostMallocCoherent));
+      PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_pred_dev), c->h_pred, 0));
+    } else {
+      PLR_HIP(c, hipMalloc(&c->d_h, (size_t)c->n * sizeof(double)));
+    }
+  }
   int rc = stage_theta_from_host(c, theta);
   if (rc != PLR_OK) return rc;
   rc = enqueue_pass(c, kind, loss_mode, alpha, beta, c->h_out_dev, -1);
@@ -776,6 +809,9 @@ int plr_create(plr_ctx** out, int device_id) {
 void plr_destroy(plr_ctx* c) {
   if (!c) return;
   free_shape(c);
+  if (c->out_stage) (void)hipHostFree(c->out_stage);
+  for (hipStream_t st : c->out_stream)
+    if (st) (void)hipStreamDestroy(st);
   if (c->ev0) (void)hipEventDestroy(c->ev0);
   if (c->ev1) (void)hipEventDestroy(c->ev1);
   if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -784,7 +820,7 @@ void plr_destroy(plr_ctx* c) {
 
 int plr_alloc_data(plr_ctx* c, int64_t n, int64_t d) {
   if (!c) return PLR_ERR_INVALID;
-  return alloc_shape(c, n, d);
+  return alloc_shape(c, n, d, /*zero_fill=*/true);
 }
 
 int plr_set_data_chunk(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
@@ -799,7 +835,7 @@ int plr_set_data(plr_ctx* c, const double* X, int64_t n, int64_t d, int64_t ldx,
   if (!c) return PLR_ERR_INVALID;
   if (n > 0 && (!X || !y)) return fail(c, PLR_ERR_INVALID, "X and y must not be NULL");
   if (ldx < d) return fail(c, PLR_ERR_INVALID, "ldx must be >= d");
-  int rc = alloc_shape(c, n, d);
+  int rc = alloc_shape(c, n, d, /*zero_fill=*/false);  // every row is uploaded right below
   if (rc != PLR_OK) return rc;
   return upload_rows(c, 0, n, X, ldx, y);
 }
@@ -888,13 +924,103 @@ int plr_calc_loss(plr_ctx* c, const double* theta, double* loss_sum, int64_t* n_
   return PLR_OK;
 }
 
+// n doubles from the device into the caller's (pageable) buffer.  One plain
+// copy command moves them through the runtime's own staging at ~10 GB/s; for
+// tall shards that is several times the kernel.  Large results therefore go
+// through kCopyLanes independent lanes, each with two pinned staging blocks on
+// a stream of its own: the DMA into one block overlaps the host copy out of
+// the other, and the lanes overlap each other.
+constexpr int kCopyLanes = 4;
+constexpr size_t kCopyBlock = 4u << 20;
+
+// pinned host memory -> the caller's buffer, kCopyLanes threads
+static void copy_host_parallel(double* out, const double* src, size_t count) {
+  if (count * sizeof(double) < (8u << 20)) {
+    memcpy(out, src, count * sizeof(double));
+    return;
+  }
+  std::thread th[kCopyLanes];
+  const size_t per = (count + kCopyLanes - 1) / kCopyLanes;
+  for (int l = 0; l < kCopyLanes; ++l)
+    th[l] = std::thread([=]() {
+      const size_t lo = std::min(count, (size_t)l * per), hi = std::min(count, lo + per);
+      if (hi > lo) memcpy(out + lo, src + lo, (hi - lo) * sizeof(double));
+    });
+  for (int l = 0; l < kCopyLanes; ++l) th[l].join();
+}
+
+static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t count) {
+  const size_t bytes = count * sizeof(double);
+  if (bytes < 4 * kCopyBlock) {
+    PLR_HIP(c, hipMemcpy(out, dev, bytes, hipMemcpyDeviceToHost));
+    return PLR_OK;
+  }
+  if (!c->out_stage) {
+    PLR_HIP(c, hipHostMalloc(&c->out_stage, 2 * kCopyLanes * kCopyBlock, hipHostMallocDefault));
+    for (int l = 0; l < kCopyLanes; ++l)
+      PLR_HIP(c, hipStreamCreateWithFlags(&c->out_stream[l], hipStreamNonBlocking));
+  }
+  hipError_t errs[kCopyLanes];
+  std::thread th[kCopyLanes];
+  const size_t per_lane = ((count + kCopyLanes - 1) / kCopyLanes + 511) & ~(size_t)511;
+  for (int l = 0; l < kCopyLanes; ++l) {
+    errs[l] = hipSuccess;
+    th[l] = std::thread([&, l]() {
+      if (hipSetDevice(c->device) != hipSuccess) {
+        errs[l] = hipErrorInvalidDevice;
+        return;
+      }
+      const size_t lo = std::min(count, (size_t)l * per_lane);
+      const size_t hi = std::min(count, lo + per_lane);
+      char* stage = static_cast<char*>(c->out_stage) + (size_t)l * 2 * kCopyBlock;
+      const size_t blk = kCopyBlock / sizeof(double);
+      hipStream_t st = c->out_stream[l];
+      // block k is in flight while block k - 1 is copied out
+      size_t issued = lo, drained = lo;
+      int slot = 0;
+      auto issue = [&]() {
+        const size_t m = std::min(blk, hi - issued);
+        const hipError_t e = hipMemcpyAsync(stage + (size_t)slot * kCopyBlock, dev + issued,
+                                            m * sizeof(double), hipMemcpyDeviceToHost, st);
+        if (e != hipSuccess) errs[l] = e;
+        issued += m;
+        slot ^= 1;
+      };
+      if (issued < hi) issue();
+      while (drained < hi && errs[l] == hipSuccess) {
+        const hipError_t e = hipStreamSynchronize(st);  // the block issued last has landed
+        if (e != hipSuccess) {
+          errs[l] = e;
+          break;
+        }
+        const int ready = slot ^ 1;
+        const size_t m = std::min(blk, hi - drained);
+        if (issued < hi) issue();                       // next block on its way ...
+        memcpy(out + drained, stage + (size_t)ready * kCopyBlock, m * sizeof(double));  // ... during this
+        drained += m;
+      }
+    });
+  }
+  for (int l = 0; l < kCopyLanes; ++l) th[l].join();
+  for (int l = 0; l < kCopyLanes; ++l)
+    if (errs[l] != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(c, PLR_ERR_HIP,
+                  std::string("copying the predictions out failed: ") + hipGetErrorString(errs[l]));
+    }
+  return PLR_OK;
+}
+
 static int predict_rows(plr_ctx* c, PassKind kind, const double* theta, double* out) {
   if (!c) return PLR_ERR_INVALID;
   if (!out && c->n > 0) return fail(c, PLR_ERR_INVALID, "output must not be NULL");
   int rc = run_pass(c, kind, theta, plr::kLossNone, 0., 0.);
   if (rc != PLR_OK) return rc;
-  if (c->n > 0)
-    PLR_HIP(c, hipMemcpy(out, c->d_h, (size_t)c->n * sizeof(double), hipMemcpyDeviceToHost));
+  if (c->n > 0 && c->h_pred) {
+    copy_host_parallel(out, c->h_pred, (size_t)c->n);
+    return PLR_OK;
+  }
+  if (c->n > 0) return copy_rows_out(c, out, c->d_h, (size_t)c->n);
   return PLR_OK;
 }
 

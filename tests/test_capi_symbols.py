@@ -30,6 +30,26 @@ def test_library_exports_every_declared_symbol():
     assert loaded.plr_last_error(None) is not None
 
 
+def test_header_is_plain_c99_and_a_c_caller_links(tmp_path):
+    """include/plr.h is a C header: it compiles as C99 with -pedantic -Wall -Werror on its own,
+    and the plain-C caller that binds it links against libplr.so (no C++ runtime needed by
+    the caller)."""
+    import subprocess
+
+    from paracel_amd import capi
+
+    probe = tmp_path / "probe.c"
+    probe.write_text('#include "plr.h"\nint main(void) { return (int)PLR_OK; }\n')
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only",
+                    "-I", os.path.join(ROOT, "include"), str(probe)], check=True)
+    out = tmp_path / "plr_c_caller"
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror",
+                    "-I", os.path.join(ROOT, "include"), "-o", str(out),
+                    os.path.join(ROOT, "paracel_amd", "examples", "plr_c_caller.c"),
+                    "-L", os.path.dirname(capi.lib_path()), "-lplr"], check=True)
+    assert out.exists()
+
+
 def test_product_does_not_touch_the_oracle():
     # the oracle is test infrastructure: nothing under paracel_amd/ or include/ may
     # import, link or load it

@@ -342,6 +342,22 @@ def test_chunked_upload_equals_whole(plr, gen):
     assert loss == loss2
 
 
+def test_rows_never_uploaded_read_as_zero_rows(plr, oracle, gen):
+    # plr_alloc_data reserves a zero-filled shard: a row range the caller never sends behaves
+    # as rows of zeros with label 0 (h = 1/2 each), not as whatever the memory held before
+    X, y, th = make(gen, 3000, 130)
+    plr.set_data(np.full((3000, 130), 7.5), np.ones(3000))   # leave something behind
+    plr.alloc_data(3000, 130)
+    plr.set_data_chunk(0, X[:1000], y[:1000])
+    plr.set_data_chunk(2000, X[2000:], y[2000:])
+    Xz, yz = X.copy(), y.copy()
+    Xz[1000:2000] = 0.0
+    yz[1000:2000] = 0.0
+    g, loss, _ = plr.loss_grad(th)
+    assert rel(g, oracle.gsum(Xz, yz, th)) <= GRAD_TOL
+    assert abs(loss - oracle.calc_loss_sum(Xz, yz, th)) <= LOSS_TOL * loss
+
+
 def test_pitched_input(plr, oracle, gen):
     X, y, th = make(gen, 500, 333)
     wide = np.full((500, 400), np.nan)
@@ -501,6 +517,13 @@ def test_a_shard_that_does_not_fit_is_refused_cleanly(plr, oracle, gen):
     with pytest.raises(PlrError) as e:
         plr.loss_grad(np.zeros(0))
     assert e.value.code == -4
+    # a row count whose byte size wraps around 64 bits is refused before any allocation
+    # (it must not come back as a small allocation that the kernels then run past)
+    for n_bad, d_bad in ((1 << 61, 1000), (1 << 62, 3), ((1 << 63) - 1, 70), (1 << 58, 40000)):
+        with pytest.raises(PlrError) as e:
+            plr.alloc_data(n_bad, d_bad)
+        assert e.value.code == -1 and "64 bits" in str(e.value), (n_bad, d_bad, str(e.value))
+        assert plr.shape == (0, 0)
     # and is usable again
     plr.set_data(X, y)
     g, _, _ = plr.loss_grad(th)
