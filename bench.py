@@ -71,6 +71,8 @@ PER_CONFIG = ["c1_dense_100k_x_100", "c3_tall_10m_x_256", "c4_wide_200k_x_16384"
 # A one-GPU box gives a job 16 CPUs whatever os.cpu_count() shows there.
 CPU_SHARE = 16
 
+KEEP_BIAS_COLUMN = False  # --keep-bias-column
+
 
 def measured_traffic(cfg, kernel_info):
     ent = MEASURED_TRAFFIC.get(cfg.name)
@@ -91,6 +93,9 @@ def parse_args():
     ap.add_argument("--workload", default=None,
                     help="time only this workload (default: the headline c2_headline_1m_x_1000 "
                          "plus the other configurations under per_config)")
+    ap.add_argument("--keep-bias-column", action="store_true",
+                    help="workloads whose first column is the constant bias: store it in HBM "
+                         "like any other column (default: it stays on the host)")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the per_config section of a default run")
     ap.add_argument("--rows", type=int, default=0, help="override n (debugging)")
@@ -115,6 +120,9 @@ def upload(ctx, cfg, chunk_bytes=1 << 30, keep_rows=0):
     Returns the first keep_rows rows (for the CPU baseline sample)."""
     import numpy as np
 
+    # a shard as the file path builds it starts every row with the bias 1.0: say so, and
+    # the library keeps that column out of HBM (--keep-bias-column stores it, for comparison)
+    ctx.set_option("first_column_is_one", 1 if (cfg.bias_first and not KEEP_BIAS_COLUMN) else 0)
     ctx.alloc_data(cfg.n, cfg.d)
     chunk_rows = max(1, chunk_bytes // (8 * cfg.d))
     keepX, keepy = [], []
@@ -424,7 +432,9 @@ def per_config_entry(rec):
 
 
 def main():
+    global KEEP_BIAS_COLUMN
     a = parse_args()
+    KEEP_BIAS_COLUMN = a.keep_bias_column
     if a.gpus != 1:
         print("bench.py measures one GPU's shard: this build has no multi-GPU path "
               "(run with --gpus 1)", file=sys.stderr)

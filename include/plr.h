@@ -169,6 +169,15 @@ int plr_set_timing(plr_ctx* ctx, int enabled);
 
 /* Tuning and diagnostic switches of a context; no counterpart in the
  * reference.  Keys:
+ *   "first_column_is_one"  value != 0: the caller states that column 0 of every
+ *        shard it uploads from now on is the constant 1.0 -- the bias column
+ *        local_parser prepends (lr.cpp:83).  The library then keeps only the
+ *        other d - 1 columns in HBM (a 2^k + 1 wide row streams as a 2^k wide
+ *        one), adds theta[0] to every dot product and returns the sum of the
+ *        residuals as gsum[0]; every result is what the stored column would
+ *        have given.  The upload checks the statement row by row and fails
+ *        with PLR_ERR_INVALID at the first row that does not start with 1.0.
+ *        Applies from the next plr_set_data / plr_alloc_data.  Default 0.
  *   "column_blocks_two_sweeps"  value != 0: rows wider than 19456 columns are
  *        processed in two sweeps over X (dot products, then updates) instead
  *        of once by cooperating workgroups; applies from the next

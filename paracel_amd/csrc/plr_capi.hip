@@ -153,6 +153,15 @@ struct plr_ctx {
   double* dy = nullptr;
   int64_t n = 0, d = 0, pitch = 0;
   bool have_data = false;
+  // A first column that is 1.0 in every row (the bias column of the file path)
+  // is not stored when the caller says so: the shard then holds dcols = d - 1
+  // columns, theta's first entry lives in d_theta[bias_slot], and the sum of
+  // the residuals (d_part_res) is that column's gradient.
+  bool opt_first_col_one = false;  // plr_set_option("first_column_is_one")
+  bool bias = false;               // in force for the resident shard
+  int64_t dcols = 0;               // stored columns
+  int64_t bias_slot = 0;
+  double* d_part_res = nullptr;    // max(grid, grid_nograd)
 
   // per-shape workspace
   const Shape* var = nullptr;       // shape of the shard_pass variant in use
@@ -240,6 +249,10 @@ void free_shape(plr_ctx* c) {
   if (c->d_theta) (void)hipFree(c->d_theta);
   if (c->d_part_g) (void)hipFree(c->d_part_g);
   if (c->d_part_loss) (void)hipFree(c->d_part_loss);
+  if (c->d_part_res) (void)hipFree(c->d_part_res);
+  c->d_part_res = nullptr;
+  c->bias = false;
+  c->dcols = 0;
   if (c->d_h) (void)hipFree(c->d_h);
   if (c->h_pred) (void)hipHostFree(c->h_pred);
   c->h_pred = c->h_pred_dev = nullptr;
@@ -417,8 +430,12 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
 }
 
 int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
-  int rc = plan_shape(c, n, d);
+  c->bias = c->opt_first_col_one && d >= 2;
+  c->dcols = d - (c->bias ? 1 : 0);
+  int rc = plan_shape(c, n, c->dcols);
   if (rc != PLR_OK) return rc;
+  if (c->bias) c->info += "; first column constant 1, not stored";
+  c->bias_slot = c->theta_len;  // behind the zero padding
   // sizes are computed in size_t below: a shard whose byte count does not fit
   // in 64 bits must be refused here, not wrap around to a small allocation
   // that the kernels would then stream far past
@@ -441,7 +458,8 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
     }
   }
   const int gmax = c->grid > c->grid_nograd ? c->grid : c->grid_nograd;
-  PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)c->theta_len * sizeof(double)));
+  PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)(c->theta_len + 8) * sizeof(double)));
+  PLR_HIP(c, hipMalloc(&c->d_part_res, (size_t)gmax * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_g, (size_t)c->grid * c->pitch * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_loss, (size_t)gmax * sizeof(double)));
   if (c->team_blocks > 0) {
@@ -450,7 +468,7 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
     PLR_HIP(c, hipMalloc(&c->d_z, (size_t)n * sizeof(double)));
     PLR_HIP(c, hipMalloc(&c->d_res, (size_t)n * sizeof(double)));
   }
-  PLR_HIP(c, hipHostMalloc(&c->h_theta, (size_t)c->theta_len * sizeof(double),
+  PLR_HIP(c, hipHostMalloc(&c->h_theta, (size_t)(c->theta_len + 8) * sizeof(double),
                            hipHostMallocMapped | hipHostMallocCoherent));
   PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_theta_dev), c->h_theta, 0));
   // results land in host memory straight from the finishing kernel (no
@@ -458,11 +476,11 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
   PLR_HIP(c, hipHostMalloc(&c->h_out, (size_t)(d + 1) * sizeof(double),
                            hipHostMallocMapped | hipHostMallocCoherent));
   PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_out_dev), c->h_out, 0));
-  memset(c->h_theta, 0, (size_t)c->theta_len * sizeof(double));
-  PLR_HIP(c, hipMemsetAsync(c->d_theta, 0, (size_t)c->theta_len * sizeof(double), c->stream));
-  if (n > 0 && c->pitch != d)  // the pad column must read as zero
-    PLR_HIP(c, hipMemset2DAsync(c->dX + d, (size_t)c->pitch * sizeof(double), 0,
-                                (size_t)(c->pitch - d) * sizeof(double), (size_t)n,
+  memset(c->h_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double));
+  PLR_HIP(c, hipMemsetAsync(c->d_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double), c->stream));
+  if (n > 0 && c->pitch != c->dcols)  // the pad column must read as zero
+    PLR_HIP(c, hipMemset2DAsync(c->dX + c->dcols, (size_t)c->pitch * sizeof(double), 0,
+                                (size_t)(c->pitch - c->dcols) * sizeof(double), (size_t)n,
                                 c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
   c->have_data = true;
@@ -489,7 +507,17 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
   if (row0 < 0 || nrows < 0 || row0 + nrows > c->n)
     return fail(c, PLR_ERR_INVALID, "row range outside the reserved shard");
   PLR_HIP(c, hipSetDevice(c->device));
-  if (ldx == c->pitch && c->d == c->pitch) {  // same pitch, no pad column: one linear copy
+  const int skip = c->bias ? 1 : 0;  // the constant first column stays on the host
+  if (c->bias) {
+    for (int64_t r = 0; r < nrows; ++r)
+      if (X[r * ldx] != 1.) {
+        char b[160];
+        snprintf(b, sizeof b, "first_column_is_one is set, but row %lld starts with %.17g",
+                 (long long)(row0 + r), X[r * ldx]);
+        return fail(c, PLR_ERR_INVALID, b);
+      }
+  }
+  if (!c->bias && ldx == c->pitch && c->d == c->pitch) {  // same pitch, no pad column: one linear copy
     PLR_HIP(c, hipMemcpy(c->dX + row0 * c->pitch, X,
                          (size_t)nrows * c->pitch * sizeof(double), hipMemcpyHostToDevice));
   } else {
@@ -524,8 +552,8 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
         rc = fail(c, PLR_ERR_HIP, "upload: waiting for a staging buffer failed");
       for (int64_t r = 0; r < m && rc == PLR_OK; ++r) {
         double* dst = stage[k] + r * c->pitch;
-        memcpy(dst, X + (r0 + r) * ldx, (size_t)c->d * sizeof(double));
-        for (int64_t j = c->d; j < c->pitch; ++j) dst[j] = 0.;
+        memcpy(dst, X + (r0 + r) * ldx + skip, (size_t)c->dcols * sizeof(double));
+        for (int64_t j = c->dcols; j < c->pitch; ++j) dst[j] = 0.;
       }
       if (rc == PLR_OK &&
           (hipMemcpyAsync(c->dX + (row0 + r0) * c->pitch, stage[k],
@@ -576,6 +604,8 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   pa.loss_mode = predict ? (unsigned)plr::kLossNone : loss_mode;
   pa.identity_link = (kind == kPassPredictLinear || loss_mode == plr::kLossSquared) ? 1 : 0;
 
+  pa.theta_bias = c->bias ? c->d_theta + c->bias_slot : nullptr;
+  pa.part_res = c->bias ? c->d_part_res : nullptr;
   pa.width = c->pitch;
   pa.z_buf = nullptr;
   pa.z_accumulate = 0;
@@ -610,6 +640,8 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     ta.nteams = c->nteams;
     ta.blk_chunks = c->team_blk_chunks;
     ta.nch_rt = c->team_blk_chunks / plr::kTeamWaves;
+    ta.theta_bias = pa.theta_bias;
+    ta.part_res = pa.part_res;
     ta.zeros = c->d_theta + c->theta_len - plr::kChunkCols;  // the padding never changes
     ta.zx = c->d_zx;
     ta.status = reinterpret_cast<unsigned*>(c->d_zx + c->zx_words);
@@ -641,7 +673,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     hipLaunchKernelGGL(plr::residual_pass, dim3(grid), dim3(256), 0, c->stream,
                        (const double*)c->d_z, (const double*)pa.y, grad ? c->d_res : nullptr,
                        pred_out, c->d_part_loss, c->n, pa.loss_mode,
-                       pa.identity_link);
+                       pa.identity_link, pa.theta_bias, pa.part_res);
     PLR_HIP(c, hipGetLastError());
     // sweep 2: rank-1 updates, block by block
     if (grad) {
@@ -662,6 +694,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   } else {
     // empty shard: the finishing kernel needs zeroed partials
     PLR_HIP(c, hipMemsetAsync(c->d_part_loss, 0, (size_t)grid * sizeof(double), c->stream));
+    PLR_HIP(c, hipMemsetAsync(c->d_part_res, 0, (size_t)grid * sizeof(double), c->stream));
     if (grad)
       PLR_HIP(c, hipMemsetAsync(c->d_part_g, 0, (size_t)grid * c->pitch * sizeof(double),
                                 c->stream));
@@ -675,8 +708,10 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     fa.theta = c->d_theta;
     fa.out = out;
     fa.pitch = c->pitch;
-    fa.d = c->d;
+    fa.d = c->dcols;
     fa.n = c->n;
+    fa.part_res = pa.part_res;
+    fa.theta_bias = c->d_theta + c->bias_slot;
     fa.nparts = c->team_blocks > 0 ? c->nteams : grid;  // a team shares one row of partials
     fa.nparts_loss = fa.nparts;
     fa.delta_mode = (kind == kPassDelta) ? (train_round >= 0 ? 2 : 1) : 0;
@@ -685,7 +720,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     fa.coff2 = 2. * beta * alpha;
     fa.theta_rw = c->d_theta;
     fa.loss_slot = (train_round >= 0 && c->d_curve) ? c->d_curve + train_round : nullptr;
-    const int fgrid = grad ? (int)ceil_div(c->d, plr::kFinCols) : 1;
+    const int fgrid = grad ? (int)ceil_div(c->dcols, plr::kFinCols) : 1;
     hipLaunchKernelGGL(plr::finish_pass, dim3(fgrid),
                        dim3(plr::kFinCols * plr::kFinSlices), 0, c->stream, fa);
     PLR_HIP(c, hipGetLastError());
@@ -698,7 +733,8 @@ int stage_theta_from_host(plr_ctx* c, const double* theta) {
   memcpy(c->h_theta, theta, (size_t)c->d * sizeof(double));
   const int sgrid = (int)((c->d + 1023) / 1024 > 64 ? 64 : (c->d + 1023) / 1024);
   hipLaunchKernelGGL(plr::stage_theta, dim3(sgrid), dim3(256), 0, c->stream,
-                     (const double*)c->h_theta_dev, c->d_theta, c->d);
+                     (const double*)c->h_theta_dev, c->d_theta, c->d, c->bias ? 1 : 0,
+                     c->bias_slot);
   PLR_HIP(c, hipGetLastError());
   return PLR_OK;
 }
@@ -899,8 +935,12 @@ int plr_train_dgd(plr_ctx* c, double* theta, double alpha, double beta, int roun
     rc = enqueue_pass(c, kPassDelta, loss_mode, alpha, beta, c->d_train_out, rd);
     if (rc != PLR_OK) return rc;
   }
-  PLR_HIP(c, hipMemcpyAsync(c->h_theta, c->d_theta, (size_t)c->d * sizeof(double),
+  const int skip = c->bias ? 1 : 0;
+  PLR_HIP(c, hipMemcpyAsync(c->h_theta + skip, c->d_theta, (size_t)c->dcols * sizeof(double),
                             hipMemcpyDeviceToHost, c->stream));
+  if (c->bias)
+    PLR_HIP(c, hipMemcpyAsync(c->h_theta, c->d_theta + c->bias_slot, sizeof(double),
+                              hipMemcpyDeviceToHost, c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
   rc = check_team_status(c);
   if (rc != PLR_OK) return rc;
@@ -1116,6 +1156,10 @@ int plr_set_option(plr_ctx* c, const char* key, int64_t value) {
     c->team_spin_limit = (unsigned)value;
     return PLR_OK;
   }
+  if (strcmp(key, "first_column_is_one") == 0) {
+    c->opt_first_col_one = value != 0;  // takes effect at the next plr_set_data / plr_alloc_data
+    return PLR_OK;
+  }
   if (strcmp(key, "column_blocks_two_sweeps") == 0) {
     c->opt_two_sweeps = value != 0;  // takes effect at the next plr_set_data / plr_alloc_data
     return PLR_OK;
@@ -1237,6 +1281,8 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
     pa.z_buf = nullptr;
     pa.z_accumulate = 0;
     pa.res_in = nullptr;
+    pa.theta_bias = nullptr;
+    pa.part_res = nullptr;
     hipLaunchKernelGGL(fn, dim3(grid), dim3(threads), 0, stream, pa);
     PLR_NA_HIP(hipGetLastError());
   } else {
@@ -1262,6 +1308,8 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
   fa.coff2 = 0.;
   fa.theta_rw = nullptr;
   fa.loss_slot = nullptr;
+  fa.part_res = nullptr;
+  fa.theta_bias = nullptr;
   hipLaunchKernelGGL(plr::finish_pass, dim3((int)ceil_div(d, plr::kFinCols)),
                      dim3(plr::kFinCols * plr::kFinSlices), 0, stream, fa);
   PLR_NA_HIP(hipGetLastError());

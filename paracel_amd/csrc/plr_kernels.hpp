@@ -97,7 +97,48 @@ struct PassArgs {
   double* z_buf;         // n: x.theta accumulated over the column blocks
   int z_accumulate;      // 0: this block stores its partial dot, 1: adds to it
   const double* res_in;  // n: residual per row, computed between the two sweeps
+  // A first column that is 1.0 in every row (the bias column the worker's
+  // parser prepends, lr.cpp:83) is not stored: X, theta and part_g then hold
+  // the OTHER columns, theta_bias points at the coefficient of the constant
+  // column (added to every dot product) and part_res receives, per
+  // workgroup, the sum of the residuals -- that column's gradient.
+  const double* theta_bias;  // nullptr: every column is stored
+  double* part_res;          // [grid], or nullptr
 };
+
+// loss and residual sums of a pass travel together
+struct RowSums {
+  double loss = 0.;
+  double res = 0.;
+};
+
+// Fold the waves' sums in wave order; thread 0 stores the workgroup's partials.
+template <int NW>
+__device__ __forceinline__ void emit_row_sums(const RowSums& s, int lane, int wave,
+                                              double* part_loss, double* part_res) {
+  __shared__ double lx[NW], rx[NW];
+  double wl = s.loss, wr = s.res;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) {
+    wl += __shfl_xor(wl, m, 64);
+    wr += __shfl_xor(wr, m, 64);
+  }
+  if (lane == 0) {
+    lx[wave] = wl;
+    rx[wave] = wr;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double a = 0., b = 0.;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      a += lx[w];
+      b += rx[w];
+    }
+    part_loss[blockIdx.x] = a;
+    if (part_res) part_res[blockIdx.x] = b;
+  }
+}
 
 // What one launch of shard_pass does with a tile.
 enum : int {
@@ -221,6 +262,7 @@ struct WaveCtx {
   int tail_slot;      // lane holding the tail dot of row my_row
   uint32_t tail_off;  // byte offset of the lane's pair from the tile base
   int tail_src[4];    // per tail load: lane holding the residual of its row
+  double bias;        // theta of the constant first column that is not stored, or 0
 };
 
 // Geometry of the tail stage: a tile's R rows are covered by TL loads of
@@ -238,6 +280,12 @@ __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
                                           const double* tile_base, int64_t row0,
                                           v2d (&x)[R][NCH], v2d (&xt)[TL > 0 ? TL : 1],
                                           double& yv) {
+  // The chunk that straddles the row end is loaded under the lane mask when it
+  // is the wave's last slot: lanes past the row end then request nothing
+  // (fewer cache lines touched per load).  Those loads are issued together,
+  // after all the others of the tile, so that the mask changes once per tile
+  // and the run of back-to-back loads stays unbroken.
+  const bool masked_last = w.ragged_c == NCH - 1;  // uniform
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const char* rowp = reinterpret_cast<const char*>(tile_base + (int64_t)r * a.pitch);
@@ -245,12 +293,18 @@ __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       x[r][c] = v2d{0., 0.};
-      // uniform, except that a one-chunk row loads its ragged chunk under the
-      // lane mask: lanes past the row end then request nothing (every load of
-      // the tile sits under the same mask, so the run of loads stays unbroken)
-      if (rv && (ALLCH || c < w.my_nch) && (NCH > 1 || w.ragged_c < 0 || w.lane_in_ragged))
+      if (rv && (ALLCH || c < w.my_nch) && !(c == NCH - 1 && masked_last))  // uniform
         x[r][c] = load_x(reinterpret_cast<const v2d*>(
             rowp + w.lane_off + (uint32_t)(c * kChunkCols * sizeof(double))));
+    }
+  }
+  if (masked_last && w.lane_in_ragged) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const char* rowp = reinterpret_cast<const char*>(tile_base + (int64_t)r * a.pitch);
+      if (FULL || (row0 + r) < a.n)  // uniform
+        x[r][NCH - 1] = load_x(reinterpret_cast<const v2d*>(
+            rowp + w.lane_off + (uint32_t)((NCH - 1) * kChunkCols * sizeof(double))));
     }
   }
   if constexpr (TL > 0) {
@@ -280,7 +334,7 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
                                              int64_t row0, v2d (&x)[R][NCH],
                                              const v2d (&xt)[TL > 0 ? TL : 1], double yv,
                                              const v2d (&th)[NCH], const v2d* thl, v2d tht,
-                                             v2d (&acc)[NCH], v2d& acct, double& loss_acc,
+                                             v2d (&acc)[NCH], v2d& acct, RowSums& sums,
                                              double* zbuf, double& h_keep, int64_t& h_row) {
   const int lane = w.lane;
   const int64_t myrow_g = row0 + w.my_row;
@@ -372,14 +426,17 @@ __device__ __forceinline__ void compute_tile(const PassArgs& a, const WaveCtx& w
 
     // ---- sigmoid, residual, loss for the row this lane holds ----
     double h, l;
-    row_terms(z, yv, a.loss_mode, a.identity_link, h, l);
+    row_terms(z + w.bias, yv, a.loss_mode, a.identity_link, h, l);
     res = my_valid ? (h - yv) : 0.;
     // predictions are not stored here but after the NEXT tile's loads have been
     // issued (see the tile loop): a store in front of them would have to be
     // acknowledged before any of their data counts as returned
     h_keep = h;
     h_row = (my_valid && lane < R && w.wc == 0) ? myrow_g : -1;
-    if (my_valid && lane < R && w.wc == 0) loss_acc += l;
+    if (my_valid && lane < R && w.wc == 0) {
+      sums.loss += l;
+      sums.res += res;
+    }
   }
 
   // ---- rank-1 update of the gradient slab from the same registers ----
@@ -488,7 +545,8 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
     if (THL) thl[c * kWave] = t;
     thr[c] = t;
   }
-  double loss_acc = 0.;
+  RowSums sums;
+  w.bias = (MODE == kPassFused && a.theta_bias) ? *a.theta_bias : 0.;
 
   __shared__ double zx[(WCOL > 1) ? 2 * WCOL * R : 1];
 
@@ -516,7 +574,7 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
                                              yv);
     store_kept();
     compute_tile<NCH, R, WCOL, GRAD, true, THL, MODE, TL>(a, w, tile * R, x, xt, yv, thr, thl,
-                                                          tht, acc, acct, loss_acc,
+                                                          tht, acc, acct, sums,
                                                           zx + par * kZ, h_keep, h_row);
   }
   if (tile < a.ntiles) {
@@ -526,7 +584,7 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
                                               yv);
     store_kept();
     compute_tile<NCH, R, WCOL, GRAD, false, THL, MODE, TL>(a, w, tile * R, x, xt, yv, thr, thl,
-                                                           tht, acc, acct, loss_acc,
+                                                           tht, acc, acct, sums,
                                                            zx + par * kZ, h_keep, h_row);
   }
   store_kept();
@@ -569,18 +627,8 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
       emit(acct, lane < kLpr && w.tail_in, out + slab_col0 + kBodyCols + 2 * tail_pair);
     }
   }
-  if constexpr (MODE == kPassFused) {  // the sweeps of a blocked row carry no loss
-    __shared__ double lx[WCOL * WROW];
-    const double wl = wave_sum(loss_acc);
-    if (lane == 0) lx[wave] = wl;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      double s = 0.;
-#pragma unroll
-      for (int w = 0; w < WCOL * WROW; ++w) s += lx[w];
-      a.part_loss[blockIdx.x] = s;
-    }
-  }
+  if constexpr (MODE == kPassFused)  // the sweeps of a blocked row carry no loss
+    emit_row_sums<WCOL * WROW>(sums, lane, wave, a.part_loss, a.part_res);
 }
 
 // ---------------------------------------------------------------------------
@@ -612,8 +660,9 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void packed_pass(PassArgs a) {
   const int my_chunk = row_of_lane<SL>(pos);  // chunk of the group whose row ends up here
 
   const v2d th = *reinterpret_cast<const v2d*>(a.theta + 2 * pos);
+  const double bias = a.theta_bias ? *a.theta_bias : 0.;
   v2d acc = v2d{0., 0.};
-  double loss_acc = 0.;
+  RowSums sums;
   // a tile's predictions are stored after the next tile's loads have been
   // issued (a store in front of them would have to be acknowledged first)
   double h_keep[U];
@@ -691,11 +740,14 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void packed_pass(PassArgs a) {
       }
       const bool valid = FULL || myrow[g] < a.n;
       double h, l;
-      row_terms(z, yv[g], a.loss_mode, a.identity_link, h, l);
+      row_terms(z + bias, yv[g], a.loss_mode, a.identity_link, h, l);
       const double res = valid ? (h - yv[g]) : 0.;
       h_keep[g] = h;
       h_row[g] = valid ? myrow[g] : -1;
-      if (valid) loss_acc += l;
+      if (valid) {
+        sums.loss += l;
+        sums.res += res;
+      }
       if (GRAD) {
 #pragma unroll
         for (int c = 0; c < SL; ++c) {
@@ -739,18 +791,7 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void packed_pass(PassArgs a) {
       *reinterpret_cast<v2d*>(a.part_g + (int64_t)blockIdx.x * P + 2 * lane) = s;
     }
   }
-  {
-    __shared__ double lx[WROW];
-    const double wl = wave_sum(loss_acc);
-    if (lane == 0) lx[wr] = wl;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      double s = 0.;
-#pragma unroll
-      for (int w = 0; w < WROW; ++w) s += lx[w];
-      a.part_loss[blockIdx.x] = s;
-    }
-  }
+  emit_row_sums<WROW>(sums, lane, wr, a.part_loss, a.part_res);
 }
 
 // ---------------------------------------------------------------------------
@@ -786,8 +827,9 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
 
   const v2d th_lo = *reinterpret_cast<const v2d*>(a.theta + 2 * q);
   const v2d th_hi = *reinterpret_cast<const v2d*>(a.theta + kWave + 2 * q);  // zero past the row
+  const double bias = a.theta_bias ? *a.theta_bias : 0.;
   v2d acc_lo = v2d{0., 0.}, acc_hi = v2d{0., 0.};
-  double loss_acc = 0.;
+  RowSums sums;
 
   const int64_t group = (int64_t)blockIdx.x * WROW + wr;
   const int64_t ngroups = (int64_t)gridDim.x * WROW;
@@ -856,11 +898,14 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
     for (int s = ilog2(G); s < 5; ++s) z += __shfl_xor(z, 1 << s, kWave);
 
     double h, l;
-    row_terms(z, yv, a.loss_mode, a.identity_link, h, l);
+    row_terms(z + bias, yv, a.loss_mode, a.identity_link, h, l);
     const double res = valid ? (h - yv) : 0.;
     h_keep = h;
     h_row = (valid && owner) ? myrow : -1;
-    if (valid && owner) loss_acc += l;
+    if (valid && owner) {
+      sums.loss += l;
+      sums.res += res;
+    }
     if (GRAD) {
 #pragma unroll
       for (int g = 0; g < G; ++g) {
@@ -909,18 +954,7 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
       if (hi_in) *reinterpret_cast<v2d*>(out + kWave + 2 * q) = hi;
     }
   }
-  {
-    __shared__ double lx[WROW];
-    const double wl = wave_sum(loss_acc);
-    if (lane == 0) lx[wr] = wl;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      double s = 0.;
-#pragma unroll
-      for (int w = 0; w < WROW; ++w) s += lx[w];
-      a.part_loss[blockIdx.x] = s;
-    }
-  }
+  emit_row_sums<WROW>(sums, lane, wr, a.part_loss, a.part_res);
 }
 
 // ---------------------------------------------------------------------------
@@ -974,6 +1008,8 @@ struct TeamArgs {
   int nteams;                // grid = nteams * nblk, nteams a multiple of kXcds
   int blk_chunks;            // 128-column chunks per block (a multiple of 8)
   int nch_rt;                // chunks per wave = blk_chunks / 8  (<= NCH)
+  const double* theta_bias;  // as in PassArgs
+  double* part_res;          // [nteams], or nullptr
   unsigned long long* zx;    // [nteams][kTeamSlots][nblk][2] exchange slots
   unsigned* status;          // [0]: set when a wait gave up
   unsigned spin_limit;
@@ -1030,7 +1066,8 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
     const double* tp = (c < a.nch_rt) ? a.theta + (c0 + c) * kChunkCols : a.zeros;
     thl[c * kWave] = *reinterpret_cast<const v2d*>(tp + 2 * lane);
   }
-  double loss_acc = 0.;
+  double loss_acc = 0., res_acc = 0.;
+  const double bias = a.theta_bias ? *a.theta_bias : 0.;
   bool gave_up = false;
 
   // Uniform base + 32-bit lane offset: no address registers per chunk.  A chunk
@@ -1128,13 +1165,14 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
     if (have_prev) {
       const int64_t row = team + (t - 1) * a.nteams;
       const double yv = a.y ? a.y[row] : 0.;
-      double z = 0.;
+      double z = bias;
       for (int b = 0; b < a.nblk; ++b) z += zp[par][b];
       double h, l;
       row_terms(z, yv, kLoss, kIdentity, h, l);
       const double res = h - yv;
       if (blk == 0 && threadIdx.x == 0) {
         loss_acc += l;
+        res_acc += res;
         if (a.h_out) store_h(a.h_out + row, h);
       }
       if (GRAD) {
@@ -1170,7 +1208,10 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
       if (c < my_nch && (c != ragged_c || lane_in_ragged))
         *reinterpret_cast<v2d*>(out + (int64_t)c * kChunkCols) = acc[c];
   }
-  if (blk == 0 && threadIdx.x == 0) a.part_loss[team] = loss_acc;
+  if (blk == 0 && threadIdx.x == 0) {
+    a.part_loss[team] = loss_acc;
+    if (a.part_res) a.part_res[team] = res_acc;
+  }
 }
 
 // Pure streaming read of a buffer with shard_pass's access pattern (a wave
@@ -1203,33 +1244,37 @@ __global__ __launch_bounds__(256) void residual_pass(const double* __restrict__ 
                                                      double* __restrict__ res,
                                                      double* __restrict__ h_out,
                                                      double* __restrict__ part_loss, int64_t n,
-                                                     unsigned loss_mode, int identity_link) {
-  __shared__ double lx[4];
-  double loss_acc = 0.;
+                                                     unsigned loss_mode, int identity_link,
+                                                     const double* __restrict__ theta_bias,
+                                                     double* __restrict__ part_res) {
+  const double bias = theta_bias ? *theta_bias : 0.;
+  RowSums sums;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
        i += (int64_t)gridDim.x * blockDim.x) {
     const double yv = y ? y[i] : 0.;
     double h, l;
-    row_terms(z[i], yv, loss_mode, identity_link, h, l);
+    row_terms(z[i] + bias, yv, loss_mode, identity_link, h, l);
     if (res) res[i] = h - yv;
     if (h_out) store_h(h_out + i, h);
-    loss_acc += l;
+    sums.loss += l;
+    sums.res += h - yv;
   }
-  const double wl = wave_sum(loss_acc);
-  if ((threadIdx.x & (kWave - 1)) == 0) lx[threadIdx.x / kWave] = wl;
-  __syncthreads();
-  if (threadIdx.x == 0) part_loss[blockIdx.x] = ((lx[0] + lx[1]) + lx[2]) + lx[3];
+  emit_row_sums<4>(sums, threadIdx.x & (kWave - 1), threadIdx.x / kWave, part_loss, part_res);
 }
 
 // theta arrives in pinned, device-mapped host memory; this one-workgroup
 // kernel moves it into the zero-padded device copy the pass reads.  A kernel
 // on the pass's own stream instead of a copy command: no hand-over between
 // the copy engine and the compute queue in front of every step.
+// skip = 1: host_theta[0] belongs to the constant first column, which the
+// shard does not store; it goes to dev_theta[bias_slot] and the rest moves up.
 __global__ __launch_bounds__(256) void stage_theta(const double* __restrict__ host_theta,
-                                                   double* __restrict__ dev_theta, int64_t d) {
-  for (int64_t i = threadIdx.x + (int64_t)blockIdx.x * blockDim.x; i < d;
+                                                   double* __restrict__ dev_theta, int64_t d,
+                                                   int skip, int64_t bias_slot) {
+  for (int64_t i = threadIdx.x + (int64_t)blockIdx.x * blockDim.x; i < d - skip;
        i += (int64_t)gridDim.x * blockDim.x)
-    dev_theta[i] = host_theta[i];
+    dev_theta[i] = host_theta[i + skip];
+  if (skip && blockIdx.x == 0 && threadIdx.x == 0) dev_theta[bias_slot] = host_theta[0];
 }
 
 // theta already on the device -> the zero-padded copy the pass reads: entries
@@ -1255,10 +1300,15 @@ struct FinishArgs {
   const double* part_g;   // [nparts][pitch]
   const double* part_loss;  // [nparts]
   const double* theta;
-  double* out;            // d doubles (gsum or delta), then out[d] = loss_sum
+  double* out;            // the gradient (or delta) of every column, then the loss sum
   int64_t pitch;
-  int64_t d;
+  int64_t d;              // stored columns: part_g[.][0 .. d)
   int64_t n;
+  // a constant first column that is not stored (PassArgs::theta_bias): its
+  // gradient is the sum of the residuals (part_res), its theta sits in
+  // *theta_bias; the stored columns then land at out[1 ..], the loss at out[d + 1]
+  const double* part_res;  // [nparts_loss], or nullptr
+  double* theta_bias;
   int nparts;             // rows of part_g
   int nparts_loss;        // entries of part_loss
   int delta_mode;         // 0: out = gsum; 1: out = -alpha*gsum - coff2*n*theta;
@@ -1301,7 +1351,7 @@ __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a
         g = -a.alpha * g - (a.coff2 * (double)a.n) * th;
         if (a.delta_mode == 2) a.theta_rw[col] = th + g;  // this thread owns column col
       }
-      a.out[col] = g;
+      a.out[col + (a.part_res ? 1 : 0)] = g;
     }
     __syncthreads();
   }
@@ -1318,8 +1368,31 @@ __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a
       for (int k = 1; k < kFinCols * kFinSlices / kWave; ++k) t += flat[threadIdx.x + k * kWave];
       t = wave_sum(t);
       if (threadIdx.x == 0) {
-        a.out[a.d] = t;
+        a.out[a.d + (a.part_res ? 1 : 0)] = t;
         if (a.loss_slot) *a.loss_slot = t;
+      }
+    }
+    if (a.part_res && a.have_grad) {  // the unstored constant column: same fold over its partials
+      __syncthreads();
+      double r = 0.;
+      for (int p = threadIdx.x; p < a.nparts_loss; p += kFinCols * kFinSlices) r += a.part_res[p];
+      sm[sl][cx] = r;
+      __syncthreads();
+      if (threadIdx.x < kWave) {
+        const double* flat = &sm[0][0];
+        double t = flat[threadIdx.x];
+#pragma unroll
+        for (int k = 1; k < kFinCols * kFinSlices / kWave; ++k) t += flat[threadIdx.x + k * kWave];
+        t = wave_sum(t);
+        if (threadIdx.x == 0) {
+          double g = t;
+          if (a.delta_mode) {
+            const double th = *a.theta_bias;
+            g = -a.alpha * g - (a.coff2 * (double)a.n) * th;
+            if (a.delta_mode == 2) *a.theta_bias = th + g;
+          }
+          a.out[0] = g;
+        }
       }
     }
   }

@@ -87,12 +87,14 @@ class Config:
 
     def __init__(self, name, n, d, seed, kind, scale, lam, lr=0.1, zero_prob=0.0,
                  outlier_mod=0, outlier_scale=1.0, theta_scale=1.0, theta_nonzero=1.0,
-                 theta0_zero=False):
+                 theta0_zero=False, bias_first=False):
         self.name, self.n, self.d, self.seed = name, n, d, seed
         self.spec = GenSpec(seed, kind, outlier_mod, scale, zero_prob, outlier_scale)
         self.lam, self.lr = lam, lr
         self.theta_scale, self.theta_nonzero = theta_scale, theta_nonzero
         self.theta0_zero = theta0_zero
+        # column 0 is the constant 1.0 the worker's parser prepends (lr.cpp:83)
+        self.bias_first = bias_first
 
     @property
     def alpha(self):
@@ -123,6 +125,8 @@ class Config:
         """Rows [row0, row0+nrows) of the shard and their labels.  `out` (a
         C-contiguous nrows x d array) is filled in place when given."""
         X = gen_X(self.spec, row0, nrows, self.d, threads, out=out)
+        if self.bias_first:
+            X[:, 0] = 1.0
         y = gen_labels(self.spec, row0, X, self.theta_star(), threads)
         return X, y
 
@@ -153,7 +157,10 @@ def configs():
         # that ends two columns past a chunk boundary (tail-stage kernel variant)
         "x_bias_10m_x_257": Config("x_bias_10m_x_257", 10_000_000, 257, 0x5EED0008, UNIFORM, 1.0,
                                    lam=0.001, outlier_mod=100, outlier_scale=100.0,
-                                   theta_scale=0.1),
+                                   theta_scale=0.1, bias_first=True),
+        # 2048 features + the bias column
+        "x_bias_1m_x_2049": Config("x_bias_1m_x_2049", 1_000_000, 2049, 0x5EED000C, NORMAL,
+                                   1.0 / np.sqrt(2049), lam=0.01, bias_first=True),
         # rows of 65..96 columns at HBM-resident size: the half-wave-per-row kernel
         "x_short_30m_x_66": Config("x_short_30m_x_66", 30_000_000, 66, 0x5EED0009, NORMAL,
                                    1.0 / np.sqrt(66), lam=0.01),

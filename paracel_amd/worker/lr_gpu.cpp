@@ -69,12 +69,16 @@ void logistic_regression_gpu::set_samples(const double* X, int64_t n, int64_t d,
                                           const double* y) {
   n_local = n;
   data_dim = d;
+  check(plr_set_option(gpu, "first_column_is_one", 0), "plr_set_option");  // rows as given
   check(plr_set_data(gpu, X, n, d, ldx, y), "plr_set_data");
   flat.clear();
   labels.clear();
 }
 
 void logistic_regression_gpu::upload() {
+  // rows built by local_parser / predict start with the bias 1.0 (lr.cpp:83,99):
+  // that column need not be kept in HBM
+  check(plr_set_option(gpu, "first_column_is_one", 1), "plr_set_option");
   check(plr_set_data(gpu, flat.data(), n_local, data_dim, data_dim, labels.data()),
         "plr_set_data");
   std::vector<double>().swap(flat);

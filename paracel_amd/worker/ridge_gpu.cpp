@@ -22,6 +22,9 @@ ridge_regression_gpu::ridge_regression_gpu(const std::string& hosts_dct_str,
       alpha(_alpha),
       beta(_beta) {
   check(plr_create(&gpu, device_id), "plr_create");
+  // every shard this worker uploads starts its rows with the bias 1.0
+  // (ridge.hpp:149,168): that column need not be kept in HBM
+  check(plr_set_option(gpu, "first_column_is_one", 1), "plr_set_option");
 }
 
 ridge_regression_gpu::~ridge_regression_gpu() { plr_destroy(gpu); }

@@ -212,6 +212,62 @@ def test_rows_wider_than_the_fused_kernels(plr, oracle, gen, n, d, two_sweeps):
     assert rel(t5, oracle.train_dgd(X, y, np.zeros(d), 0.1 / n, 0.005, 5)) <= 1e-10
 
 
+@pytest.mark.parametrize("n,d", [(300, 2), (1000, 3), (4099, 17), (2051, 65), (2000, 66), (999, 98),
+                                 (3001, 129), (40003, 257), (2051, 1001), (1500, 1025),
+                                 (700, 2049), (130, 4097), (70, 8193), (37, 16385), (90, 19458),
+                                 (200, 33001)])
+def test_constant_first_column_is_not_stored(plr, oracle, gen, n, d):
+    # "first_column_is_one": the bias column the file path prepends (lr.cpp:83) stays on the
+    # host; every result must be what the stored column gives (the oracle sees the full X)
+    from paracel_amd import PlrError
+
+    print("case n=%d d=%d" % (n, d), flush=True)
+    X, _, th = make(gen, n, d, seed=0xB1A5 + d)
+    X[:, 0] = 1.0
+    spec = gen.GenSpec(77, gen.NORMAL, 0, 1.0, 0.0, 1.0)
+    y = gen.gen_labels(spec, 0, X, gen.gen_vec(77, gen.STREAM_THETA_STAR, d, gen.NORMAL, 1.0))
+    plr.set_option("first_column_is_one", 1)
+    plr.set_data(X, y)
+    info = plr.kernel_info()
+    print(info, flush=True)
+    assert "not stored" in info and plr.shape == (n, d)
+    g, loss, n_out = plr.loss_grad(th)
+    g_ref = oracle.gsum(X, y, th)
+    assert n_out == n and g.shape == (d,)
+    assert rel(g, g_ref) <= GRAD_TOL
+    assert abs(g[0] - g_ref[0]) <= 1e-10 * max(abs(g_ref[0]), np.linalg.norm(g_ref) / d)
+    want = oracle.calc_loss_sum(X, y, th)
+    assert abs(loss - want) <= LOSS_TOL * want
+    delta, _ = plr.dgd_delta(th, 0.1 / n, 0.005)
+    assert rel(delta, oracle.dgd_delta(X, y, th, 0.1 / n, 0.005)) <= GRAD_TOL
+    l1, _ = plr.calc_loss(th, 1)
+    assert abs(l1 - want) <= LOSS_TOL * want
+    assert np.max(np.abs(plr.predict(th) - oracle.predict(X, th))) <= 1e-14
+    np.testing.assert_allclose(plr.predict_linear(th), X @ th, rtol=0, atol=1e-12)
+    t5 = plr.train_dgd(np.zeros(d), 0.1 / n, 0.005, 5)
+    assert rel(t5, oracle.train_dgd(X, y, np.zeros(d), 0.1 / n, 0.005, 5)) <= 1e-10
+    # chunked upload of the same shard, same bits
+    plr.alloc_data(n, d)
+    h = n // 2
+    plr.set_data_chunk(h, X[h:], y[h:])
+    plr.set_data_chunk(0, X[:h], y[:h])
+    g2, loss2, _ = plr.loss_grad(th)
+    np.testing.assert_array_equal(g, g2)
+    assert loss == loss2
+    # a row that does not start with 1.0 is refused, by row number
+    Xb = X.copy()
+    Xb[n // 3, 0] = 1.0000001
+    with pytest.raises(PlrError) as e:
+        plr.set_data(Xb, y)
+    assert e.value.code == -1 and "row %d" % (n // 3) in str(e.value)
+    # switched off again: the column is stored, same results to rounding
+    plr.set_option("first_column_is_one", 0)
+    plr.set_data(X, y)
+    assert "not stored" not in plr.kernel_info()
+    g3, loss3, _ = plr.loss_grad(th)
+    assert rel(g3, g) <= 1e-12 and abs(loss3 - loss) <= 1e-12 * loss
+
+
 def test_wide_row_exchange_gives_up_instead_of_hanging(plr, oracle, gen):
     # a workgroup that never hears from its partners must not spin for ever: with the poll
     # limit at 0 every wait that does not find its partial at the first look gives up, the
