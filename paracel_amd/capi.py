@@ -153,10 +153,18 @@ class Plr:
         self._check(self._lib.plr_alloc_data(self._h, n, d))
 
     def set_data_chunk(self, row0, X, y):
-        X = np.ascontiguousarray(X, dtype=np.float64)
-        y = _vec(y, X.shape[0], "y")
-        self._check(self._lib.plr_set_data_chunk(self._h, row0, X.shape[0], _p(X),
-                                                 X.shape[1], _p(y)))
+        X = np.asarray(X, dtype=np.float64)
+        if X.ndim != 2:
+            raise ValueError("X must be 2-D")
+        if X.shape[0] and X.strides[1] != 8:
+            X = np.ascontiguousarray(X)
+        m, d = X.shape
+        ldx = X.strides[0] // 8 if m > 1 else d
+        if ldx < d:
+            X = np.ascontiguousarray(X)
+            ldx = d
+        y = _vec(y, m, "y")
+        self._check(self._lib.plr_set_data_chunk(self._h, row0, m, _p(X), ldx, _p(y)))
 
     @property
     def shape(self):

@@ -84,24 +84,52 @@ const team_fn kTeam[2][5] = {
 constexpr int64_t kHostPredictCols = 192;  // from this pitch on predictions go straight to host
 constexpr unsigned kTeamSpinLimit = 1u << 22;  // polls before a wait for a partner gives up
 
-// Narrow rows (d <= 64): power-of-two pitch, several whole rows per chunk.
-struct PackedVariant {
-  int logp, U, wrow;
+// Narrow rows (d <= 64): row-tiled layout, a lane per row.
+struct LaneVariant {
+  int np, U, wrow;
   pass_fn fn[2];  // [grad]
 };
-#define PLR_PACKED(LOGP, U, WROW, MINW)                       \
-  {LOGP, U, WROW,                                             \
-   {plr::packed_pass<LOGP, U, WROW, MINW, false>, plr::packed_pass<LOGP, U, WROW, MINW, true>}}
-// indexed by log2(pitch) - 1; tile shapes from sweeps (6.3-7.0 TB/s for pitch
-// 8..64; pitch 2 and 4 are bound by one exp/log per 16-32 bytes)
-const PackedVariant kPacked[] = {
-    PLR_PACKED(1, 4, 4, 4),  // pitch 2
-    PLR_PACKED(2, 4, 4, 3),  // pitch 4
-    PLR_PACKED(3, 2, 4, 3),  // pitch 8
-    PLR_PACKED(4, 2, 4, 2),  // pitch 16
-    PLR_PACKED(5, 2, 2, 1),  // pitch 32
-    PLR_PACKED(6, 1, 2, 1),  // pitch 64
+#define PLR_LANE(NP, U, WROW, MINW)                       \
+  {NP, U, WROW,                                           \
+   {plr::lane_pass<NP, U, WROW, MINW, false>, plr::lane_pass<NP, U, WROW, MINW, true>}}
+// indexed by column pairs - 1; tiles per group, waves and register budget from
+// sweeps over every combination on 1.6 GB shards (6.45-6.9 TB/s from 6
+// columns up; 4 columns 5.9, 2 columns 4.2: one exp/log per 16-32 bytes)
+const LaneVariant kLane[] = {
+    PLR_LANE(1, 2, 2, 3),  // 2 columns
+    PLR_LANE(2, 2, 4, 3),
+    PLR_LANE(3, 4, 4, 1),
+    PLR_LANE(4, 1, 4, 3),
+    PLR_LANE(5, 2, 2, 3),
+    PLR_LANE(6, 2, 4, 3),
+    PLR_LANE(7, 1, 4, 4),
+    PLR_LANE(8, 1, 4, 2),  // 16 columns
+    PLR_LANE(9, 1, 4, 2),
+    PLR_LANE(10, 1, 4, 2),
+    PLR_LANE(11, 1, 4, 3),
+    PLR_LANE(12, 1, 4, 3),
+    PLR_LANE(13, 1, 4, 2),
+    PLR_LANE(14, 1, 4, 1),
+    PLR_LANE(15, 1, 2, 2),
+    PLR_LANE(16, 1, 2, 2),  // 32 columns
+    PLR_LANE(17, 2, 2, 1),
+    PLR_LANE(18, 1, 4, 2),
+    PLR_LANE(19, 1, 4, 1),
+    PLR_LANE(20, 1, 4, 1),
+    PLR_LANE(21, 1, 4, 1),
+    PLR_LANE(22, 2, 4, 1),
+    PLR_LANE(23, 1, 4, 1),
+    PLR_LANE(24, 1, 2, 1),
+    PLR_LANE(25, 1, 4, 1),
+    PLR_LANE(26, 1, 2, 1),
+    PLR_LANE(27, 1, 2, 1),
+    PLR_LANE(28, 1, 2, 1),
+    PLR_LANE(29, 1, 4, 1),
+    PLR_LANE(30, 2, 4, 1),
+    PLR_LANE(31, 1, 2, 1),
+    PLR_LANE(32, 1, 2, 1),  // 64 columns
 };
+static_assert(sizeof(kLane) / sizeof(kLane[0]) == plr_plan::kMaxLaneCols / 2, "one variant per width");
 
 // Rows of 65..96 columns: a half-wave per row, G row pairs per tile.
 struct PairVariant {
@@ -170,7 +198,9 @@ struct plr_ctx {
   int grid = 0, grid_nograd = 0;
   bool allch = false;
   int tail_cols = 0;            // columns handled by the variant's tail stage
-  const PackedVariant* packed = nullptr;  // d <= 64: packed-row kernel
+  const LaneVariant* lane = nullptr;      // d <= 64: row-tiled layout, lane_pass
+  int64_t n_alloc = 0;                    // rows the shard buffer holds (lane path: whole groups)
+  double* up_dev = nullptr;               // lane path: device staging of uploaded row-major rows
   const PairVariant* pair = nullptr;      // 65..96 columns: half-wave rows
   bool blocked = false;         // rows wider than the widest fused variant: column blocks
   // ... read once by teams of workgroups (team_blocks > 0), else in two sweeps
@@ -239,6 +269,8 @@ void release_upload_staging(plr_ctx* c) {
     c->up_stage[k] = nullptr;
   }
   c->up_stage_bytes = 0;
+  if (c->up_dev) (void)hipFree(c->up_dev);
+  c->up_dev = nullptr;
 }
 
 void free_shape(plr_ctx* c) {
@@ -273,7 +305,8 @@ void free_shape(plr_ctx* c) {
   c->have_data = false;
   c->curve_len = 0;
   c->blocked = false;
-  c->packed = nullptr;
+  c->lane = nullptr;
+  c->n_alloc = 0;
   c->pair = nullptr;
   c->tail_cols = 0;
   c->var = nullptr;
@@ -294,29 +327,29 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   c->nch_rt = pl.nch_rt;
   c->allch = pl.allch;
   c->tail_cols = pl.tail_cols;
-  if (pl.path == plr_plan::kPathPacked) {
-    const PackedVariant* pv = &kPacked[pl.logp - 1];
-    const int threads = plr::kWave * pv->wrow;
-    c->packed = pv;
-    c->var = &kBlockShape;  // unused by the packed path, kept non-null
+  if (pl.path == plr_plan::kPathLane) {
+    const LaneVariant* lv = &kLane[pl.np - 1];
+    const int threads = plr::kWave * lv->wrow;
+    c->lane = lv;
+    c->var = &kBlockShape;  // unused by this path, kept non-null
     c->nch_rt = 1;
     int occ = 0, occ2 = 0;
     PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                   &occ, reinterpret_cast<const void*>(pv->fn[1]), threads, 0));
+                   &occ, reinterpret_cast<const void*>(lv->fn[1]), threads, 0));
     PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                   &occ2, reinterpret_cast<const void*>(pv->fn[0]), threads, 0));
+                   &occ2, reinterpret_cast<const void*>(lv->fn[0]), threads, 0));
     if (occ < 1 || occ2 < 1)
       return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
-    const int64_t ntiles = ceil_div(n, (int64_t)plr::kWave * pv->U);
-    const int64_t want = std::max<int64_t>(1, ceil_div(ntiles, pv->wrow));
+    const int64_t ngroups = ceil_div(n, (int64_t)plr::kWave * lv->U);
+    const int64_t want = std::max<int64_t>(1, ceil_div(ngroups, lv->wrow));
     c->grid = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ);
     c->grid_nograd = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ2);
     char b[256];
     snprintf(b, sizeof b,
-             "packed_pass<pitch=%lld,U=%d,WROW=%d> %d rows per tile, grid=%d x %d threads "
-             "(occupancy %d blocks/CU, %d CUs)",
-             (long long)c->pitch, pv->U, pv->wrow, plr::kWave * pv->U, c->grid, threads, occ,
-             c->num_cu);
+             "lane_pass<NP=%d,U=%d,WROW=%d> row-tiled layout, pitch=%lld, %d rows per group, "
+             "grid=%d x %d threads (occupancy %d blocks/CU, %d CUs)",
+             lv->np, lv->U, lv->wrow, (long long)c->pitch, plr::kWave * lv->U, c->grid, threads,
+             occ, c->num_cu);
     c->info = b;
     return PLR_OK;
   }
@@ -440,16 +473,27 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
   // in 64 bits must be refused here, not wrap around to a small allocation
   // that the kernels would then stream far past
   const size_t slack_bytes = std::max<size_t>((size_t)c->theta_len * sizeof(double), 64u << 10);
-  if ((uint64_t)n > (UINT64_MAX / sizeof(double) - slack_bytes) / (uint64_t)c->pitch)
+  // the row-tiled layout holds whole groups of tiles; the rows past n are zeros
+  const int64_t group_rows = c->lane ? (int64_t)plr::kWave * c->lane->U : 1;
+  if (n > INT64_MAX - group_rows)
+    return fail(c, PLR_ERR_INVALID, "n * pitch * 8 bytes does not fit in 64 bits");
+  const int64_t n_alloc = ceil_div(n, group_rows) * group_rows;
+  if ((uint64_t)n_alloc > (UINT64_MAX / sizeof(double) - slack_bytes) / (uint64_t)c->pitch)
     return fail(c, PLR_ERR_INVALID, "n * pitch * 8 bytes does not fit in 64 bits");
   c->n = n;
+  c->n_alloc = n_alloc;
   c->d = d;
   // lanes of the chunk that straddles the end of the last row read (and then
   // discard) up to one slab past it: keep that much slack mapped
-  const size_t xbytes = (size_t)n * c->pitch * sizeof(double) + slack_bytes;
+  const size_t xbytes = (size_t)n_alloc * c->pitch * sizeof(double) + slack_bytes;
   if (n > 0) {
     PLR_HIP(c, hipMalloc(&c->dX, xbytes));
     PLR_HIP(c, hipMalloc(&c->dy, (size_t)n * sizeof(double)));
+    if (c->lane && !zero_fill) {
+      // the last group of tiles: its rows past n are never uploaded
+      const size_t last = (size_t)(n_alloc - group_rows) * c->pitch * sizeof(double);
+      PLR_HIP(c, hipMemsetAsync(reinterpret_cast<char*>(c->dX) + last, 0, xbytes - last, c->stream));
+    }
     if (zero_fill) {
       // a shard that is filled row range by row range: rows the caller never
       // sends must read as zeros, not as whatever the memory held
@@ -478,7 +522,7 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
   PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_out_dev), c->h_out, 0));
   memset(c->h_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double));
   PLR_HIP(c, hipMemsetAsync(c->d_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double), c->stream));
-  if (n > 0 && c->pitch != c->dcols)  // the pad column must read as zero
+  if (n > 0 && c->pitch != c->dcols && !c->lane)  // the pad column must read as zero
     PLR_HIP(c, hipMemset2DAsync(c->dX + c->dcols, (size_t)c->pitch * sizeof(double), 0,
                                 (size_t)(c->pitch - c->dcols) * sizeof(double), (size_t)n,
                                 c->stream));
@@ -517,7 +561,8 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
         return fail(c, PLR_ERR_INVALID, b);
       }
   }
-  if (!c->bias && ldx == c->pitch && c->d == c->pitch) {  // same pitch, no pad column: one linear copy
+  const bool tiled = c->lane != nullptr;
+  if (!tiled && !c->bias && ldx == c->pitch && c->d == c->pitch) {  // same pitch, no pad column: one linear copy
     PLR_HIP(c, hipMemcpy(c->dX + row0 * c->pitch, X,
                          (size_t)nrows * c->pitch * sizeof(double), hipMemcpyHostToDevice));
   } else {
@@ -525,8 +570,14 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
     // (~1 GB/s).  Repack the rows at the device pitch into two pinned staging
     // buffers on the host and send those as linear copies, the packing of one
     // overlapping the transfer of the other.
-    const int64_t chunk_rows = std::max<int64_t>(1, (int64_t)(32u << 20) / (c->pitch * 8));
-    const size_t stage_bytes = (size_t)chunk_rows * c->pitch * sizeof(double);
+    // Row-tiled shards: the rows go, stored columns only, into a staging
+    // buffer on the device, and tile_rows brings each block into the layout
+    // (same stream: the next block's copy waits for it).  Host rows that are
+    // already dense are sent from where they lie.
+    const int64_t sp = tiled ? c->dcols : c->pitch;  // pitch of the staged rows
+    const bool direct = tiled && !c->bias && ldx == c->dcols;
+    const int64_t chunk_rows = std::max<int64_t>(1, (int64_t)(32u << 20) / (sp * 8));
+    const size_t stage_bytes = (size_t)chunk_rows * sp * sizeof(double);
     int rc = PLR_OK;
     if (c->up_stage_bytes < stage_bytes) {  // kept for the shard's lifetime: chunked uploads reuse them
       release_upload_staging(c);
@@ -536,6 +587,10 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
           (void)hipGetLastError();
           rc = fail(c, PLR_ERR_NOMEM, "cannot allocate the pinned upload staging buffers");
         }
+      }
+      if (rc == PLR_OK && tiled && hipMalloc(&c->up_dev, stage_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        rc = fail(c, PLR_ERR_NOMEM, "cannot allocate the device upload staging buffer");
       }
       if (rc != PLR_OK) {
         release_upload_staging(c);
@@ -550,16 +605,26 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
       const int64_t m = std::min<int64_t>(chunk_rows, nrows - r0);
       if (r0 >= 2 * chunk_rows && hipEventSynchronize(done[k]) != hipSuccess)
         rc = fail(c, PLR_ERR_HIP, "upload: waiting for a staging buffer failed");
-      for (int64_t r = 0; r < m && rc == PLR_OK; ++r) {
-        double* dst = stage[k] + r * c->pitch;
+      for (int64_t r = 0; r < m && rc == PLR_OK && !direct; ++r) {
+        double* dst = stage[k] + r * sp;
         memcpy(dst, X + (r0 + r) * ldx + skip, (size_t)c->dcols * sizeof(double));
-        for (int64_t j = c->dcols; j < c->pitch; ++j) dst[j] = 0.;
+        for (int64_t j = c->dcols; j < sp; ++j) dst[j] = 0.;
       }
-      if (rc == PLR_OK &&
-          (hipMemcpyAsync(c->dX + (row0 + r0) * c->pitch, stage[k],
-                          (size_t)m * c->pitch * sizeof(double), hipMemcpyHostToDevice,
-                          c->stream) != hipSuccess ||
-           hipEventRecord(done[k], c->stream) != hipSuccess))
+      const double* src = direct ? X + r0 * ldx : stage[k];
+      double* dst = tiled ? c->up_dev : c->dX + (row0 + r0) * c->pitch;
+      if (rc == PLR_OK && hipMemcpyAsync(dst, src, (size_t)m * sp * sizeof(double),
+                                         hipMemcpyHostToDevice, c->stream) != hipSuccess)
+        rc = fail(c, PLR_ERR_HIP, "upload: host-to-device copy failed");
+      if (rc == PLR_OK && tiled) {
+        const int np = c->lane->np;
+        const int64_t threads = ceil_div(m, plr::kWave) * plr::kWave * np;
+        hipLaunchKernelGGL(plr::tile_rows, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
+                           c->stream, (const double*)c->up_dev, sp, m, (int)c->dcols, c->dX,
+                           row0 + r0, np);
+        if (hipGetLastError() != hipSuccess)
+          rc = fail(c, PLR_ERR_HIP, "upload: launching the tiling kernel failed");
+      }
+      if (rc == PLR_OK && hipEventRecord(done[k], c->stream) != hipSuccess)
         rc = fail(c, PLR_ERR_HIP, "upload: host-to-device copy failed");
     }
     if (hipStreamSynchronize(c->stream) != hipSuccess && rc == PLR_OK)
@@ -585,7 +650,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
   const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
   const int grid = grad ? c->grid : c->grid_nograd;
-  const int threads = c->packed ? plr::kWave * c->packed->wrow
+  const int threads = c->lane ? plr::kWave * c->lane->wrow
                       : c->pair ? plr::kWave * c->pair->wrow
                                 : plr::kWave * v->wcol * v->wrow;
 
@@ -612,8 +677,8 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   pa.res_in = nullptr;
 
   if (c->timing) PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
-  if (c->packed) {
-    hipLaunchKernelGGL(c->packed->fn[grad ? 1 : 0], dim3(grid), dim3(threads), 0, c->stream, pa);
+  if (c->lane) {
+    hipLaunchKernelGGL(c->lane->fn[grad ? 1 : 0], dim3(grid), dim3(threads), 0, c->stream, pa);
     PLR_HIP(c, hipGetLastError());
   } else if (c->pair) {
     hipLaunchKernelGGL(c->pair->fn[grad ? 1 : 0], dim3(grid), dim3(threads), 0, c->stream, pa);

@@ -280,12 +280,12 @@ __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
                                           const double* tile_base, int64_t row0,
                                           v2d (&x)[R][NCH], v2d (&xt)[TL > 0 ? TL : 1],
                                           double& yv) {
-  // The chunk that straddles the row end is loaded under the lane mask when it
-  // is the wave's last slot: lanes past the row end then request nothing
-  // (fewer cache lines touched per load).  Those loads are issued together,
-  // after all the others of the tile, so that the mask changes once per tile
-  // and the run of back-to-back loads stays unbroken.
-  const bool masked_last = w.ragged_c == NCH - 1;  // uniform
+  // The chunk that straddles the row end is loaded whole; compute_tile drops
+  // its lanes past the row end.  (Loading it under the lane mask instead, so
+  // that those lanes request nothing, was measured on 3 GB shards for every
+  // variant: 1-8 % slower from 98 to 3500 columns, whether the masked loads
+  // were interleaved with the others of the tile or issued as a group behind
+  // them.)
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const char* rowp = reinterpret_cast<const char*>(tile_base + (int64_t)r * a.pitch);
@@ -293,18 +293,9 @@ __device__ __forceinline__ void load_tile(const PassArgs& a, const WaveCtx& w,
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       x[r][c] = v2d{0., 0.};
-      if (rv && (ALLCH || c < w.my_nch) && !(c == NCH - 1 && masked_last))  // uniform
+      if (rv && (ALLCH || c < w.my_nch))  // uniform
         x[r][c] = load_x(reinterpret_cast<const v2d*>(
             rowp + w.lane_off + (uint32_t)(c * kChunkCols * sizeof(double))));
-    }
-  }
-  if (masked_last && w.lane_in_ragged) {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const char* rowp = reinterpret_cast<const char*>(tile_base + (int64_t)r * a.pitch);
-      if (FULL || (row0 + r) < a.n)  // uniform
-        x[r][NCH - 1] = load_x(reinterpret_cast<const v2d*>(
-            rowp + w.lane_off + (uint32_t)((NCH - 1) * kChunkCols * sizeof(double))));
     }
   }
   if constexpr (TL > 0) {
@@ -632,166 +623,152 @@ __global__ __launch_bounds__(kWave* WCOL* WROW, MINW) void shard_pass(PassArgs a
 }
 
 // ---------------------------------------------------------------------------
-// Narrow rows (d <= 64).  With a row shorter than a 128-column chunk most lanes
-// of shard_pass would idle, so the shard is stored with a power-of-two pitch
-// P = 2..64 and a chunk (128 consecutive doubles, one dwordx4 per lane) holds
-// 128/P WHOLE rows: lane l owns the column pair 2*(l % SL) of row l / SL of
-// every chunk, SL = P/2 lanes per row.  A group of SL chunks carries 64 rows;
-// the transposing butterfly over the SL lanes of a row leaves every lane with
-// ONE distinct row of the group, so the 64 lanes evaluate 64 different
-// sigmoids / loss terms at once.  The residuals travel back inside the row's
-// lane segment (ds_bpermute), the rank-1 update runs on the registers the
-// rows were loaded into, and the per-lane accumulators (one column pair
-// each) are folded over the segments once, at the end.  U groups per tile
-// keep 16-32 KiB of loads in flight per wave.
+// Narrow rows in the row-tiled layout: a lane per row.
+//
+// The library owns the layout of the shard in HBM, and for rows of at most 64
+// columns it stores tiles of 64 rows column pair by column pair:
+//   X[((tile * NP + p) * 64 + r) * 2 + {0, 1}] = columns 2p, 2p+1 of row 64*tile + r
+// (NP = ceil(d / 2) pairs; an odd d is padded with one zero column, rows are
+// padded with zero rows to whole groups of U tiles).  Lane r of a wave then
+// owns row r of a tile whatever the width: every load instruction moves a
+// dense 1 KiB, the dot product is a chain of FMAs inside the lane in column
+// order (the reference's own order, ext_utility.hpp:171-174) with theta
+// broadcast from LDS, all 64 lanes evaluate 64 different sigmoid / loss terms,
+// labels and predictions are dense 512-byte accesses, and the rank-1 update
+// needs no residual exchange.  The per-lane gradient accumulators are summed
+// over the lanes once, at the end of the kernel.
 //
 // Same reference loops as shard_pass (lr.cpp:69-72,132-138,322-330,361-363).
-template <int LOGP, int U, int WROW, int MINW, bool GRAD>
-__global__ __launch_bounds__(kWave* WROW, MINW) void packed_pass(PassArgs a) {
-  constexpr int P = 1 << LOGP;       // pitch in doubles
-  constexpr int SL = P / 2;          // lanes per row
-  constexpr int RPC = kWave / SL;    // rows per chunk
-  constexpr int kTileRows = kWave * U;
-  static_assert(LOGP >= 1 && LOGP <= 6, "packed rows are 2..64 doubles wide");
+// tile_rows (below) brings uploaded row-major rows into this layout.
+template <int NP, int U, int WROW, int MINW, bool GRAD>
+__global__ __launch_bounds__(kWave* WROW, MINW) void lane_pass(PassArgs a) {
+  static_assert(NP >= 1 && NP <= 32, "lane-per-row tiles hold rows of 2..64 columns");
   const int lane = threadIdx.x & (kWave - 1);
   const int wr = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int pos = lane & (SL - 1);   // which column pair of the row
-  const int seg = lane / SL;         // which row of a chunk
-  const int my_chunk = row_of_lane<SL>(pos);  // chunk of the group whose row ends up here
 
-  const v2d th = *reinterpret_cast<const v2d*>(a.theta + 2 * pos);
+  __shared__ v2d th_lds[NP];
+  if (threadIdx.x < NP) th_lds[threadIdx.x] = *reinterpret_cast<const v2d*>(a.theta + 2 * threadIdx.x);
+  __syncthreads();
   const double bias = a.theta_bias ? *a.theta_bias : 0.;
-  v2d acc = v2d{0., 0.};
+
+  v2d acc[NP];
+#pragma unroll
+  for (int p = 0; p < NP; ++p) acc[p] = v2d{0., 0.};
   RowSums sums;
-  // a tile's predictions are stored after the next tile's loads have been
+  // a group's predictions are stored after the next group's loads have been
   // issued (a store in front of them would have to be acknowledged first)
   double h_keep[U];
-  int64_t h_row[U];
+  int64_t h_row0 = -1;
 #pragma unroll
-  for (int g = 0; g < U; ++g) {
-    h_keep[g] = 0.;
-    h_row[g] = -1;
-  }
+  for (int u = 0; u < U; ++u) h_keep[u] = 0.;
   auto store_kept = [&]() {
-    if (a.h_out) {
+    if (a.h_out && h_row0 >= 0) {
 #pragma unroll
-      for (int g = 0; g < U; ++g)
-        if (h_row[g] >= 0) store_h(a.h_out + h_row[g], h_keep[g]);
+      for (int u = 0; u < U; ++u) {
+        const int64_t row = h_row0 + u * kWave;
+        if (row < a.n) store_h(a.h_out + row, h_keep[u]);
+      }
     }
   };
 
-  const int64_t group0 = (int64_t)blockIdx.x * WROW + wr;
-  const int64_t ngroups = (int64_t)gridDim.x * WROW;
-  const int64_t nfull = a.n / kTileRows;
-  const int64_t ntiles = (a.n + kTileRows - 1) / kTileRows;
-
-  auto tile_body = [&](int64_t tile, auto full_tag) {
-    constexpr bool FULL = decltype(full_tag)::value;
-    const int64_t row0 = tile * kTileRows;
-    const v2d* base = reinterpret_cast<const v2d*>(a.X + row0 * P) + lane;
-    v2d x[U][SL];
+  constexpr int64_t kGroupRows = (int64_t)kWave * U;
+  const int64_t ngroups = (a.n + kGroupRows - 1) / kGroupRows;
+  const int64_t stride = (int64_t)gridDim.x * WROW;
+#pragma clang loop unroll(disable)
+  for (int64_t g = (int64_t)blockIdx.x * WROW + wr; g < ngroups; g += stride) {
+    const v2d* base = reinterpret_cast<const v2d*>(a.X) + g * (U * NP * kWave) + lane;
+    v2d x[U][NP];
 #pragma unroll
-    for (int g = 0; g < U; ++g)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int c = 0; c < SL; ++c) {
-        const int k = g * SL + c;
-        x[g][c] = load_x(base + (int64_t)k * kWave);
-        if (!FULL && row0 + (int64_t)k * RPC + seg >= a.n) x[g][c] = v2d{0., 0.};
-      }
-    store_kept();
+      for (int p = 0; p < NP; ++p) x[u][p] = load_x(base + (u * NP + p) * kWave);
+    const int64_t row0 = g * kGroupRows + lane;
     double yv[U];
-    int64_t myrow[U];
 #pragma unroll
-    for (int g = 0; g < U; ++g) {
-      myrow[g] = row0 + ((int64_t)g * SL + my_chunk) * RPC + seg;
-      yv[g] = 0.;
-      if ((FULL || myrow[g] < a.n) && a.y) yv[g] = a.y[myrow[g]];
+    for (int u = 0; u < U; ++u) {
+      const int64_t row = row0 + u * kWave;
+      yv[u] = (a.y && row < a.n) ? a.y[row] : 0.;
     }
+    store_kept();
+    // keeps the theta reads inside the loop: hoisted, they would occupy
+    // 4 * NP registers next to x and acc
+    asm volatile("" ::: "memory");
 #pragma unroll
-    for (int g = 0; g < U; ++g) {
-      typename RowVec<SL>::type p;
+    for (int u = 0; u < U; ++u) {
+      double z = 0.;
 #pragma unroll
-      for (int c = 0; c < SL; ++c) {
-        const double t = fma(x[g][c].x, th.x, x[g][c].y * th.y);
-        if constexpr (SL == 1)
-          p = t;
-        else
-          p[c] = t;
+      for (int p = 0; p < NP; ++p) {
+        const v2d th = th_lds[p];
+        z = fma(x[u][p].x, th.x, z);
+        z = fma(x[u][p].y, th.y, z);
       }
-      // reduce over the SL lanes of a row; lane (seg, pos) keeps chunk my_chunk
-      double z;
-      if constexpr (SL == 1) {
-        z = p;
-      } else {
-#pragma unroll
-        for (int s = 0; s < ilog2(SL); ++s) {
-          const int cnt = SL >> (s + 1);
-          const int m = 1 << s;
-          const bool up = (lane & m) != 0;
-#pragma unroll
-          for (int k = 0; k < cnt; ++k) {
-            const double lo = p[k], hi = p[k + cnt];
-            const double send = up ? lo : hi;
-            const double keep = up ? hi : lo;
-            p[k] = keep + __shfl_xor(send, m, kWave);
-          }
-        }
-        z = p[0];
-      }
-      const bool valid = FULL || myrow[g] < a.n;
+      const bool valid = row0 + u * kWave < a.n;
       double h, l;
-      row_terms(z + bias, yv[g], a.loss_mode, a.identity_link, h, l);
-      const double res = valid ? (h - yv[g]) : 0.;
-      h_keep[g] = h;
-      h_row[g] = valid ? myrow[g] : -1;
+      row_terms(z + bias, yv[u], a.loss_mode, a.identity_link, h, l);
+      const double res = valid ? (h - yv[u]) : 0.;
+      h_keep[u] = h;
       if (valid) {
         sums.loss += l;
         sums.res += res;
       }
       if (GRAD) {
 #pragma unroll
-        for (int c = 0; c < SL; ++c) {
-          // the residual of this lane's row in chunk c sits in the lane of
-          // the same segment that kept chunk c
-          const double rr =
-              (SL == 1) ? res : __shfl(res, (lane & ~(SL - 1)) | lane_of_row<SL>(c), kWave);
-          acc.x = fma(rr, x[g][c].x, acc.x);
-          acc.y = fma(rr, x[g][c].y, acc.y);
+        for (int p = 0; p < NP; ++p) {
+          acc[p].x = fma(res, x[u][p].x, acc[p].x);
+          acc[p].y = fma(res, x[u][p].y, acc[p].y);
         }
       }
     }
-  };
-
-  int64_t tile = group0;
-#pragma clang loop unroll(disable)
-  for (; tile < nfull; tile += ngroups) tile_body(tile, std::true_type{});
-  if (tile < ntiles) tile_body(tile, std::false_type{});
+    h_row0 = row0;
+  }
   store_kept();
 
   if (GRAD) {
-    // fold the row segments: lanes 0..SL-1 end up with the wave's totals
+    __shared__ v2d gx[(WROW > 1) ? (WROW - 1) * NP : 1];
 #pragma unroll
-    for (int m = SL; m < kWave; m <<= 1) {
-      acc.x += __shfl_xor(acc.x, m, kWave);
-      acc.y += __shfl_xor(acc.y, m, kWave);
+    for (int p = 0; p < NP; ++p) {
+      acc[p].x = wave_sum(acc[p].x);
+      acc[p].y = wave_sum(acc[p].y);
+      if (WROW > 1 && wr > 0 && lane == 0) gx[(wr - 1) * NP + p] = acc[p];
     }
-    __shared__ v2d gx[(WROW > 1) ? (WROW - 1) * SL : 1];
-    if (WROW > 1) {
-      if (wr > 0 && lane < SL) gx[(wr - 1) * SL + lane] = acc;
-      __syncthreads();
-    }
-    if (wr == 0 && lane < SL) {
-      v2d s = acc;
+    if (WROW > 1) __syncthreads();
+    if (wr == 0 && lane == 0) {
 #pragma unroll
-      for (int w = 1; w < WROW; ++w) {
-        const v2d o = gx[(w - 1) * SL + lane];
-        s.x += o.x;
-        s.y += o.y;
+      for (int p = 0; p < NP; ++p) {
+        v2d s = acc[p];
+#pragma unroll
+        for (int w = 1; w < WROW; ++w) {
+          const v2d o = gx[(w - 1) * NP + p];
+          s.x += o.x;
+          s.y += o.y;
+        }
+        *reinterpret_cast<v2d*>(a.part_g + (int64_t)blockIdx.x * (2 * NP) + 2 * p) = s;
       }
-      *reinterpret_cast<v2d*>(a.part_g + (int64_t)blockIdx.x * P + 2 * lane) = s;
     }
   }
   emit_row_sums<WROW>(sums, lane, wr, a.part_loss, a.part_res);
+}
+
+// Row-major rows (src: nrows x src_pitch doubles, the first `cols` of each
+// used) into the row-tiled layout above, as rows row0 .. row0+nrows-1 of the
+// shard.  One thread per (row, column pair); columns at or past `cols` are
+// written as zeros.  Runs once per uploaded block of rows.
+__global__ void tile_rows(const double* src, int64_t src_pitch, int64_t nrows, int cols,
+                          double* X, int64_t row0, int np) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  // consecutive threads take consecutive rows of one column pair: the stores
+  // of a wave are one dense KiB
+  const int64_t blk = i / ((int64_t)kWave * np);       // block of 64 source rows
+  const int rem = (int)(i % ((int64_t)kWave * np));
+  const int p = rem / kWave, r = rem % kWave;
+  const int64_t srow = blk * kWave + r;
+  if (srow >= nrows) return;
+  const double* sp = src + srow * src_pitch + 2 * p;
+  v2d v;
+  v.x = (2 * p < cols) ? sp[0] : 0.;
+  v.y = (2 * p + 1 < cols) ? sp[1] : 0.;
+  const int64_t row = row0 + srow;
+  reinterpret_cast<v2d*>(X)[((row / kWave) * np + p) * kWave + (row % kWave)] = v;
 }
 
 // ---------------------------------------------------------------------------

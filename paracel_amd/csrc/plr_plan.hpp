@@ -1,5 +1,5 @@
 // Width -> layout and kernel variant, as a pure host function (no HIP types):
-// which of the three paths a shard of d columns takes, its row pitch in HBM,
+// which of the four paths a shard of d columns takes, its row pitch in HBM,
 // and for the fused path the shard_pass variant with its run-time chunk
 // count.  Kept apart from the kernels so that the choice can be checked on a
 // CPU for every width (the GPU side then only adds occupancy and grid size).
@@ -10,7 +10,7 @@
 namespace plr_plan {
 
 constexpr int kChunkCols = 128;          // columns per chunk (a double2 per lane)
-constexpr int64_t kMaxPackedCols = 64;   // up to here: packed rows, power-of-two pitch
+constexpr int64_t kMaxLaneCols = 64;     // up to here: row-tiled layout, a lane per row (lane_pass)
 constexpr int64_t kMaxPairPitch = 96;    // up to this pitch: a half-wave per row (pair_pass)
 constexpr int64_t kMaxFusedCols = 19456; // beyond: column blocks, two sweeps over X
 constexpr int kBlkNch = 16, kBlkWcol = 8;
@@ -33,14 +33,14 @@ static const Shape kShapes[] = {
 };
 constexpr int kNumShapes = (int)(sizeof(kShapes) / sizeof(kShapes[0]));
 
-enum Path { kPathPacked = 0, kPathFused = 1, kPathBlocked = 2, kPathPair = 3 };
+enum Path { kPathLane = 0, kPathFused = 1, kPathBlocked = 2, kPathPair = 3 };
 
 struct Plan {
   Path path;
   int64_t pitch;      // doubles per row in HBM (>= d; pad columns are zero)
   int64_t theta_len;  // doubles of the zero-padded device copy of theta
-  // packed path
-  int logp;           // log2(pitch)
+  // lane path: tiles of 64 rows stored column pair by column pair
+  int np;             // column pairs per row = pitch / 2
   // fused path
   int variant;        // index into kShapes
   int64_t chunks;     // ceil(pitch / 128)
@@ -60,12 +60,10 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool plan_width(int64_t d, Plan& p) {
   p = Plan();
   p.variant = -1;
-  if (d <= kMaxPackedCols) {
-    int logp = 1;
-    while ((int64_t(1) << logp) < d) ++logp;
-    p.path = kPathPacked;
-    p.logp = logp;
-    p.pitch = int64_t(1) << logp;
+  if (d <= kMaxLaneCols) {
+    p.path = kPathLane;
+    p.np = (int)((d + 1) / 2);
+    p.pitch = 2 * (int64_t)p.np;
     p.theta_len = kChunkCols;
     return true;
   }

@@ -25,10 +25,10 @@ static void print_plan(int64_t d) {
     printf("d=%lld: no variant\n", (long long)d);
     return;
   }
-  static const char* names[] = {"packed", "fused", "blocked", "pair"};
+  static const char* names[] = {"lane", "fused", "blocked", "pair"};
   printf("d=%lld path=%s pitch=%lld theta_len=%lld", (long long)d, names[p.path],
          (long long)p.pitch, (long long)p.theta_len);
-  if (p.path == kPathPacked) printf(" logp=%d", p.logp);
+  if (p.path == kPathLane) printf(" np=%d", p.np);
   if (p.path == kPathFused) {
     const Shape& s = kShapes[p.variant];
     printf(" variant=%d NCH=%d R=%d WCOL=%d WROW=%d THL=%d TL=%d chunks=%lld nch_rt=%d allch=%d tail=%d",
@@ -52,14 +52,13 @@ int main(int argc, char** argv) {
       continue;
     }
     CHECK(p.pitch >= d && p.pitch % 2 == 0, d);
-    CHECK(p.theta_len >= p.pitch || p.path == kPathPacked, d);
+    CHECK(p.theta_len >= p.pitch, d);
     CHECK(p.path != kPathFused || p.pitch > kMaxPairPitch, d);
-    if (p.path == kPathPacked) {
-      CHECK(d <= kMaxPackedCols && p.logp >= 1 && p.logp <= 6, d);
-      CHECK(p.pitch == (int64_t(1) << p.logp) && (p.pitch / 2 < d || d == 1), d);
-      CHECK(p.theta_len >= p.pitch, d);
+    if (p.path == kPathLane) {
+      CHECK(d <= kMaxLaneCols && p.np >= 1 && p.np <= 32, d);
+      CHECK(p.pitch == 2 * p.np && p.pitch - d < 2, d);
     } else if (p.path == kPathPair) {
-      CHECK(d > kMaxPackedCols && p.pitch <= kMaxPairPitch && p.pitch - d < 2, d);
+      CHECK(d > kMaxLaneCols && p.pitch <= kMaxPairPitch && p.pitch - d < 2, d);
       CHECK(p.theta_len >= kChunkCols, d);  // both column pairs of every lane read theta
     } else if (p.path == kPathBlocked) {
       CHECK(d > kMaxFusedCols && p.pitch % 16 == 0 && p.pitch - d < 16, d);
@@ -76,7 +75,7 @@ int main(int argc, char** argv) {
         CHECK(ceil_div(p.pitch, kChunkCols) > (int64_t)kMaxTeamBlocks * kBlkWcol * kTeamNch, d);
       }
     } else {
-      CHECK(d > kMaxPackedCols && d <= kMaxFusedCols, d);
+      CHECK(d > kMaxLaneCols && d <= kMaxFusedCols, d);
       CHECK(p.variant >= 0 && p.variant < kNumShapes, d);
       if (p.variant < 0 || p.variant >= kNumShapes) continue;
       const Shape& s = kShapes[p.variant];

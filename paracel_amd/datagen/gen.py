@@ -169,10 +169,13 @@ def configs():
         # config 1's shape (the reference tutorial's 100 features) at HBM-resident size
         "x_c1shape_20m_x_100": Config("x_c1shape_20m_x_100", 20_000_000, 100, 0x5EED000B, NORMAL,
                                       1.0, lam=0.01, theta0_zero=True),
-        # narrow rows: the packed-row kernel (several whole rows per 128-double chunk)
+        # narrow rows: the row-tiled layout, a lane per row
         "x_narrow_30m_x_16": Config("x_narrow_30m_x_16", 30_000_000, 16, 0x5EED0007, NORMAL, 0.25,
                                     lam=0.01),
-        # wider than the widest fused kernel: the column-blocked two-sweep path
+        # ... at a width that is neither a power of two nor even
+        "x_narrow_10m_x_41": Config("x_narrow_10m_x_41", 10_000_000, 41, 0x5EED000D, NORMAL,
+                                    1.0 / np.sqrt(41), lam=0.01),
+        # wider than the widest one-workgroup kernel: column blocks, a team of workgroups per row
         "x_verywide_100k_x_32768": Config("x_verywide_100k_x_32768", 100_000, 32768, 0x5EED0006,
                                           NORMAL, 1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
         # end-to-end through the host parameter server

@@ -300,8 +300,9 @@ NARROW = [(n, d) for d in (1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 48, 63, 64)
 
 
 @pytest.mark.parametrize("n,d", NARROW)
-def test_narrow_rows_packed_kernel(plr, oracle, gen, n, d):
-    # d <= 64: power-of-two device pitch, several whole rows per 128-double chunk
+def test_narrow_rows_lane_per_row(plr, oracle, gen, n, d):
+    # d <= 64: the shard is stored in tiles of 64 rows, column pair by column pair, and a
+    # lane owns a row
     print("case n=%d d=%d" % (n, d), flush=True)
     X, y, th = make(gen, n, d, scale=1.0 / np.sqrt(d), theta_scale=1.0)
     plr.set_data(X, y)
@@ -324,6 +325,42 @@ def test_narrow_rows_packed_kernel(plr, oracle, gen, n, d):
         assert abs(lq - wq) <= 1e-12 * wq
         np.testing.assert_allclose(plr.predict_linear(th), oracle.predict_linear(X, th), rtol=0,
                                    atol=1e-13)
+
+
+def test_every_narrow_width_and_the_tiling_of_uploaded_rows(plr, oracle, gen):
+    # every width of the row-tiled layout, rows sent in pieces that start and end inside a
+    # tile, from host rows with a stride, and with the constant first column left on the host
+    for d in range(1, 65):
+        n = 64 * 9 + (d * 7) % 61
+        print("case d=%d n=%d" % (d, n), flush=True)
+        X, y, th = make(gen, n, d, scale=1.0 / np.sqrt(d), theta_scale=1.0)
+        want_g, want_l = oracle.gsum(X, y, th), oracle.calc_loss_sum(X, y, th)
+        plr.set_data(X, y)
+        g, loss, _ = plr.loss_grad(th)
+        assert rel(g, want_g) <= GRAD_TOL and abs(loss - want_l) <= LOSS_TOL * want_l
+        # the same rows in three pieces, out of order, the host rows 3 doubles apart
+        wide = np.zeros((n, d + 3))
+        wide[:, :d] = X
+        cuts = [0, 37 + d, 64 * 5 - 1, n]
+        plr.alloc_data(n, d)
+        for k in (2, 0, 1):
+            lo, hi = cuts[k], cuts[k + 1]
+            plr.set_data_chunk(lo, wide[lo:hi, :d], y[lo:hi])
+        g2, loss2, _ = plr.loss_grad(th)
+        np.testing.assert_array_equal(g2, g)
+        assert loss2 == loss
+        np.testing.assert_allclose(plr.predict(th), oracle.predict(X, th), rtol=0, atol=1e-14)
+        if d >= 2:
+            Xb = X.copy()
+            Xb[:, 0] = 1.0
+            plr.set_option("first_column_is_one", 1)
+            try:
+                plr.set_data(Xb, y)
+                gb, lb, _ = plr.loss_grad(th)
+            finally:
+                plr.set_option("first_column_is_one", 0)
+            wl = oracle.calc_loss_sum(Xb, y, th)
+            assert rel(gb, oracle.gsum(Xb, y, th)) <= GRAD_TOL and abs(lb - wl) <= LOSS_TOL * wl
 
 
 def test_theta_zero_closed_forms(plr, gen):

@@ -43,5 +43,7 @@ def test_the_benchmark_shapes_take_the_intended_variants():
     assert (p["NCH"], p["R"], p["WCOL"]) == ("4", "16", "1")
     p = plan(257)        # 256 features + bias: two chunks and a two-column tail
     assert (p["NCH"], p["TL"], p["tail"], p["pitch"]) == ("2", "1", "2", "258")
-    assert plan(16)["path"] == "packed" and plan(64)["logp"] == "6"
+    assert plan(16)["path"] == "lane" and plan(64)["np"] == "32"
+    assert plan(41)["np"] == "21" and plan(41)["pitch"] == "42"   # no padding beyond an even width
+    assert plan(65)["path"] == "pair"
     assert plan(19456)["path"] == "fused" and plan(19457)["path"] == "blocked"
