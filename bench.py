@@ -39,29 +39,57 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # uses, so a changed variant choice yields null instead of a stale figure.
 MEASURED_TRAFFIC = {
     "c2_headline_1m_x_1000": (
-        1000000, "shard_pass<NCH=8,R=4,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=8 tail=0 pitch=1000 "
-        "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)", 8056281406,
+        1000000, "shard_pass<NCH=8,R=4,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=8 tail=0 "
+        "pitch=1000 grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)", 8053921965,
         "profiles/shard_pass_c2_headline_1m_x_1000.md"),
     "c3_tall_10m_x_256": (
-        10000000, "shard_pass<NCH=2,R=32,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=2 tail=0 pitch=256 "
-        "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)", 20560480416,
+        10000000, "shard_pass<NCH=2,R=32,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=2 tail=0 "
+        "pitch=256 grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)", 20560491247,
         "profiles/shard_pass_c3_tall_10m_x_256.md"),
     "c4_wide_200k_x_16384": (
-        200000, "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=0> nch_rt=16 tail=0 pitch=16384 "
-        "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26261496415,
+        200000, "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=0> nch_rt=16 tail=0 "
+        "pitch=16384 grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26261495689,
         "profiles/shard_pass_c4_wide_200k_x_16384.md"),
     "c4b_wide_200k_x_16385": (
-        200000, "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=1> nch_rt=16 tail=16 pitch=16400 "
-        "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26287132305,
+        200000, "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=1> nch_rt=16 tail=16 "
+        "pitch=16400 grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26287140587,
         "profiles/shard_pass_c4b_wide_200k_x_16385.md"),
     "c5_e2e_2m_x_512": (
-        2000000, "shard_pass<NCH=4,R=16,WCOL=1,WROW=2,ALLCH=1,TL=0> nch_rt=4 tail=0 pitch=512 "
-        "grid=512 x 128 threads (occupancy 2 blocks/CU, 256 CUs)", 8210208784,
+        2000000, "shard_pass<NCH=4,R=16,WCOL=1,WROW=2,ALLCH=1,TL=0> nch_rt=4 tail=0 "
+        "pitch=512 grid=512 x 128 threads (occupancy 2 blocks/CU, 256 CUs)", 8210221472,
         "profiles/shard_pass_c5_e2e_2m_x_512.md"),
+    "x_short_30m_x_66": (
+        30000000, "pair_pass<G=8,WROW=4> pitch=66, 16 rows per tile, grid=512 x 256 "
+        "threads (occupancy 2 blocks/CU, 256 CUs)", 16139391035,
+        "profiles/pair_pass_x_short_30m_x_66.md"),
+    "x_short_30m_x_72": (
+        30000000, "pair_pass<G=8,WROW=4> pitch=72, 16 rows per tile, grid=512 x 256 "
+        "threads (occupancy 2 blocks/CU, 256 CUs)", 17582792859,
+        "profiles/pair_pass_x_short_30m_x_72.md"),
+    "x_c1shape_20m_x_100": (
+        20000000, "shard_pass<NCH=1,R=16,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=1 tail=0 "
+        "pitch=100 grid=512 x 256 threads (occupancy 2 blocks/CU, 256 CUs)", 16453025582,
+        "profiles/shard_pass_x_c1shape_20m_x_100.md"),
     "x_bias_10m_x_257": (
-        10000000, "shard_pass<NCH=2,R=16,WCOL=1,WROW=4,ALLCH=1,TL=1> nch_rt=2 tail=2 pitch=258 "
-        "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)", 21175219596,
-        "profiles/shard_pass_tail_stage_x_bias_10m_x_257.md"),
+        10000000, "shard_pass<NCH=2,R=32,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=2 tail=0 "
+        "pitch=256 grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs); first column constant 1, not stored", 20560610893,
+        "profiles/shard_pass_x_bias_10m_x_257.md"),
+    "x_bias_1m_x_2049": (
+        1000000, "shard_pass<NCH=16,R=2,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=16 tail=0 "
+        "pitch=2048 grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs); first column constant 1, not stored", 16404274547,
+        "profiles/shard_pass_x_bias_1m_x_2049.md"),
+    "x_narrow_30m_x_16": (
+        30000000, "lane_pass<NP=8,U=1,WROW=4> row-tiled layout, pitch=16, 64 rows per "
+        "group, grid=768 x 256 threads (occupancy 3 blocks/CU, 256 CUs)", 4080193979,
+        "profiles/lane_pass_x_narrow_30m_x_16.md"),
+    "x_narrow_10m_x_41": (
+        10000000, "lane_pass<NP=21,U=1,WROW=4> row-tiled layout, pitch=42, 64 rows per "
+        "group, grid=512 x 256 threads (occupancy 2 blocks/CU, 256 CUs)", 3440406063,
+        "profiles/lane_pass_x_narrow_10m_x_41.md"),
+    "x_verywide_100k_x_32768": (
+        100000, "team_pass<NCH=8> 4 column blocks of 64 chunks, 64 teams, pitch=32768 "
+        "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26284495840,
+        "profiles/team_pass_x_verywide_100k_x_32768.md"),
 }
 
 # The other configurations a default run times after the headline.
