@@ -83,9 +83,9 @@ MEASURED_TRAFFIC = {
         "group, grid=768 x 256 threads (occupancy 3 blocks/CU, 256 CUs)", 4080193979,
         "profiles/lane_pass_x_narrow_30m_x_16.md"),
     "x_narrow_10m_x_41": (
-        10000000, "lane_pass<NP=21,U=1,WROW=4> row-tiled layout, pitch=42, 64 rows per "
-        "group, grid=512 x 256 threads (occupancy 2 blocks/CU, 256 CUs)", 3440406063,
-        "profiles/lane_pass_x_narrow_10m_x_41.md"),
+        10000000, "lane2_pass<NP=21,U=2,WROW=1> row-tiled layout, pitch=42, 128 rows per "
+        "group, grid=1024 x 128 threads (occupancy 4 blocks/CU, 256 CUs)", 3440511974,
+        "profiles/lane2_pass_x_narrow_10m_x_41.md"),
     "x_verywide_100k_x_32768": (
         100000, "team_pass<NCH=8> 4 column blocks of 64 chunks, 64 teams, pitch=32768 "
         "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26284495840,

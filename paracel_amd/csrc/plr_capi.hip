@@ -86,15 +86,18 @@ constexpr unsigned kTeamSpinLimit = 1u << 22;  // polls before a wait for a part
 
 // Narrow rows (d <= 64): row-tiled layout, a lane per row.
 struct LaneVariant {
-  int np, U, wrow;
-  pass_fn fn[2];  // [grad]
+  int np, U, wrow, wcol;  // wcol 2: a pair of waves shares every tile (lane2_pass)
+  pass_fn fn[2];          // [grad]
 };
 #define PLR_LANE(NP, U, WROW, MINW)                       \
-  {NP, U, WROW,                                           \
+  {NP, U, WROW, 1,                                        \
    {plr::lane_pass<NP, U, WROW, MINW, false>, plr::lane_pass<NP, U, WROW, MINW, true>}}
+#define PLR_LANE2(NP, U, MINW) \
+  {NP, U, 1, 2, {plr::lane2_pass<NP, U, MINW, false>, plr::lane2_pass<NP, U, MINW, true>}}
 // indexed by column pairs - 1; tiles per group, waves and register budget from
-// sweeps over every combination on 1.6 GB shards (6.45-6.9 TB/s from 6
-// columns up; 4 columns 5.9, 2 columns 4.2: one exp/log per 16-32 bytes)
+// sweeps over every combination on 1.6 GB shards (6.75-7.0 TB/s from 6
+// columns up; 4 columns 5.9, 2 columns 4.2: one exp/log per 16-32 bytes).
+// From 30 columns on a wave pair per tile is faster than a wave (+1-7 %).
 const LaneVariant kLane[] = {
     PLR_LANE(1, 2, 2, 3),  // 2 columns
     PLR_LANE(2, 2, 4, 3),
@@ -110,24 +113,24 @@ const LaneVariant kLane[] = {
     PLR_LANE(12, 1, 4, 3),
     PLR_LANE(13, 1, 4, 2),
     PLR_LANE(14, 1, 4, 1),
-    PLR_LANE(15, 1, 2, 2),
-    PLR_LANE(16, 1, 2, 2),  // 32 columns
-    PLR_LANE(17, 2, 2, 1),
-    PLR_LANE(18, 1, 4, 2),
-    PLR_LANE(19, 1, 4, 1),
-    PLR_LANE(20, 1, 4, 1),
-    PLR_LANE(21, 1, 4, 1),
-    PLR_LANE(22, 2, 4, 1),
-    PLR_LANE(23, 1, 4, 1),
-    PLR_LANE(24, 1, 2, 1),
-    PLR_LANE(25, 1, 4, 1),
-    PLR_LANE(26, 1, 2, 1),
-    PLR_LANE(27, 1, 2, 1),
-    PLR_LANE(28, 1, 2, 1),
-    PLR_LANE(29, 1, 4, 1),
-    PLR_LANE(30, 2, 4, 1),
-    PLR_LANE(31, 1, 2, 1),
-    PLR_LANE(32, 1, 2, 1),  // 64 columns
+    PLR_LANE2(15, 2, 2),  // 30 columns
+    PLR_LANE2(16, 2, 2),  // 32 columns
+    PLR_LANE2(17, 2, 2),
+    PLR_LANE2(18, 2, 2),
+    PLR_LANE2(19, 2, 2),
+    PLR_LANE2(20, 2, 2),
+    PLR_LANE2(21, 2, 2),
+    PLR_LANE2(22, 2, 2),
+    PLR_LANE2(23, 2, 2),
+    PLR_LANE2(24, 2, 2),
+    PLR_LANE2(25, 1, 2),  // 50 columns
+    PLR_LANE2(26, 1, 2),
+    PLR_LANE2(27, 1, 2),
+    PLR_LANE2(28, 1, 2),
+    PLR_LANE2(29, 1, 2),
+    PLR_LANE2(30, 1, 2),
+    PLR_LANE2(31, 1, 2),
+    PLR_LANE2(32, 1, 2),  // 64 columns
 };
 static_assert(sizeof(kLane) / sizeof(kLane[0]) == plr_plan::kMaxLaneCols / 2, "one variant per width");
 
@@ -329,7 +332,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   c->tail_cols = pl.tail_cols;
   if (pl.path == plr_plan::kPathLane) {
     const LaneVariant* lv = &kLane[pl.np - 1];
-    const int threads = plr::kWave * lv->wrow;
+    const int threads = plr::kWave * lv->wrow * lv->wcol;
     c->lane = lv;
     c->var = &kBlockShape;  // unused by this path, kept non-null
     c->nch_rt = 1;
@@ -346,9 +349,9 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
     c->grid_nograd = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ2);
     char b[256];
     snprintf(b, sizeof b,
-             "lane_pass<NP=%d,U=%d,WROW=%d> row-tiled layout, pitch=%lld, %d rows per group, "
+             "%s<NP=%d,U=%d,WROW=%d> row-tiled layout, pitch=%lld, %d rows per group, "
              "grid=%d x %d threads (occupancy %d blocks/CU, %d CUs)",
-             lv->np, lv->U, lv->wrow, (long long)c->pitch, plr::kWave * lv->U, c->grid, threads,
+             lv->wcol == 2 ? "lane2_pass" : "lane_pass", lv->np, lv->U, lv->wrow, (long long)c->pitch, plr::kWave * lv->U, c->grid, threads,
              occ, c->num_cu);
     c->info = b;
     return PLR_OK;
@@ -650,7 +653,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
   const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
   const int grid = grad ? c->grid : c->grid_nograd;
-  const int threads = c->lane ? plr::kWave * c->lane->wrow
+  const int threads = c->lane ? plr::kWave * c->lane->wrow * c->lane->wcol
                       : c->pair ? plr::kWave * c->pair->wrow
                                 : plr::kWave * v->wcol * v->wrow;
 

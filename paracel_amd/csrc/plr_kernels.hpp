@@ -749,6 +749,123 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void lane_pass(PassArgs a) {
   emit_row_sums<WROW>(sums, lane, wr, a.part_loss, a.part_res);
 }
 
+// lane_pass for the wider tiles (34..64 columns), where rows and accumulators
+// of a whole tile fill the registers of a wave (one wave per SIMD): a PAIR of
+// waves shares every tile, each holding half of the column pairs of the same
+// 64 rows, so that twice as many waves fit.  The halves of a row's dot product
+// meet in LDS (double-buffered, one barrier per group of tiles; a workgroup is
+// one pair, so the barrier couples nobody else) and are added in wave order;
+// both waves then evaluate the row terms and update their own columns.
+template <int NP, int U, int MINW, bool GRAD>
+__global__ __launch_bounds__(2 * kWave, MINW) void lane2_pass(PassArgs a) {
+  static_assert(NP >= 2 && NP <= 32, "lane-per-row tiles hold rows of 2..64 columns");
+  constexpr int NPW = (NP + 1) / 2;  // column pairs per wave
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wc = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int p0 = wc * NPW;
+  // an odd number of pairs: the second wave's last slot lies past the row
+  const bool short_last = (NP & 1) && wc == 1;  // uniform
+
+  __shared__ v2d th_lds[2 * NPW];
+  __shared__ double zx[2][2][U][kWave];
+  if (threadIdx.x < 2 * NPW)  // theta is zero-padded far beyond the row
+    th_lds[threadIdx.x] = *reinterpret_cast<const v2d*>(a.theta + 2 * threadIdx.x);
+  __syncthreads();
+  const double bias = a.theta_bias ? *a.theta_bias : 0.;
+
+  v2d acc[NPW];
+#pragma unroll
+  for (int p = 0; p < NPW; ++p) acc[p] = v2d{0., 0.};
+  RowSums sums;
+  double h_keep[U];
+  int64_t h_row0 = -1;
+#pragma unroll
+  for (int u = 0; u < U; ++u) h_keep[u] = 0.;
+  auto store_kept = [&]() {
+    if (a.h_out && h_row0 >= 0 && wc == 0) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t row = h_row0 + u * kWave;
+        if (row < a.n) store_h(a.h_out + row, h_keep[u]);
+      }
+    }
+  };
+
+  constexpr int64_t kGroupRows = (int64_t)kWave * U;
+  const int64_t ngroups = (a.n + kGroupRows - 1) / kGroupRows;
+  int par = 0;
+#pragma clang loop unroll(disable)
+  for (int64_t g = blockIdx.x; g < ngroups; g += gridDim.x, par ^= 1) {
+    const v2d* base = reinterpret_cast<const v2d*>(a.X) + g * (U * NP * kWave) + p0 * kWave + lane;
+    v2d x[U][NPW];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int p = 0; p < NPW; ++p) {
+        x[u][p] = v2d{0., 0.};
+        if (!(p == NPW - 1 && short_last)) x[u][p] = load_x(base + (u * NP + p) * kWave);
+      }
+    const int64_t row0 = g * kGroupRows + lane;
+    double yv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t row = row0 + u * kWave;
+      yv[u] = (a.y && row < a.n) ? a.y[row] : 0.;
+    }
+    store_kept();
+    asm volatile("" ::: "memory");  // keeps the theta reads inside the loop
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      double z = 0.;
+#pragma unroll
+      for (int p = 0; p < NPW; ++p) {
+        const v2d th = th_lds[p0 + p];
+        z = fma(x[u][p].x, th.x, z);
+        z = fma(x[u][p].y, th.y, z);
+      }
+      zx[par][wc][u][lane] = z;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const double z = zx[par][0][u][lane] + zx[par][1][u][lane];
+      const bool valid = row0 + u * kWave < a.n;
+      double h, l;
+      row_terms(z + bias, yv[u], a.loss_mode, a.identity_link, h, l);
+      const double res = valid ? (h - yv[u]) : 0.;
+      h_keep[u] = h;
+      if (valid && wc == 0) {
+        sums.loss += l;
+        sums.res += res;
+      }
+      if (GRAD) {
+#pragma unroll
+        for (int p = 0; p < NPW; ++p) {
+          acc[p].x = fma(res, x[u][p].x, acc[p].x);
+          acc[p].y = fma(res, x[u][p].y, acc[p].y);
+        }
+      }
+    }
+    h_row0 = row0;
+  }
+  store_kept();
+
+  if (GRAD) {
+#pragma unroll
+    for (int p = 0; p < NPW; ++p) {
+      acc[p].x = wave_sum(acc[p].x);
+      acc[p].y = wave_sum(acc[p].y);
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int p = 0; p < NPW; ++p)
+        if (!(p == NPW - 1 && short_last))
+          *reinterpret_cast<v2d*>(a.part_g + (int64_t)blockIdx.x * (2 * NP) + 2 * (p0 + p)) = acc[p];
+    }
+  }
+  emit_row_sums<2>(sums, lane, wc, a.part_loss, a.part_res);
+}
+
 // Row-major rows (src: nrows x src_pitch doubles, the first `cols` of each
 // used) into the row-tiled layout above, as rows row0 .. row0+nrows-1 of the
 // shard.  One thread per (row, column pair); columns at or past `cols` are
