@@ -96,6 +96,11 @@ MEASURED_TRAFFIC = {
 PER_CONFIG = ["c1_dense_100k_x_100", "c3_tall_10m_x_256", "c4_wide_200k_x_16384",
               "c4b_wide_200k_x_16385", "c5_e2e_2m_x_512"]
 
+# Shapes beyond the five configurations, one per kernel family and layout, timed last in
+# a default run (GPU only) and reported under other_shapes.
+OTHER_SHAPES = ["x_narrow_30m_x_16", "x_narrow_10m_x_41", "x_short_30m_x_66",
+                "x_c1shape_20m_x_100", "x_bias_10m_x_257", "x_verywide_100k_x_32768"]
+
 # A one-GPU box gives a job 16 CPUs whatever os.cpu_count() shows there.
 CPU_SHARE = 16
 
@@ -125,7 +130,7 @@ def parse_args():
                     help="workloads whose first column is the constant bias: store it in HBM "
                          "like any other column (default: it stays on the host)")
     ap.add_argument("--headline-only", action="store_true",
-                    help="skip the per_config section of a default run")
+                    help="skip the per_config and other_shapes sections of a default run")
     ap.add_argument("--rows", type=int, default=0, help="override n (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-rows", type=int, default=0)
@@ -510,6 +515,13 @@ def main():
             "cpu_cores": (e2e.get("cpu_baseline") or {}).get("cores"),
             "step": e2e["config"]["step"]}
         out["per_config"] = per
+        extra = {}
+        for other in OTHER_SHAPES:
+            try:
+                extra[other] = per_config_entry(run_step(a, cfgs[other], False))
+            except Exception as e:  # the headline line must survive a shape that does not fit
+                extra[other] = {"error": "%s: %s" % (type(e).__name__, e)}
+        out["other_shapes"] = extra
     print(json.dumps(out), flush=True)
 
 
