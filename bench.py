@@ -23,6 +23,7 @@ bounded row sample, scaled linearly in n to the full shard.
 import argparse
 import json
 import os
+import subprocess
 import sys
 import time
 
@@ -142,6 +143,9 @@ def parse_args():
                          "plr_ps_server over ZeroMQ) instead of the bare gradient step")
     ap.add_argument("--no-dense-ps", action="store_true",
                     help="with --e2e: start the server with its dense-vector fast path off")
+    ap.add_argument("--parse", action="store_true",
+                    help="the loader instead of the gradient step: sample text -> resident shard "
+                         "on the device (plr_set_data_csv) against the host's parsers")
     ap.add_argument("--ps-roundtrip", action="store_true",
                     help="host only: microseconds per paracel_read / paracel_bupdate round trip "
                          "against plr_ps_server, dense fast path on and off")
@@ -447,6 +451,96 @@ def run_step(a, cfg, with_cpu, full_cpu_sample=False, cpu_reps=(4, 20)):
     return out
 
 
+def run_parse(a, cfg):
+    """Sample text -> resident shard (lr.cpp:76-93): plr_set_data_csv on the device against
+    the host's threaded parser and the reference's std::stod per field on one core.  The
+    text has the workload's width (k = d - 1 features + label, six decimals like the
+    reference's sample data); ~2 GB of it are parsed in one call."""
+    import tempfile
+
+    import numpy as np
+
+    from oracle import oracle
+    from paracel_amd import Plr
+
+    k = cfg.d - 1
+    rng = np.random.default_rng(cfg.seed)
+    block_rows = max(64, int(48e6 // (k * 9.3 + 2)))
+    pool = np.array(["%.6f" % v for v in rng.normal(size=200000) * cfg.spec.scale * 3])
+    idx = rng.integers(0, pool.size, size=(block_rows, k))
+    lab = rng.integers(0, 2, size=block_rows)
+    t0 = time.time()
+    block = "\n".join(",".join(pool[idx[i]]) + ",%d" % lab[i] for i in range(block_rows)) + "\n"
+    block = block.encode()
+    reps = max(1, int(2.0e9 // len(block)))
+    print("# text block: %d rows x %d fields, %.1f MB, built in %.1f s; parsed %d times over "
+          "(%.2f GB)" % (block_rows, k + 1, len(block) / 1e6, time.time() - t0, reps,
+                         reps * len(block) / 1e9), file=sys.stderr, flush=True)
+    ctx = Plr(0)
+    ctx.set_data_csv(block)                          # warm-up: one block
+    pieces = [block] * reps
+    nbytes = reps * len(block)
+    calls = []
+    for _ in range(max(1, min(a.steps, 5))):
+        t0 = time.perf_counter()
+        n, d = ctx.set_data_csv(pieces)
+        calls.append(time.perf_counter() - t0)
+        kern_ms = ctx.timing()[0]
+    assert (n, d) == (block_rows * reps, cfg.d)
+    info = ctx.kernel_info()
+    # the shard it left: spot-check against the oracle's parser on the first block
+    Xo, yo = oracle.local_parser(block[:block.index(b"\n", 2000000) + 1].decode())
+    X, y = ctx.get_data(0, Xo.shape[0])
+    assert X.tobytes() == Xo.tobytes() and y.tobytes() == yo.tobytes()
+    ctx.close()
+    call = float(np.median(calls))
+    # CPU: the reference's path (strtod per field, one core) on 20 MB; the host's own
+    # threaded parser on one block through plr_shard_tool
+    sample = block[:block.index(b"\n", min(len(block) - 2, 20000000)) + 1]
+    t0 = time.perf_counter()
+    oracle.local_parser(sample.decode())
+    stod_s = time.perf_counter() - t0
+    host = {}
+    with tempfile.NamedTemporaryFile(suffix=".csv") as f:
+        f.write(block)
+        f.flush()
+        for th in (1, cpu_threads()):
+            r = subprocess.run([os.path.join(ROOT, "paracel_amd", "plr_shard_tool"), "time",
+                                f.name, str(th), "0"], capture_output=True, text=True, check=True)
+            nn, dd, t_split, t_parse = r.stdout.split()
+            host[th] = (float(t_split), float(t_parse))
+    fields = n * cfg.d
+    # bytes the parsing kernel must move: the text once, 8 bytes per field written
+    alg = nbytes + 8 * fields
+    out = {
+        "metric": "csv_parse_gb_per_sec", "value": nbytes / call / 1e9, "unit": "GB/s of text",
+        "n_gpus": 1, "steps": len(calls), "warmup": 1, "ms_per_step": 1e3 * call,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8 -> f64",
+        "data": "synthetic",
+        "config": {"workload": cfg.name + " as text", "rows": n, "fields_per_row": cfg.d,
+                   "text_bytes": nbytes, "step": "plr_set_data_csv: text host->device, row "
+                   "offsets, parse into the resident shard (text in pageable host memory, so "
+                   "the call includes its PCIe transfer)", "kernel": info},
+        "roofline": {"bound": "hbm", "achieved": alg / (kern_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": alg / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "kernel": "csv_parse", "kernel_ms": kern_ms,
+                     "algorithmic_bytes": alg,
+                     "text_gbs_kernel_only": nbytes / (kern_ms * 1e-3) / 1e9},
+        "cpu_baseline": {
+            "value": len(block) / sum(host[cpu_threads()]) / 1e9, "unit": "GB/s of text",
+            "cores": cpu_threads(), "kind": "port",
+            "sample": "one %.0f MB block: line split %.2f s + parse %.2f s on %d threads "
+                      "(shard_io.hpp's parser: std::stod's values, short decimals on an exact "
+                      "fast path)" % (len(block) / 1e6, host[cpu_threads()][0],
+                                      host[cpu_threads()][1], cpu_threads()),
+            "value_1core": len(block) / sum(host[1]) / 1e9,
+            "reference_stod_1core_gbs": len(sample) / stod_s / 1e9,
+            "reference_stod_sample": "strtod per field as lr.cpp:76-93 does (oracle port), "
+                                     "%.0f MB" % (len(sample) / 1e6)},
+    }
+    print(json.dumps(out), flush=True)
+
+
 def per_config_entry(rec):
     """The per_config summary of one bare-step record."""
     r = rec["roofline"]
@@ -493,6 +587,9 @@ def main():
         return
     if a.train:
         run_train(a, cfg)
+        return
+    if a.parse:
+        run_parse(a, cfg)
         return
 
     with_cpu = not a.no_cpu_baseline

@@ -68,6 +68,31 @@ int plr_alloc_data(plr_ctx* ctx, int64_t n, int64_t d);
 int plr_set_data_chunk(plr_ctx* ctx, int64_t row0, int64_t nrows,
                        const double* X, int64_t ldx, const double* y);
 
+/* The same from the sample text itself: local_parser (lr.cpp:76-93) on the
+ * device.  text[0..nspans) / len[] are the worker's pieces of the input (the
+ * lines paracel_load hands it, lr.cpp:303, as they lie in the files), every
+ * non-empty line "f1<sep>f2<sep>...<sep>fk<sep>label".  The resident shard is
+ * what local_parser builds -- the sample [1.0, f1..fk] (d = k + 1 columns,
+ * *d_out) and the label -- with every field's value exactly std::stod's: the
+ * device converts the spellings for which one rounding gives that value, the
+ * rest (more than 15 significant digits, inf, nan, hex, blanks, trailing
+ * characters) are converted by std::stod on the host.  Empty fields are
+ * skipped like the reference's str_split does.  *n_out receives the number
+ * of samples.  Errors as the reference's parser would raise them (a field
+ * std::stod rejects, a line with another number of fields) come back as
+ * PLR_ERR_INVALID with the line number; lines of a single field are refused
+ * with PLR_ERR_UNSUPPORTED.  The text is copied; the caller keeps it.
+ * (plr_get_timing's last_ms afterwards: the duration of the parsing kernel.) */
+int plr_set_data_csv(plr_ctx* ctx, const char* const* text, const int64_t* len,
+                     int nspans, char sep, int64_t* n_out, int64_t* d_out);
+
+/* Rows row0 .. row0+nrows-1 of the resident shard back in the form
+ * plr_set_data takes (row-major, pitch ldx >= d; X or y may be NULL): what a
+ * worker needs to write its binary shard cache after plr_set_data_csv.  No
+ * counterpart in the reference. */
+int plr_get_data(plr_ctx* ctx, int64_t row0, int64_t nrows, double* X,
+                 int64_t ldx, double* y);
+
 /* One fused pass over the shard with theta (d doubles):
  *   gsum[j]  = sum_i (h_i - y_i) * x_ij,  h_i = 1/(1+exp(-x_i.theta))
  *              (lr.cpp:69-72 with ext_utility.hpp:171-174; the data term of

@@ -26,6 +26,9 @@ SYMBOLS = [
     ("plr_set_data", C.c_int, [_ctx, _dp, C.c_int64, C.c_int64, C.c_int64, _dp]),
     ("plr_alloc_data", C.c_int, [_ctx, C.c_int64, C.c_int64]),
     ("plr_set_data_chunk", C.c_int, [_ctx, C.c_int64, C.c_int64, _dp, C.c_int64, _dp]),
+    ("plr_set_data_csv", C.c_int, [_ctx, C.POINTER(C.c_char_p), _i64p, C.c_int, C.c_char, _i64p,
+                                   _i64p]),
+    ("plr_get_data", C.c_int, [_ctx, C.c_int64, C.c_int64, _dp, C.c_int64, _dp]),
     ("plr_loss_grad", C.c_int, [_ctx, _dp, _dp, _dp, _i64p, C.c_uint]),
     ("plr_dgd_delta", C.c_int, [_ctx, _dp, C.c_double, C.c_double, _dp, _dp]),
     ("plr_dgd_delta_linear", C.c_int, [_ctx, _dp, C.c_double, C.c_double, _dp, _dp]),
@@ -165,6 +168,30 @@ class Plr:
             ldx = d
         y = _vec(y, m, "y")
         self._check(self._lib.plr_set_data_chunk(self._h, row0, m, _p(X), ldx, _p(y)))
+
+    def set_data_csv(self, texts, sep=","):
+        """Sample text (bytes, or a list of pieces) -> resident shard, parsed on the device;
+        returns (n, d) with d counting the constant first column."""
+        if isinstance(texts, (bytes, bytearray, memoryview)):
+            texts = [texts]
+        texts = [bytes(t) for t in texts]
+        arr = (C.c_char_p * len(texts))(*texts)
+        lens = (C.c_int64 * len(texts))(*[len(t) for t in texts])
+        n, d = C.c_int64(), C.c_int64()
+        self._shape = None
+        self._check(self._lib.plr_set_data_csv(self._h, arr, lens, len(texts),
+                                               sep.encode()[0:1], C.byref(n), C.byref(d)))
+        return n.value, d.value
+
+    def get_data(self, row0=0, nrows=None):
+        """Rows of the resident shard as (X, y) in the form set_data takes."""
+        n, d = self.shape
+        if nrows is None:
+            nrows = n - row0
+        X = np.empty((nrows, d))
+        y = np.empty(nrows)
+        self._check(self._lib.plr_get_data(self._h, row0, nrows, _p(X), d, _p(y)))
+        return X, y
 
     @property
     def shape(self):

@@ -12,7 +12,9 @@
 #include <mutex>
 #include <string>
 #include <thread>
+#include <vector>
 
+#include "plr_csv.hpp"
 #include "plr_kernels.hpp"
 #include "plr_plan.hpp"
 
@@ -213,6 +215,8 @@ struct plr_ctx {
   int64_t zx_words = 0;
   unsigned team_spin_limit = kTeamSpinLimit;
   bool opt_two_sweeps = false;  // plr_set_option("column_blocks_two_sweeps")
+  bool synth_first_col = false; // the shard being reserved comes from plr_set_data_csv
+  int csv_slow_fields = 0;      // fields of the last plr_set_data_csv the host converted
   bool team_check = false;      // a team pass ran since the status word was last read
   double* d_z = nullptr;        // n: blocked rows only, x.theta accumulated over the blocks
   double* d_res = nullptr;      // n: blocked rows only, residual per row
@@ -466,7 +470,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
 }
 
 int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
-  c->bias = c->opt_first_col_one && d >= 2;
+  c->bias = (c->opt_first_col_one || c->synth_first_col) && d >= 2;
   c->dcols = d - (c->bias ? 1 : 0);
   int rc = plan_shape(c, n, c->dcols);
   if (rc != PLR_OK) return rc;
@@ -942,6 +946,266 @@ int plr_set_data(plr_ctx* c, const double* X, int64_t n, int64_t d, int64_t ldx,
   int rc = alloc_shape(c, n, d, /*zero_fill=*/false);  // every row is uploaded right below
   if (rc != PLR_OK) return rc;
   return upload_rows(c, 0, n, X, ldx, y);
+}
+
+// ---------------------------------------------------------------------------
+// plr_set_data_csv: the worker's share of the sample text, parsed on the device
+
+namespace {
+
+struct DevBuf {  // device memory released on every exit path
+  void* p = nullptr;
+  ~DevBuf() {
+    if (p) (void)hipFree(p);
+  }
+};
+
+// fields of the first non-empty line (maximal runs of non-separator bytes)
+int64_t first_line_fields(const char* const* text, const int64_t* len, int nspans, char sep) {
+  for (int s = 0; s < nspans; ++s) {
+    const char* t = text[s];
+    int64_t i = 0;
+    while (i < len[s] && t[i] == '\n') ++i;
+    if (i == len[s]) continue;
+    int64_t fields = 0;
+    bool in_field = false;
+    for (; i < len[s] && t[i] != '\n'; ++i) {
+      if (t[i] == sep) {
+        in_field = false;
+      } else if (!in_field) {
+        in_field = true;
+        ++fields;
+      }
+    }
+    return fields;
+  }
+  return 0;
+}
+
+}  // namespace
+
+int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, int nspans,
+                     char sep, int64_t* n_out, int64_t* d_out) {
+  if (!c) return PLR_ERR_INVALID;
+  if (nspans < 0 || (nspans > 0 && (!text || !len)))
+    return fail(c, PLR_ERR_INVALID, "text and len must not be NULL");
+  if (sep == '\n' || sep == '\0') return fail(c, PLR_ERR_INVALID, "bad separator");
+  int64_t total = 0;
+  for (int s = 0; s < nspans; ++s) {
+    if (len[s] < 0 || (len[s] > 0 && !text[s]))
+      return fail(c, PLR_ERR_INVALID, "bad text span");
+    total += len[s] + 1;  // a newline behind every span keeps their lines apart
+  }
+  const int64_t d = first_line_fields(text, len, nspans, sep);
+  if (n_out) *n_out = 0;
+  if (d_out) *d_out = d;
+  if (d == 0) {  // no sample line at all: an empty shard
+    PLR_HIP(c, hipSetDevice(c->device));
+    free_shape(c);
+    return PLR_OK;
+  }
+  if (d < 2)
+    return fail(c, PLR_ERR_UNSUPPORTED, "lines of one field (a label and no feature) are not "
+                                        "parsed on the device");
+  if (d > (int64_t)INT32_MAX) return fail(c, PLR_ERR_INVALID, "too many fields in a line");
+  PLR_HIP(c, hipSetDevice(c->device));
+  free_shape(c);
+
+  // the text, spans back to back, padded with newlines
+  DevBuf d_text, d_counts, d_first, d_rows, d_slow, d_ctl;
+  const int64_t padded = (total + 15) / 16 * 16 + plr::kCsvPadBytes;
+  if (hipMalloc(&d_text.p, (size_t)padded) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(c, PLR_ERR_NOMEM, "cannot allocate the device copy of the sample text");
+  }
+  unsigned char* dt = static_cast<unsigned char*>(d_text.p);
+  std::vector<int64_t> span_at(nspans + 1, 0);  // device offset of every span
+  for (int s = 0; s < nspans; ++s) {
+    if (len[s])
+      PLR_HIP(c, hipMemcpyAsync(dt + span_at[s], text[s], (size_t)len[s], hipMemcpyHostToDevice,
+                                c->stream));
+    PLR_HIP(c, hipMemsetAsync(dt + span_at[s] + len[s], '\n', 1, c->stream));
+    span_at[s + 1] = span_at[s] + len[s] + 1;
+  }
+  PLR_HIP(c, hipMemsetAsync(dt + total, '\n', (size_t)(padded - total), c->stream));
+
+  // rows: count, running sum, offsets
+  const int64_t nblocks = (total + plr::kCsvBlockBytes - 1) / plr::kCsvBlockBytes;
+  if (nblocks > (int64_t)INT32_MAX) return fail(c, PLR_ERR_INVALID, "sample text too large");
+  PLR_HIP(c, hipMalloc(&d_counts.p, (size_t)nblocks * sizeof(int)));
+  PLR_HIP(c, hipMalloc(&d_first.p, (size_t)nblocks * sizeof(int64_t)));
+  PLR_HIP(c, hipMalloc(&d_ctl.p, 4 * sizeof(int64_t)));  // [0] rows, [1] bad row, [2] slow fields
+  int64_t* ctl = static_cast<int64_t*>(d_ctl.p);
+  hipLaunchKernelGGL(plr::csv_count_rows, dim3((unsigned)nblocks), dim3(plr::kCsvThreads), 0,
+                     c->stream, dt, total, static_cast<int*>(d_counts.p));
+  hipLaunchKernelGGL(plr::csv_scan_counts, dim3(1), dim3(1024), 0, c->stream,
+                     static_cast<const int*>(d_counts.p), nblocks,
+                     static_cast<int64_t*>(d_first.p), ctl);
+  PLR_HIP(c, hipGetLastError());
+  int64_t n = 0;
+  PLR_HIP(c, hipMemcpyAsync(&n, ctl, sizeof n, hipMemcpyDeviceToHost, c->stream));
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  if (n_out) *n_out = n;
+
+  // the shard: k = d - 1 feature columns; the sample's constant first column is not stored
+  c->synth_first_col = true;
+  int rc = alloc_shape_buffers(c, n, d, /*zero_fill=*/true);
+  c->synth_first_col = false;
+  if (rc != PLR_OK) {
+    free_shape(c);
+    return rc;
+  }
+  PLR_HIP(c, hipMalloc(&d_rows.p, (size_t)std::max<int64_t>(n, 1) * sizeof(int64_t)));
+  hipLaunchKernelGGL(plr::csv_row_starts, dim3((unsigned)nblocks), dim3(plr::kCsvThreads), 0,
+                     c->stream, dt, total, static_cast<const int64_t*>(d_first.p),
+                     static_cast<int64_t*>(d_rows.p));
+  PLR_HIP(c, hipGetLastError());
+
+  const int slow_cap = 1 << 20;
+  PLR_HIP(c, hipMalloc(&d_slow.p, (size_t)slow_cap * sizeof(plr::CsvSlow)));
+  const int64_t ctl_init[3] = {n, INT64_MAX, 0};
+  PLR_HIP(c, hipMemcpyAsync(ctl, ctl_init, sizeof ctl_init, hipMemcpyHostToDevice, c->stream));
+  plr::CsvArgs ca;
+  ca.text = dt;
+  ca.len = total;
+  ca.row_start = static_cast<const int64_t*>(d_rows.p);
+  ca.n = n;
+  ca.d = (int)d;
+  ca.sep = (unsigned char)sep;
+  ca.X = c->dX;
+  ca.y = c->dy;
+  ca.pitch = c->pitch;
+  ca.np = c->lane ? c->lane->np : 0;
+  ca.slow = static_cast<plr::CsvSlow*>(d_slow.p);
+  ca.slow_cap = slow_cap;
+  ca.slow_count = reinterpret_cast<int*>(ctl + 2);
+  ca.bad_row = reinterpret_cast<long long*>(ctl + 1);
+  const int64_t want = (n + 3) / 4;
+  const unsigned grid = (unsigned)std::min<int64_t>(std::max<int64_t>(want, 1), (int64_t)c->num_cu * 8);
+  if (c->timing) PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
+  hipLaunchKernelGGL(plr::csv_parse, dim3(grid), dim3(256), 0, c->stream, ca);
+  PLR_HIP(c, hipGetLastError());
+  if (c->timing) PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
+  int64_t res[3] = {0, 0, 0};
+  PLR_HIP(c, hipMemcpyAsync(res, ctl, sizeof res, hipMemcpyDeviceToHost, c->stream));
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+
+  auto give_up = [&](int code, const std::string& msg) {
+    free_shape(c);
+    return fail(c, code, msg);
+  };
+  if (res[1] != INT64_MAX)  // parse_lines' message for the same input
+    return give_up(PLR_ERR_INVALID, "ragged sample line " + std::to_string(res[1]));
+  const int nslow = (int)(res[2] & 0xffffffff);
+  if (nslow > slow_cap)
+    return give_up(PLR_ERR_UNSUPPORTED,
+                   "more than 2^20 fields need the host's number parser: parse this input there");
+  if (nslow > 0) {
+    // spellings the device does not convert: std::stod on the host's copy of the text
+    std::vector<plr::CsvSlow> slow(nslow);
+    PLR_HIP(c, hipMemcpy(slow.data(), d_slow.p, (size_t)nslow * sizeof(plr::CsvSlow),
+                         hipMemcpyDeviceToHost));
+    std::vector<int64_t> xi, yi;
+    std::vector<double> xv, yv;
+    for (const plr::CsvSlow& f : slow) {
+      int s = 0;
+      while (s + 1 < nspans && f.pos >= span_at[s + 1]) ++s;
+      const char* p = text[s] + (f.pos - span_at[s]);
+      const char* const end = text[s] + len[s];
+      int64_t flen = f.len;
+      if (flen < 0) {
+        flen = 0;
+        while (p + flen < end && p[flen] != sep && p[flen] != '\n') ++flen;
+      }
+      double v;
+      try {
+        v = std::stod(std::string(p, (size_t)flen));
+      } catch (const std::exception& e) {  // what the reference's parser would have thrown
+        return give_up(PLR_ERR_INVALID, std::string(e.what()) + ": field " +
+                                            std::to_string(f.col) + " of sample line " +
+                                            std::to_string(f.row));
+      }
+      if (f.col == d - 1) {
+        yi.push_back(f.row);
+        yv.push_back(v);
+      } else if (c->lane) {
+        const int64_t np = c->lane->np;
+        xi.push_back(((((f.row >> 6) * np + (f.col >> 1)) << 6) + (f.row & 63)) * 2 + (f.col & 1));
+        xv.push_back(v);
+      } else {
+        xi.push_back(f.row * c->pitch + f.col);
+        xv.push_back(v);
+      }
+    }
+    auto patch = [&](double* base, const std::vector<int64_t>& idx,
+                     const std::vector<double>& val) -> int {
+      if (idx.empty()) return PLR_OK;
+      DevBuf di, dv;
+      PLR_HIP(c, hipMalloc(&di.p, idx.size() * sizeof(int64_t)));
+      PLR_HIP(c, hipMalloc(&dv.p, val.size() * sizeof(double)));
+      PLR_HIP(c, hipMemcpy(di.p, idx.data(), idx.size() * sizeof(int64_t), hipMemcpyHostToDevice));
+      PLR_HIP(c, hipMemcpy(dv.p, val.data(), val.size() * sizeof(double), hipMemcpyHostToDevice));
+      hipLaunchKernelGGL(plr::csv_patch, dim3((unsigned)((idx.size() + 255) / 256)), dim3(256), 0,
+                         c->stream, base, static_cast<const int64_t*>(di.p),
+                         static_cast<const double*>(dv.p), (int64_t)idx.size());
+      PLR_HIP(c, hipGetLastError());
+      PLR_HIP(c, hipStreamSynchronize(c->stream));
+      return PLR_OK;
+    };
+    rc = patch(c->dX, xi, xv);
+    if (rc == PLR_OK) rc = patch(c->dy, yi, yv);
+    if (rc != PLR_OK) {
+      free_shape(c);
+      return rc;
+    }
+  }
+  c->csv_slow_fields = nslow;
+  if (c->timing) {  // plr_get_timing's last_ms: the parsing kernel
+    float ms = 0.f;
+    PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
+    c->last_ms = ms;
+  }
+  return PLR_OK;
+}
+
+int plr_get_data(plr_ctx* c, int64_t row0, int64_t nrows, double* X, int64_t ldx, double* y) {
+  if (!c) return PLR_ERR_INVALID;
+  if (!c->have_data) return fail(c, PLR_ERR_NODATA, "no shard resident: call plr_set_data first");
+  if (row0 < 0 || nrows < 0 || row0 + nrows > c->n)
+    return fail(c, PLR_ERR_INVALID, "row range outside the resident shard");
+  if (nrows == 0) return PLR_OK;
+  if (!X && !y) return fail(c, PLR_ERR_INVALID, "X and y must not both be NULL");
+  if (X && ldx < c->d) return fail(c, PLR_ERR_INVALID, "ldx must be >= d");
+  PLR_HIP(c, hipSetDevice(c->device));
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  const int skip = c->bias ? 1 : 0;
+  if (X && c->lane) {
+    // row-tiled shard: blocks of rows are brought to row-major form on the device first
+    const int64_t cols = c->dcols;
+    const int64_t chunk_rows = std::max<int64_t>(1, (int64_t)(32u << 20) / (cols * 8));
+    DevBuf stage;
+    PLR_HIP(c, hipMalloc(&stage.p, (size_t)std::min(chunk_rows, nrows) * cols * sizeof(double)));
+    for (int64_t r0 = 0; r0 < nrows; r0 += chunk_rows) {
+      const int64_t m = std::min(chunk_rows, nrows - r0);
+      hipLaunchKernelGGL(plr::untile_rows, dim3((unsigned)ceil_div(m * cols, 256)), dim3(256), 0,
+                         c->stream, (const double*)c->dX, row0 + r0, m, (int)cols, c->lane->np,
+                         static_cast<double*>(stage.p));
+      PLR_HIP(c, hipGetLastError());
+      PLR_HIP(c, hipMemcpy2DAsync(X + r0 * ldx + skip, (size_t)ldx * sizeof(double), stage.p,
+                                  (size_t)cols * sizeof(double), (size_t)cols * sizeof(double),
+                                  (size_t)m, hipMemcpyDeviceToHost, c->stream));
+      PLR_HIP(c, hipStreamSynchronize(c->stream));
+    }
+  } else if (X) {
+    PLR_HIP(c, hipMemcpy2D(X + skip, (size_t)ldx * sizeof(double), c->dX + row0 * c->pitch,
+                           (size_t)c->pitch * sizeof(double), (size_t)c->dcols * sizeof(double),
+                           (size_t)nrows, hipMemcpyDeviceToHost));
+  }
+  if (X && skip)
+    for (int64_t r = 0; r < nrows; ++r) X[r * ldx] = 1.;
+  if (y)
+    PLR_HIP(c, hipMemcpy(y, c->dy + row0, (size_t)nrows * sizeof(double), hipMemcpyDeviceToHost));
+  return PLR_OK;
 }
 
 int plr_loss_grad(plr_ctx* c, const double* theta, double* gsum, double* loss_sum,

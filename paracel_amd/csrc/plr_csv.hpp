@@ -1,0 +1,287 @@
+// Sample text -> resident shard, on the device.
+//
+// The reference's local_parser (alg/classification/logistic_regression/
+// lr.cpp:76-93) turns every line "f1,f2,...,fk,label" into the sample
+// [1.0, f1..fk] and its label with std::stod per field; for file-fed runs that
+// parse, not the training pass, is what a worker waits for.  Here the worker's
+// byte range of the input is copied to HBM as it is and parsed there:
+//
+//   csv_count_rows   line starts per 4 KiB block of text
+//   csv_scan_counts  their running sum (one workgroup): first row of a block
+//   csv_row_starts   byte offset of every row
+//   csv_parse        a wave per row: separators by ballot, one lane per field
+//                    that starts in the wave's 64-byte window, the field's
+//                    characters fetched from the neighbouring lanes
+//
+// A field is converted on the device only when that is exact: the spelling
+// [-]digits[.digits][e[+-]digits] with at most 15 significant digits and a
+// decimal exponent within +-22.  Its digits are then an exact double, 10^|e|
+// is an exact double, and the one multiplication or division rounds once --
+// the correctly rounded value, which is what strtod returns (Clinger's fast
+// path; the host parser in worker/shard_io.hpp takes the same route).  Every
+// other spelling is put on a list the host resolves with std::stod itself, so
+// values and errors are the reference's for every input.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace plr {
+
+constexpr int kCsvThreads = 256;
+constexpr int kCsvBytesPerThread = 16;
+constexpr int kCsvBlockBytes = kCsvThreads * kCsvBytesPerThread;  // 4 KiB
+constexpr int kCsvMaxFieldChars = 32;  // longer fields go to the host
+constexpr int kCsvPadBytes = 256;      // '\n' behind the text: a window may read past the end
+
+// a field the device did not convert
+struct CsvSlow {
+  int64_t row;   // row of the shard
+  int64_t pos;   // byte offset of the field's first character in the device text
+  int32_t col;   // field index in the line (0 .. d-1; d-1 is the label)
+  int32_t len;   // characters, or -1: longer than one window shows (the host finds its end)
+};
+
+struct CsvArgs {
+  const unsigned char* text;  // len bytes followed by kCsvPadBytes of '\n'
+  int64_t len;
+  const int64_t* row_start;   // n byte offsets
+  int64_t n;
+  int d;                      // fields per line: k features, then the label
+  unsigned char sep;
+  double* X;                  // the shard: the k features of every row (the constant
+  double* y;                  //   first column of the reference's sample is not stored)
+  int64_t pitch;
+  int np;                     // > 0: row-tiled layout with np column pairs per row
+  CsvSlow* slow;
+  int slow_cap;
+  int* slow_count;
+  long long* bad_row;         // smallest row whose field count is not d
+};
+
+// line starts among the 16 bytes at `base` (a line starts after a newline, or
+// at offset 0, and is not empty); their offsets go to out[] when given
+__device__ __forceinline__ int csv_starts16(const unsigned char* t, int64_t base, int64_t len,
+                                            int64_t* out) {
+  if (base >= len) return 0;
+  const uint4 v = *reinterpret_cast<const uint4*>(t + base);
+  const unsigned w[4] = {v.x, v.y, v.z, v.w};
+  unsigned char prev = base == 0 ? (unsigned char)'\n' : t[base - 1];
+  int c = 0;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const unsigned char ch = (unsigned char)(w[k >> 2] >> (8 * (k & 3)));
+    if (base + k < len && ch != '\n' && prev == '\n') {
+      if (out) out[c] = base + k;
+      ++c;
+    }
+    prev = ch;
+  }
+  return c;
+}
+
+__global__ __launch_bounds__(kCsvThreads) void csv_count_rows(const unsigned char* t, int64_t len,
+                                                              int* counts) {
+  __shared__ int part[kCsvThreads / 64];
+  const int64_t base = ((int64_t)blockIdx.x * kCsvThreads + threadIdx.x) * kCsvBytesPerThread;
+  int c = csv_starts16(t, base, len, nullptr);
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) c += __shfl_xor(c, m, 64);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int s = 0;
+    for (int w = 0; w < kCsvThreads / 64; ++w) s += part[w];
+    counts[blockIdx.x] = s;
+  }
+}
+
+// exclusive running sum of counts[0..nblocks) into first_row[], the total into *total
+__global__ __launch_bounds__(1024) void csv_scan_counts(const int* counts, int64_t nblocks,
+                                                        int64_t* first_row, int64_t* total) {
+  __shared__ int64_t wsum[16];
+  __shared__ int64_t carry_s;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) carry_s = 0;
+  __syncthreads();
+  for (int64_t i0 = 0; i0 < nblocks; i0 += 1024) {
+    const int64_t i = i0 + threadIdx.x;
+    const int64_t v = i < nblocks ? counts[i] : 0;
+    int64_t s = v;  // inclusive scan inside the wave
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+      const int64_t o = __shfl_up(s, m, 64);
+      if (lane >= m) s += o;
+    }
+    if (lane == 63) wsum[wave] = s;
+    __syncthreads();
+    int64_t before = carry_s;
+    for (int w = 0; w < wave; ++w) before += wsum[w];
+    if (i < nblocks) first_row[i] = before + s - v;
+    __syncthreads();
+    if (threadIdx.x == 1023) carry_s = before + s;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *total = carry_s;
+}
+
+__global__ __launch_bounds__(kCsvThreads) void csv_row_starts(const unsigned char* t, int64_t len,
+                                                              const int64_t* first_row,
+                                                              int64_t* row_start) {
+  __shared__ int part[kCsvThreads / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t base = ((int64_t)blockIdx.x * kCsvThreads + threadIdx.x) * kCsvBytesPerThread;
+  int64_t pos[kCsvBytesPerThread];
+  const int c = csv_starts16(t, base, len, pos);
+  int s = c;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) {
+    const int o = __shfl_up(s, m, 64);
+    if (lane >= m) s += o;
+  }
+  if (lane == 63) part[wave] = s;
+  __syncthreads();
+  int before = 0;
+  for (int w = 0; w < wave; ++w) before += part[w];
+  int64_t* out = row_start + first_row[blockIdx.x] + before + s - c;
+  for (int k = 0; k < c; ++k) out[k] = pos[k];
+}
+
+// exact powers of ten
+__device__ const double kCsvPow10[23] = {1e0,  1e1,  1e2,  1e3,  1e4,  1e5,  1e6,  1e7,
+                                         1e8,  1e9,  1e10, 1e11, 1e12, 1e13, 1e14, 1e15,
+                                         1e16, 1e17, 1e18, 1e19, 1e20, 1e21, 1e22};
+
+__device__ __forceinline__ int csv_wave_max(int v) {
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) {
+    const int o = __shfl_xor(v, m, 64);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+__global__ __launch_bounds__(256) void csv_parse(CsvArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave0 = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t nwaves = (int64_t)gridDim.x * 4;
+  const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));  // lanes before mine
+
+  for (int64_t r = wave0; r < a.n; r += nwaves) {
+    int64_t pos = a.row_start[r];
+    int nfields = 0;       // fields of this row seen so far (uniform)
+    bool prev_sep = true;  // the byte in front of the window ends a field (or the row starts here)
+    bool done = false;
+    while (!done) {
+      // 128 bytes of the row: `cur` is this window, `nxt` the one behind it (the
+      // text is padded with newlines, so both loads stay inside the buffer)
+      const int cur = a.text[pos + lane];
+      const int nxt = a.text[pos + 64 + lane];
+      const unsigned long long nl_cur = __ballot(cur == '\n');
+      const unsigned long long sep_cur = __ballot(cur == a.sep);
+      const unsigned long long term_cur = nl_cur | sep_cur;
+      const unsigned long long term_nxt = __ballot(nxt == '\n' || nxt == a.sep);
+      const int endp = nl_cur ? __builtin_ctzll(nl_cur) : 64;  // the row's bytes are lanes < endp
+      done = nl_cur != 0;
+      // a field starts at a byte that is no terminator and follows one
+      const bool after_term = lane == 0 ? prev_sep : ((term_cur >> (lane - 1)) & 1ull) != 0;
+      const bool start = lane < endp && ((term_cur >> lane) & 1ull) == 0 && after_term;
+      const unsigned long long start_mask = __ballot(start);
+      int flen = 0;
+      bool bad = false;
+      if (start) {
+        const unsigned long long t1 = lane == 63 ? 0ull : term_cur >> (lane + 1);
+        if (t1)
+          flen = 1 + __builtin_ctzll(t1);
+        else if (term_nxt)
+          flen = 64 - lane + __builtin_ctzll(term_nxt);
+        else
+          flen = -1;  // no end in sight
+        if (flen < 0 || flen > kCsvMaxFieldChars) bad = true;
+      }
+      const int L = csv_wave_max((start && !bad) ? flen : 0);
+
+      // strtod's grammar for the exact spellings, one character per step
+      unsigned long long m = 0;
+      int sig = 0, ndig = 0, frac = 0, e10 = 0, ed = 0, st = 0;  // st: 0 int, 1 frac, 2 exp sign, 3 exp
+      bool neg = false, eneg = false;
+      for (int j = 0; j < L; ++j) {
+        const int src = lane + j;
+        const int c0 = __shfl(cur, src & 63, 64);
+        const int c1 = __shfl(nxt, src & 63, 64);
+        const int ch = src < 64 ? c0 : c1;
+        if (!start || bad || j >= flen) continue;
+        const bool digit = ch >= '0' && ch <= '9';
+        if (st <= 1) {
+          if (digit) {
+            m = m * 10ull + (unsigned long long)(ch - '0');
+            if (m) ++sig;
+            if (sig > 15) bad = true;
+            ++ndig;
+            if (st == 1) ++frac;
+          } else if (ch == '-' && j == 0) {
+            neg = true;
+          } else if (ch == '.' && st == 0) {
+            st = 1;
+          } else if ((ch == 'e' || ch == 'E') && ndig > 0) {
+            st = 2;
+          } else {
+            bad = true;
+          }
+        } else if (st == 2 && (ch == '+' || ch == '-')) {
+          eneg = ch == '-';
+          st = 3;
+        } else if (digit) {
+          st = 3;
+          e10 = e10 * 10 + (ch - '0');
+          if (e10 > 9999) bad = true;
+          ++ed;
+        } else {
+          bad = true;
+        }
+      }
+
+      if (start) {
+        const int col = nfields + __builtin_popcountll(start_mask & below);
+        int e = (eneg ? -e10 : e10) - frac;
+        if (ndig == 0 || st == 2 || (st == 3 && ed == 0) || e < -22 || e > 22) bad = true;
+        if (col < a.d) {
+          if (!bad) {
+            double v = (double)m;
+            v = e < 0 ? v / kCsvPow10[-e] : v * kCsvPow10[e];
+            if (neg) v = -v;
+            if (col == a.d - 1) {
+              a.y[r] = v;
+            } else if (a.np > 0) {
+              a.X[((((r >> 6) * a.np + (col >> 1)) << 6) + (r & 63)) * 2 + (col & 1)] = v;
+            } else {
+              a.X[r * a.pitch + col] = v;
+            }
+          } else {
+            const int k = atomicAdd(a.slow_count, 1);
+            if (k < a.slow_cap) {
+              CsvSlow s;
+              s.row = r;
+              s.pos = pos + lane;
+              s.col = col;
+              s.len = flen > kCsvMaxFieldChars ? -1 : flen;
+              a.slow[k] = s;
+            }
+          }
+        }
+      }
+      nfields += __builtin_popcountll(start_mask);
+      prev_sep = ((term_cur >> 63) & 1ull) != 0;
+      pos += 64;
+    }
+    if (nfields != a.d && lane == 0) atomicMin(a.bad_row, (long long)r);
+  }
+}
+
+// values the host converted: X or y entries by flat index
+__global__ void csv_patch(double* base, const int64_t* index, const double* value, int64_t count) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) base[index[i]] = value[i];
+}
+
+}  // namespace plr

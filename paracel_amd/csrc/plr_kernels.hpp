@@ -749,6 +749,18 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void lane_pass(PassArgs a) {
   emit_row_sums<WROW>(sums, lane, wr, a.part_loss, a.part_res);
 }
 
+// The inverse of tile_rows: rows row0 .. row0+nrows-1 of a row-tiled shard as
+// row-major rows of `cols` doubles (dst pitch = cols).
+__global__ void untile_rows(const double* X, int64_t row0, int64_t nrows, int cols, int np,
+                            double* dst) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= nrows * cols) return;
+  const int64_t r = i / cols;
+  const int col = (int)(i % cols);
+  const int64_t row = row0 + r;
+  dst[i] = X[((((row / kWave) * np + (col >> 1)) * kWave) + (row % kWave)) * 2 + (col & 1)];
+}
+
 // lane_pass for the wider tiles (34..64 columns), where rows and accumulators
 // of a whole tile fill the registers of a wave (one wave per SIMD): a PAIR of
 // waves shares every tile, each holding half of the column pairs of the same

@@ -50,6 +50,7 @@ class logistic_regression_gpu : public paralg {
 
  private:
   void load_and_parse(const std::string& fn);  // paracel_load + local_parser, cached
+  bool load_on_device(const std::string& fn);  // ... with the text parsed on the device
   void upload();                // flat rows -> HBM, then the host copy is dropped
   void check(int rc, const char* what);
 

@@ -31,6 +31,7 @@
 #include <unistd.h>
 
 #include <stdexcept>
+#include <memory>
 #include <string>
 #include <thread>
 #include <vector>
@@ -170,6 +171,46 @@ inline std::vector<std::string> load_lines(const std::string& input, int rank, i
     lines_starting_in(m.data(), f.end - f.begin, lo - f.begin, hi - f.begin, lines);
   }
   return lines;
+}
+
+// The same share of the input as load_lines returns, as it lies in the files:
+// per file one stretch of text holding exactly the lines that start inside the
+// worker's byte range (for a parser that takes the text itself).  The
+// mappings live as long as the object.
+struct OwnedText {
+  std::vector<std::unique_ptr<MappedFile> > files;
+  std::vector<const char*> text;
+  std::vector<int64_t> len;
+};
+
+inline void owned_text(const std::string& input, int rank, int np, OwnedText& out) {
+  if (np < 1 || rank < 0 || rank >= np) throw std::invalid_argument("bad worker rank");
+  const std::vector<std::string> files = expand_input(input);
+  if (files.empty()) throw std::runtime_error("cannot open " + input);
+  const std::vector<FileSpan> spans = stream_layout(files);
+  int64_t lo = 0, hi = 0;
+  owned_range(spans.back().end, rank, np, lo, hi);
+  for (const FileSpan& f : spans) {
+    if (f.end <= lo || f.begin >= hi || f.end == f.begin) continue;  // no byte of it is ours
+    const int64_t size = f.end - f.begin;
+    std::unique_ptr<MappedFile> m(new MappedFile(f.path, size));
+    const char* t = m->data();
+    int64_t b = lo - f.begin < 0 ? 0 : lo - f.begin;
+    int64_t e = hi - f.begin > size ? size : hi - f.begin;
+    if (b > 0 && t[b - 1] != '\n') {  // inside a line that belongs to an earlier range
+      const void* nl = memchr(t + b, '\n', (size_t)(size - b));
+      if (!nl) continue;
+      b = static_cast<const char*>(nl) - t + 1;
+    }
+    if (b >= e) continue;  // no line starts inside the range
+    if (t[e - 1] != '\n') {  // the line that holds the range's last byte is taken whole
+      const void* nl = memchr(t + e, '\n', (size_t)(size - e));
+      e = nl ? static_cast<const char*>(nl) - t + 1 : size;
+    }
+    out.text.push_back(t + b);
+    out.len.push_back(e - b);
+    out.files.push_back(std::move(m));
+  }
 }
 
 struct ParsedShard {

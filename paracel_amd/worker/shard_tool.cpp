@@ -2,10 +2,13 @@
 //   plr_shard_tool parse <input.csv> <rank> <np>   parse this rank's lines and write the cache
 //   plr_shard_tool info  <input.csv> <rank> <np>   validate the cache; print n d
 //   plr_shard_tool lines <input.csv> <rank> <np>   print the lines this rank owns
+//   plr_shard_tool time  <input.csv> <threads> 0   print n d and the seconds of the line split
+//                                                  and of the parse on <threads> threads
 //   plr_shard_tool owners <input> <lo_np> <hi_np>  for every np in [lo_np, hi_np] and every rank:
 //                                                  "np rank line" per owned line
 //   plr_shard_tool selftest <count> <seed> 0       parse_field against std::stod on <count>
 //                                                  random field spellings, bit for bit
+#include <chrono>
 #include <iostream>
 #include <random>
 
@@ -88,13 +91,25 @@ int main(int argc, char** argv) {
   const std::string cmd = argv[1], input = argv[2];
   const int rank = atoi(argv[3]), np = atoi(argv[4]);
   try {
-    if (rank < 0 || np < 1 || rank >= np) throw std::invalid_argument("need 0 <= rank < np");
+    if (cmd != "time" && (rank < 0 || np < 1 || rank >= np))
+      throw std::invalid_argument("need 0 <= rank < np");
     if (cmd == "lines") {
       for (const std::string& l : plr_ps::load_lines(input, rank, np)) std::cout << l << "\n";
     } else if (cmd == "parse") {
       plr_ps::ParsedShard s = plr_ps::parse_lines(plr_ps::load_lines(input, rank, np));
       if (!plr_ps::write_cache(input, rank, np, s)) throw std::runtime_error("cannot write the cache");
       std::cout << s.n << " " << s.d << "\n";
+    } else if (cmd == "time") {
+      // the host's loader and parser alone: seconds for the line split and for the
+      // parse on <rank> threads (np is ignored: the whole input)
+      using clk = std::chrono::steady_clock;
+      const auto t0 = clk::now();
+      const std::vector<std::string> lines = plr_ps::load_lines(input, 0, 1);
+      const auto t1 = clk::now();
+      plr_ps::ParsedShard s = plr_ps::parse_lines(lines, ',', rank < 1 ? 1 : rank);
+      const auto t2 = clk::now();
+      std::cout << s.n << " " << s.d << " " << std::chrono::duration<double>(t1 - t0).count()
+                << " " << std::chrono::duration<double>(t2 - t1).count() << "\n";
     } else if (cmd == "info") {
       plr_ps::ParsedShard s;
       if (!plr_ps::read_cache(input, rank, np, s)) {

@@ -1,0 +1,173 @@
+"""plr_set_data_csv: the reference's local_parser (lr.cpp:76-93) on the device.
+
+The shard it leaves resident must be, bit for bit, what the oracle's restatement of
+local_parser (strtod per field, str_split's empty-field rule, the leading 1.0) builds
+from the same text -- whichever route a field's conversion took, the device's exact
+one-rounding path or std::stod on the host.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def plr():
+    from paracel_amd import Plr
+
+    with Plr(0) as c:
+        yield c
+
+
+@pytest.fixture(scope="module")
+def oracle():
+    from oracle import oracle as o
+
+    return o
+
+
+def spell(rng, v, kind):
+    """One spelling of the number v (kind picks the route it will take)."""
+    if kind == 0:
+        return "%.6f" % v                       # short decimal: device
+    if kind == 1:
+        return "%.14e" % v                      # 15 significant digits + exponent: device
+    if kind == 2:
+        return repr(float(v))                   # shortest round-trip, up to 17 digits: mostly host
+    if kind == 3:
+        return "%d" % int(v * 1000)             # integer
+    if kind == 4:
+        return "%.17g" % v                      # 17 digits: host
+    if kind == 5:
+        return ("%.3f" % v).lstrip("0") if 0 <= v < 1 else "%.3f" % v   # ".123"
+    if kind == 6:
+        return "%.2fE%+d" % (v, int(rng.integers(-25, 26)))             # exponent near +-22
+    if kind == 7:
+        return "%d." % int(v * 10)              # "12."
+    return "%.9g" % v
+
+
+def make_text(rng, n, k, kinds, sep=",", eol="\n", blank_every=0):
+    vals = rng.normal(size=(n, k)) * 10.0 ** rng.integers(-3, 4, size=(n, k))
+    lines = []
+    for i in range(n):
+        f = [spell(rng, vals[i, j], kinds[(i * k + j) % len(kinds)]) for j in range(k)]
+        f.append(str(int(rng.integers(0, 2))))
+        lines.append(sep.join(f))
+        if blank_every and i % blank_every == 0:
+            lines.append("")
+    return eol.join(lines) + eol
+
+
+def check_equal(plr, oracle, text, pieces=None, sep=","):
+    Xo, yo = oracle.local_parser(text, sep=sep)
+    data = text.encode()
+    n, d = plr.set_data_csv(pieces if pieces is not None else data, sep=sep)
+    assert (n, d) == Xo.shape
+    assert "not stored" in plr.kernel_info()
+    X, y = plr.get_data()
+    assert X.tobytes() == Xo.tobytes()
+    assert y.tobytes() == yo.tobytes()
+    return Xo, yo
+
+
+@pytest.mark.parametrize("n,k", [(1, 1), (3, 2), (70, 5), (1000, 16), (129, 31), (257, 63),
+                                 (500, 64), (300, 65), (200, 100), (150, 257), (64, 1000),
+                                 (9, 5000), (5, 20000)])
+def test_device_parser_builds_the_oracles_shard(plr, oracle, n, k):
+    rng = np.random.default_rng(1000 * n + k)
+    print("case n=%d k=%d" % (n, k), flush=True)
+    text = make_text(rng, n, k, kinds=[0, 1, 3, 5, 6, 7, 8])
+    Xo, yo = check_equal(plr, oracle, text)
+    # ... and the passes over it are those of the same rows sent with plr_set_data
+    th = rng.normal(size=k + 1)
+    g, loss, cnt = plr.loss_grad(th)
+    plr.set_option("first_column_is_one", 1)
+    try:
+        plr.set_data(Xo, yo)
+        g2, loss2, _ = plr.loss_grad(th)
+    finally:
+        plr.set_option("first_column_is_one", 0)
+    assert cnt == n
+    np.testing.assert_array_equal(g, g2)
+    assert loss == loss2
+
+
+def test_fields_the_host_converts_and_odd_lines(plr, oracle):
+    rng = np.random.default_rng(5)
+    # 17-digit spellings, shortest round-trip reprs, blank lines, CR LF line ends
+    text = make_text(rng, 400, 9, kinds=[2, 4, 0, 1], blank_every=7)
+    check_equal(plr, oracle, text)
+    text = make_text(rng, 300, 70, kinds=[4, 2])
+    check_equal(plr, oracle, text)
+    crlf = make_text(rng, 50, 6, kinds=[0, 3], eol="\r\n")
+    check_equal(plr, oracle, crlf)
+    # inf, nan, hex floats, blanks, a plus sign, trailing characters, very long digit strings,
+    # empty fields (dropped), another separator
+    odd = ("inf,-inf,0x1p3, 2.5,+3,4.5abc,1\n"
+           "1e22,1e23,123456789012345,1234567890123456,-0,-0.0,0\n"
+           "0.000000000000000000000000000000000001,1%s,1e-5,00000000000000000000012.5,7,8,1\n"
+           % ("0" * 40))
+    Xo, _ = check_equal(plr, oracle, odd)
+    assert np.isinf(Xo[0, 1]) and Xo[0, 3] == 8.0 and np.signbit(Xo[1, 5])
+    check_equal(plr, oracle, "1,,2,,,3,1\n4,5,,6,0\n")
+    check_equal(plr, oracle, "1;2;1\n3;4;0\n", sep=";")
+    nan_line = "nan,1,1\n"
+    n, d = plr.set_data_csv(nan_line.encode())
+    X, y = plr.get_data()
+    assert (n, d) == (1, 3) and np.isnan(X[0, 1]) and X[0, 2] == 1.0 and y[0] == 1.0
+
+
+def test_pieces_of_text_and_rows_across_windows(plr, oracle):
+    rng = np.random.default_rng(9)
+    text = make_text(rng, 333, 12, kinds=[0, 1, 8])
+    data = text.encode()
+    # pieces cut at line ends, the last without its newline; an empty piece in between
+    cut1 = data.index(b"\n", len(data) // 3) + 1
+    cut2 = data.index(b"\n", 2 * len(data) // 3) + 1
+    pieces = [data[:cut1], b"", data[cut1:cut2], data[cut2:-1]]
+    check_equal(plr, oracle, text, pieces=pieces)
+    # rows of every length around the 64-byte window, fields of 1..14 digits: field starts
+    # and ends fall on every lane, many fields run on into the next window
+    lines = []
+    for _ in range(700):
+        f = [str(int(rng.integers(0, 10 ** int(rng.integers(1, 15))))) for _ in range(12)]
+        lines.append(",".join(f + [str(int(rng.integers(0, 2)))]))
+    check_equal(plr, oracle, "\n".join(lines) + "\n")
+
+
+def test_errors_are_the_reference_parsers(plr):
+    from paracel_amd import PlrError
+
+    with pytest.raises(PlrError) as e:
+        plr.set_data_csv(b"1,2,1\n3,4,5,0\n6,7,1\n")
+    assert e.value.code == -1 and "ragged sample line 1" in str(e.value)
+    with pytest.raises(PlrError) as e:
+        plr.set_data_csv(b"1,2,1\n3,abc,0\n")
+    assert e.value.code == -1 and "sample line 1" in str(e.value)
+    with pytest.raises(PlrError) as e:
+        plr.set_data_csv(b"1,1e999,1\n")        # std::stod: out of range
+    assert e.value.code == -1
+    with pytest.raises(PlrError) as e:
+        plr.set_data_csv(b"1\n0\n")             # a label and no feature
+    assert e.value.code == -5
+    # no sample line: an empty shard, no error
+    assert plr.set_data_csv(b"\n\n") == (0, 0)
+    assert plr.set_data_csv([]) == (0, 0)
+    # the context is usable afterwards
+    assert plr.set_data_csv(b"1,2,1\n") == (1, 3)
+    X, y = plr.get_data()
+    assert X.tolist() == [[1.0, 1.0, 2.0]] and y.tolist() == [1.0]
+
+
+def test_get_data_returns_what_set_data_took(plr):
+    rng = np.random.default_rng(3)
+    for n, d in [(100, 7), (130, 64), (77, 66), (50, 300), (10, 20001)]:
+        X = rng.normal(size=(n, d))
+        y = rng.integers(0, 2, size=n).astype(float)
+        plr.set_data(X, y)
+        X2, y2 = plr.get_data()
+        assert X2.tobytes() == X.tobytes() and y2.tobytes() == y.tobytes()
+        X3, y3 = plr.get_data(n // 3, n // 2)
+        assert X3.tobytes() == X[n // 3:n // 3 + n // 2].tobytes()
+        assert y3.tobytes() == y[n // 3:n // 3 + n // 2].tobytes()

@@ -97,6 +97,8 @@ def test_csv_driver_follows_the_reference_call_order(server_info, oracle, tmp_pa
     curve = np.array([float(t) for t in (outdir / "lr_loss_error_0").read_text().split()])
     assert curve.shape == (20,) and abs(curve[0] - np.log(2)) < 1e-6 and curve[-1] < curve[0]
 
+    # the first run parsed the training text on the device and wrote the binary shard cache
+    assert "parsed on the device: 400 x 7" in r.stdout and "lines got: 400" in r.stdout
     # second run: the text is not parsed again (binary shard cache), same result
     # (in the first run only test(), which re-reads the training file, found the cache)
     assert r.stdout.count("shard cache hit") == 1
@@ -110,6 +112,19 @@ def test_csv_driver_follows_the_reference_call_order(server_info, oracle, tmp_pa
     assert r2.returncode == 0, r2.stderr
     assert r2.stdout.count("shard cache hit: 400 x 7") == 2
     assert (outdir2 / "lr_theta_0").read_text() == (outdir / "lr_theta_0").read_text()
+    # third run, no cache and the host's parser: the same bytes in every output file
+    os.remove(str(train) + ".plrshard.0of1")
+    outdir3 = tmp_path / "out3"
+    cfg2["output"] = str(outdir3) + "/"
+    cfgf.write_text(json.dumps(cfg2))
+    r3 = subprocess.run([os.path.join(PKG, "plr_lr_worker"), "--server_info", server_info,
+                         "--cfg_file", str(cfgf), "--theta0", "zero"],
+                        capture_output=True, text=True, timeout=110,
+                        env=dict(os.environ, PLR_HOST_PARSE="1"))
+    assert r3.returncode == 0, r3.stderr
+    assert "parsed on the device" not in r3.stdout
+    for name in ("lr_theta_0", "pred_v_0", "lr_loss_error_0"):
+        assert (outdir3 / name).read_text() == (outdir / name).read_text()
 
 
 def test_config_5_at_full_size_through_the_server(server_info, oracle, gen, tmp_path):
