@@ -1,5 +1,7 @@
 #include "lr_gpu.hpp"
 
+#include "device_load.hpp"
+
 #include <stdlib.h>
 
 #include <chrono>
@@ -65,47 +67,14 @@ void logistic_regression_gpu::load_and_parse(const std::string& fn) {
   labels.swap(s.y);
 }
 
-// paracel_load + local_parser with the parsing done on the device: the worker's
-// share of the text goes to HBM as it lies in the files (plr_set_data_csv) and
-// the shard never exists on the host -- except once, on its way into the binary
-// cache.  False (nothing done) when the cache is fresh, when PLR_HOST_PARSE is
-// set, or when the library leaves this input to the host parser.
+// paracel_load + local_parser on the device (device_load.hpp)
 bool logistic_regression_gpu::load_on_device(const std::string& fn) {
-  const char* host = getenv("PLR_HOST_PARSE");
-  if (host && *host && *host != '0') return false;
-  const int rank = (int)get_worker_id(), np = (int)get_worker_size();
-  {
-    ShardCacheHeader h;
-    FILE* f = nullptr;
-    if (open_cache(fn, rank, np, h, f)) {
-      fclose(f);
-      return false;  // reading the cache beats any parser
-    }
-  }
-  const auto t0 = std::chrono::steady_clock::now();
-  OwnedText own;
-  owned_text(fn, rank, np, own);
   int64_t n = 0, d = 0;
-  const int rc = plr_set_data_csv(gpu, own.text.data(), own.len.data(), (int)own.text.size(), ',',
-                                  &n, &d);
-  if (rc == PLR_ERR_UNSUPPORTED) return false;
-  if (rc != PLR_OK) throw std::invalid_argument(plr_last_error(gpu));  // the parser's errors
-  std::cout << "lines got: " << n << std::endl;  // loader.hpp:93
+  if (!load_shard_on_device(gpu, fn, (int)get_worker_id(), (int)get_worker_size(), n, d))
+    return false;
   n_local = n;
   data_dim = d;
   if (kdim == 0 && data_dim > 0) kdim = (int)data_dim - 1;
-  std::cout << "parsed on the device: " << n << " x " << d << " in "
-            << std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count()
-            << " s" << std::endl;
-  if (n > 0) {  // the cache the next run starts from
-    ParsedShard s;
-    s.n = n;
-    s.d = d;
-    s.X.resize((size_t)n * d);
-    s.y.resize(n);
-    check(plr_get_data(gpu, 0, n, s.X.data(), d, s.y.data()), "plr_get_data");
-    if (!write_cache(fn, rank, np, s)) std::cout << "shard cache not written" << std::endl;
-  }
   return true;
 }
 

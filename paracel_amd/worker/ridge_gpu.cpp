@@ -1,5 +1,7 @@
 #include "ridge_gpu.hpp"
 
+#include "device_load.hpp"
+
 #include <stdlib.h>
 
 #include <iostream>
@@ -39,6 +41,15 @@ void ridge_regression_gpu::check(int rc, const char* what) {
 void ridge_regression_gpu::load_and_upload(const std::string& fn) {
   ParsedShard s;
   const int rank = (int)get_worker_id(), np = (int)get_worker_size();
+  {
+    int64_t n = 0, d = 0;
+    if (load_shard_on_device(gpu, fn, rank, np, n, d)) {  // parsed in HBM (device_load.hpp)
+      n_local = n;
+      data_dim = d;
+      if (kdim == 0 && data_dim > 0) kdim = (int)data_dim - 1;
+      return;
+    }
+  }
   if (!read_cache(fn, rank, np, s)) {
     s = parse_lines(paracel_load(fn));
     if (!write_cache(fn, rank, np, s)) std::cout << "shard cache not written" << std::endl;
