@@ -175,8 +175,10 @@ void logistic_regression_gpu::dump_result() {
 }
 
 void logistic_regression_gpu::test(const std::string& test_fn) {
-  load_and_parse(test_fn);
-  upload();
+  if (!load_on_device(test_fn)) {
+    load_and_parse(test_fn);
+    upload();
+  }
   std::cout << "loss in test dataset is: " << calc_loss() << std::endl;
   paracel_sync();
 }
