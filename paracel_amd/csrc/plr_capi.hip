@@ -960,6 +960,14 @@ struct DevBuf {  // device memory released on every exit path
   }
 };
 
+struct ShardGuard {  // a shard that was not completed does not stay resident
+  plr_ctx* c;
+  bool done = false;
+  ~ShardGuard() {
+    if (!done) free_shape(c);
+  }
+};
+
 // fields of the first non-empty line (maximal runs of non-separator bytes)
 int64_t first_line_fields(const char* const* text, const int64_t* len, int nspans, char sep) {
   for (int s = 0; s < nspans; ++s) {
@@ -1010,6 +1018,7 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   if (d > (int64_t)INT32_MAX) return fail(c, PLR_ERR_INVALID, "too many fields in a line");
   PLR_HIP(c, hipSetDevice(c->device));
   free_shape(c);
+  ShardGuard guard{c};
 
   // the text, spans back to back, padded with newlines
   DevBuf d_text, d_counts, d_first, d_rows, d_slow, d_ctl;
@@ -1051,10 +1060,7 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   c->synth_first_col = true;
   int rc = alloc_shape_buffers(c, n, d, /*zero_fill=*/true);
   c->synth_first_col = false;
-  if (rc != PLR_OK) {
-    free_shape(c);
-    return rc;
-  }
+  if (rc != PLR_OK) return rc;
   PLR_HIP(c, hipMalloc(&d_rows.p, (size_t)std::max<int64_t>(n, 1) * sizeof(int64_t)));
   hipLaunchKernelGGL(plr::csv_row_starts, dim3((unsigned)nblocks), dim3(plr::kCsvThreads), 0,
                      c->stream, dt, total, static_cast<const int64_t*>(d_first.p),
@@ -1090,10 +1096,7 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   PLR_HIP(c, hipMemcpyAsync(res, ctl, sizeof res, hipMemcpyDeviceToHost, c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
 
-  auto give_up = [&](int code, const std::string& msg) {
-    free_shape(c);
-    return fail(c, code, msg);
-  };
+  auto give_up = [&](int code, const std::string& msg) { return fail(c, code, msg); };
   if (res[1] != INT64_MAX)  // parse_lines' message for the same input
     return give_up(PLR_ERR_INVALID, "ragged sample line " + std::to_string(res[1]));
   const int nslow = (int)(res[2] & 0xffffffff);
@@ -1154,10 +1157,7 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
     };
     rc = patch(c->dX, xi, xv);
     if (rc == PLR_OK) rc = patch(c->dy, yi, yv);
-    if (rc != PLR_OK) {
-      free_shape(c);
-      return rc;
-    }
+    if (rc != PLR_OK) return rc;
   }
   c->csv_slow_fields = nslow;
   if (c->timing) {  // plr_get_timing's last_ms: the parsing kernel
@@ -1165,6 +1165,7 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
     PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
     c->last_ms = ms;
   }
+  guard.done = true;
   return PLR_OK;
 }
 
