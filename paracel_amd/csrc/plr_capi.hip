@@ -1169,6 +1169,8 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   return PLR_OK;
 }
 
+static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t count);
+
 int plr_get_data(plr_ctx* c, int64_t row0, int64_t nrows, double* X, int64_t ldx, double* y) {
   if (!c) return PLR_ERR_INVALID;
   if (!c->have_data) return fail(c, PLR_ERR_NODATA, "no shard resident: call plr_set_data first");
@@ -1179,33 +1181,35 @@ int plr_get_data(plr_ctx* c, int64_t row0, int64_t nrows, double* X, int64_t ldx
   if (X && ldx < c->d) return fail(c, PLR_ERR_INVALID, "ldx must be >= d");
   PLR_HIP(c, hipSetDevice(c->device));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
-  const int skip = c->bias ? 1 : 0;
-  if (X && c->lane) {
-    // row-tiled shard: blocks of rows are brought to row-major form on the device first
-    const int64_t cols = c->dcols;
-    const int64_t chunk_rows = std::max<int64_t>(1, (int64_t)(32u << 20) / (cols * 8));
+  if (X) {
+    // blocks of rows are brought to the caller's form on the device (dense rows of d
+    // doubles, the constant column included), then copied out through the pinned lanes
+    const int64_t d = c->d;
+    const int64_t chunk_rows = std::max<int64_t>(1, (int64_t)(256u << 20) / (d * 8));
     DevBuf stage;
-    PLR_HIP(c, hipMalloc(&stage.p, (size_t)std::min(chunk_rows, nrows) * cols * sizeof(double)));
+    PLR_HIP(c, hipMalloc(&stage.p, (size_t)std::min(chunk_rows, nrows) * d * sizeof(double)));
     for (int64_t r0 = 0; r0 < nrows; r0 += chunk_rows) {
       const int64_t m = std::min(chunk_rows, nrows - r0);
-      hipLaunchKernelGGL(plr::untile_rows, dim3((unsigned)ceil_div(m * cols, 256)), dim3(256), 0,
-                         c->stream, (const double*)c->dX, row0 + r0, m, (int)cols, c->lane->np,
-                         static_cast<double*>(stage.p));
+      hipLaunchKernelGGL(plr::gather_rows, dim3((unsigned)ceil_div(m * d, 256)), dim3(256), 0,
+                         c->stream, (const double*)c->dX, c->pitch, c->lane ? c->lane->np : 0,
+                         row0 + r0, m, (int)d, c->bias ? 1 : 0, static_cast<double*>(stage.p));
       PLR_HIP(c, hipGetLastError());
-      PLR_HIP(c, hipMemcpy2DAsync(X + r0 * ldx + skip, (size_t)ldx * sizeof(double), stage.p,
-                                  (size_t)cols * sizeof(double), (size_t)cols * sizeof(double),
-                                  (size_t)m, hipMemcpyDeviceToHost, c->stream));
       PLR_HIP(c, hipStreamSynchronize(c->stream));
+      if (ldx == d) {
+        const int rc = copy_rows_out(c, X + r0 * ldx, static_cast<const double*>(stage.p),
+                                     (size_t)(m * d));
+        if (rc != PLR_OK) return rc;
+      } else {
+        PLR_HIP(c, hipMemcpy2D(X + r0 * ldx, (size_t)ldx * sizeof(double), stage.p,
+                               (size_t)d * sizeof(double), (size_t)d * sizeof(double), (size_t)m,
+                               hipMemcpyDeviceToHost));
+      }
     }
-  } else if (X) {
-    PLR_HIP(c, hipMemcpy2D(X + skip, (size_t)ldx * sizeof(double), c->dX + row0 * c->pitch,
-                           (size_t)c->pitch * sizeof(double), (size_t)c->dcols * sizeof(double),
-                           (size_t)nrows, hipMemcpyDeviceToHost));
   }
-  if (X && skip)
-    for (int64_t r = 0; r < nrows; ++r) X[r * ldx] = 1.;
-  if (y)
-    PLR_HIP(c, hipMemcpy(y, c->dy + row0, (size_t)nrows * sizeof(double), hipMemcpyDeviceToHost));
+  if (y) {
+    const int rc = copy_rows_out(c, y, c->dy + row0, (size_t)nrows);
+    if (rc != PLR_OK) return rc;
+  }
   return PLR_OK;
 }
 

@@ -749,16 +749,22 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void lane_pass(PassArgs a) {
   emit_row_sums<WROW>(sums, lane, wr, a.part_loss, a.part_res);
 }
 
-// The inverse of tile_rows: rows row0 .. row0+nrows-1 of a row-tiled shard as
-// row-major rows of `cols` doubles (dst pitch = cols).
-__global__ void untile_rows(const double* X, int64_t row0, int64_t nrows, int cols, int np,
-                            double* dst) {
+// Rows row0 .. row0+nrows-1 of the shard as dense row-major rows of d doubles
+// (what plr_set_data takes): the inverse of the upload.  np > 0: the shard is
+// row-tiled (tile_rows); skip = 1: its constant first column is not stored and
+// comes back as 1.0.
+__global__ void gather_rows(const double* X, int64_t pitch, int np, int64_t row0, int64_t nrows,
+                            int d, int skip, double* dst) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= nrows * cols) return;
-  const int64_t r = i / cols;
-  const int col = (int)(i % cols);
+  if (i >= nrows * d) return;
+  const int64_t r = i / d;
+  const int col = (int)(i % d) - skip;
   const int64_t row = row0 + r;
-  dst[i] = X[((((row / kWave) * np + (col >> 1)) * kWave) + (row % kWave)) * 2 + (col & 1)];
+  double v = 1.;
+  if (col >= 0)
+    v = np > 0 ? X[((((row / kWave) * np + (col >> 1)) * kWave) + (row % kWave)) * 2 + (col & 1)]
+               : X[row * pitch + col];
+  dst[i] = v;
 }
 
 // lane_pass for the wider tiles (34..64 columns), where rows and accumulators
