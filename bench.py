@@ -538,7 +538,7 @@ def run_parse(a, cfg):
             "reference_stod_sample": "strtod per field as lr.cpp:76-93 does (oracle port), "
                                      "%.0f MB" % (len(sample) / 1e6)},
     }
-    print(json.dumps(out), flush=True)
+    return out
 
 
 def per_config_entry(rec):
@@ -589,7 +589,7 @@ def main():
         run_train(a, cfg)
         return
     if a.parse:
-        run_parse(a, cfg)
+        print(json.dumps(run_parse(a, cfg)), flush=True)
         return
 
     with_cpu = not a.no_cpu_baseline
@@ -611,6 +611,23 @@ def main():
             "cpu_iters_per_sec": (e2e.get("cpu_baseline") or {}).get("value"),
             "cpu_cores": (e2e.get("cpu_baseline") or {}).get("cores"),
             "step": e2e["config"]["step"]}
+        # the loader of the same configuration: its sample text parsed on the device
+        try:
+            pr = run_parse(a, cfgs["c5_e2e_2m_x_512"])
+            per["c5_e2e_2m_x_512_text_to_shard"] = {
+                "text_gb_per_sec": pr["value"], "ms_per_call": pr["ms_per_step"],
+                "text_bytes": pr["config"]["text_bytes"], "rows": pr["config"]["rows"],
+                "fields_per_row": pr["config"]["fields_per_row"],
+                "parse_kernel_ms": pr["roofline"]["kernel_ms"],
+                "parse_kernel_text_gbs": pr["roofline"]["text_gbs_kernel_only"],
+                "parse_kernel_frac_of_hbm": pr["roofline"]["frac"],
+                "cpu_text_gb_per_sec": pr["cpu_baseline"]["value"],
+                "cpu_cores": pr["cpu_baseline"]["cores"],
+                "cpu_text_gb_per_sec_1core": pr["cpu_baseline"]["value_1core"],
+                "reference_stod_1core_gbs": pr["cpu_baseline"]["reference_stod_1core_gbs"],
+                "step": pr["config"]["step"]}
+        except Exception as e:
+            per["c5_e2e_2m_x_512_text_to_shard"] = {"error": "%s: %s" % (type(e).__name__, e)}
         out["per_config"] = per
         extra = {}
         for other in OTHER_SHAPES:
