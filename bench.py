@@ -146,6 +146,9 @@ def parse_args():
     ap.add_argument("--parse", action="store_true",
                     help="the loader instead of the gradient step: sample text -> resident shard "
                          "on the device (plr_set_data_csv) against the host's parsers")
+    ap.add_argument("--parse-format", default="%.6f",
+                    help="with --parse: the printf format of the sample text's fields "
+                         "(e.g. %%.17g for full-precision spellings)")
     ap.add_argument("--ps-roundtrip", action="store_true",
                     help="host only: microseconds per paracel_read / paracel_bupdate round trip "
                          "against plr_ps_server, dense fast path on and off")
@@ -465,8 +468,10 @@ def run_parse(a, cfg):
 
     k = cfg.d - 1
     rng = np.random.default_rng(cfg.seed)
-    block_rows = max(64, int(48e6 // (k * 9.3 + 2)))
-    pool = np.array(["%.6f" % v for v in rng.normal(size=200000) * cfg.spec.scale * 3])
+    block_rows = max(64, int(48e6 // (k * (len(getattr(a, "parse_format", "%.6f") % -0.123456789) + 1)
+                                      + 2)))
+    fmt = getattr(a, "parse_format", "%.6f")
+    pool = np.array([fmt % v for v in rng.normal(size=200000) * cfg.spec.scale * 3])
     idx = rng.integers(0, pool.size, size=(block_rows, k))
     lab = rng.integers(0, 2, size=block_rows)
     t0 = time.time()
@@ -517,7 +522,8 @@ def run_parse(a, cfg):
         "n_gpus": 1, "steps": len(calls), "warmup": 1, "ms_per_step": 1e3 * call,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8 -> f64",
         "data": "synthetic",
-        "config": {"workload": cfg.name + " as text", "rows": n, "fields_per_row": cfg.d,
+        "config": {"workload": cfg.name + " as text", "field_format": fmt, "rows": n,
+                   "fields_per_row": cfg.d,
                    "text_bytes": nbytes, "step": "plr_set_data_csv: text host->device, row "
                    "offsets, parse into the resident shard (text in pageable host memory, so "
                    "the call includes its PCIe transfer)", "kernel": info},

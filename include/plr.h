@@ -74,9 +74,11 @@ int plr_set_data_chunk(plr_ctx* ctx, int64_t row0, int64_t nrows,
  * non-empty line "f1<sep>f2<sep>...<sep>fk<sep>label".  The resident shard is
  * what local_parser builds -- the sample [1.0, f1..fk] (d = k + 1 columns,
  * *d_out) and the label -- with every field's value exactly std::stod's: the
- * device converts the spellings for which one rounding gives that value, the
- * rest (more than 15 significant digits, inf, nan, hex, blanks, trailing
- * characters) are converted by std::stod on the host.  Empty fields are
+ * device converts decimal spellings of up to 19 significant digits whose
+ * correctly rounded value it can establish (all but those within 2^-30 of a
+ * unit in the last place of a rounding tie), the rest (longer digit strings,
+ * exponents beyond +-44, inf, nan, hex, blanks, trailing characters) are
+ * converted by std::stod on the host.  Empty fields are
  * skipped like the reference's str_split does.  *n_out receives the number
  * of samples.  Errors as the reference's parser would raise them (a field
  * std::stod rejects, a line with another number of fields) come back as

@@ -1084,7 +1084,7 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   ca.np = c->lane ? c->lane->np : 0;
   ca.slow = static_cast<plr::CsvSlow*>(d_slow.p);
   ca.slow_cap = slow_cap;
-  ca.slow_count = reinterpret_cast<int*>(ctl + 2);
+  ca.slow_count = reinterpret_cast<unsigned long long*>(ctl + 2);
   ca.bad_row = reinterpret_cast<long long*>(ctl + 1);
   const int64_t want = (n + 3) / 4;
   const unsigned grid = (unsigned)std::min<int64_t>(std::max<int64_t>(want, 1), (int64_t)c->num_cu * 8);
@@ -1099,10 +1099,10 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   auto give_up = [&](int code, const std::string& msg) { return fail(c, code, msg); };
   if (res[1] != INT64_MAX)  // parse_lines' message for the same input
     return give_up(PLR_ERR_INVALID, "ragged sample line " + std::to_string(res[1]));
-  const int nslow = (int)(res[2] & 0xffffffff);
-  if (nslow > slow_cap)
+  if (res[2] > (int64_t)slow_cap)
     return give_up(PLR_ERR_UNSUPPORTED,
                    "more than 2^20 fields need the host's number parser: parse this input there");
+  const int nslow = (int)res[2];
   if (nslow > 0) {
     // spellings the device does not convert: std::stod on the host's copy of the text
     std::vector<plr::CsvSlow> slow(nslow);
@@ -1160,6 +1160,7 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
     if (rc != PLR_OK) return rc;
   }
   c->csv_slow_fields = nslow;
+  c->info += "; parsed from text, " + std::to_string(nslow) + " fields converted on the host";
   if (c->timing) {  // plr_get_timing's last_ms: the parsing kernel
     float ms = 0.f;
     PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));

@@ -13,14 +13,21 @@
 //                    that starts in the wave's 64-byte window, the field's
 //                    characters fetched from the neighbouring lanes
 //
-// A field is converted on the device only when that is exact: the spelling
-// [-]digits[.digits][e[+-]digits] with at most 15 significant digits and a
-// decimal exponent within +-22.  Its digits are then an exact double, 10^|e|
-// is an exact double, and the one multiplication or division rounds once --
-// the correctly rounded value, which is what strtod returns (Clinger's fast
-// path; the host parser in worker/shard_io.hpp takes the same route).  Every
-// other spelling is put on a list the host resolves with std::stod itself, so
-// values and errors are the reference's for every input.
+// A field is converted on the device only when the result is provably strtod's,
+// the correctly rounded value of the decimal.  The spelling must be
+// [-]digits[.digits][e[+-]digits]; then
+//   * at most 15 significant digits and a decimal exponent within +-22: the
+//     digits are an exact double, 10^|e| is an exact double, and the one
+//     multiplication or division rounds once (Clinger's fast path; the host
+//     parser in worker/shard_io.hpp takes the same route);
+//   * up to 19 significant digits (what "%.17g", repr() and "%.18e" write) and
+//     an exponent within +-44: the digits, an exact 64-bit integer, are scaled
+//     in double-double arithmetic (106 bits), and the result is taken only when
+//     those 106 bits place the value clearly on one side of the nearest
+//     rounding boundary -- anything closer than 2^-30 of a unit in the last
+//     place to a tie, exact ties included, is left alone.
+// Every other field is put on a list the host resolves with std::stod itself,
+// so values and errors are the reference's for every input.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -55,7 +62,7 @@ struct CsvArgs {
   int np;                     // > 0: row-tiled layout with np column pairs per row
   CsvSlow* slow;
   int slow_cap;
-  int* slow_count;
+  unsigned long long* slow_count;
   long long* bad_row;         // smallest row whose field count is not d
 };
 
@@ -152,6 +159,44 @@ __device__ const double kCsvPow10[23] = {1e0,  1e1,  1e2,  1e3,  1e4,  1e5,  1e6
                                          1e8,  1e9,  1e10, 1e11, 1e12, 1e13, 1e14, 1e15,
                                          1e16, 1e17, 1e18, 1e19, 1e20, 1e21, 1e22};
 
+// m * 10^e for 1 <= m < 2^64 and |e| <= 44, correctly rounded -- or false when
+// 106 bits cannot tell on which side of a rounding boundary the value lies.
+// The intrinsics keep every operation a single IEEE operation (no contraction).
+__device__ __forceinline__ bool csv_scale_dd(unsigned long long m, int e, double& out) {
+  // the integer as an unevaluated sum hi + lo of two doubles, exact
+  double h = (double)m;  // round to nearest
+  double l = (double)(long long)(m - (unsigned long long)h);  // |l| <= 2^10
+  int left = e < 0 ? -e : e;
+  while (left > 0) {
+    const int k = left > 22 ? 22 : left;
+    const double p = kCsvPow10[k];  // exact
+    left -= k;
+    double a, b;
+    if (e < 0) {
+      // (h + l) / p: quotient of the high part, its exact remainder, the correction
+      a = __ddiv_rn(h, p);
+      const double r = __dadd_rn(__fma_rn(-a, p, h), l);
+      b = __ddiv_rn(r, p);
+    } else {
+      // (h + l) * p: product of the high part with its exact error, plus the low part's
+      a = __dmul_rn(h, p);
+      b = __dadd_rn(__fma_rn(h, p, -a), __dmul_rn(l, p));
+    }
+    h = __dadd_rn(a, b);                  // |b| << |a|: fast two-sum
+    l = __dadd_rn(b, __dsub_rn(a, h));
+  }
+  // h is the value rounded to nearest unless hi + lo sits next to a tie: the
+  // midpoint towards the neighbour on lo's side (below a power of two the
+  // neighbour is half as far away)
+  const long long hb = __double_as_longlong(h);  // h > 0
+  const double nb = __longlong_as_double(l < 0. ? hb - 1 : hb + 1);
+  const double half = __dmul_rn(0.5, fabs(__dsub_rn(nb, h)));
+  const double off = fabs(__dsub_rn(fabs(l), half));
+  if (off <= __dmul_rn(half, 9.313225746154785e-10)) return false;        // 2^-30
+  out = h;
+  return true;
+}
+
 __device__ __forceinline__ int csv_wave_max(int v) {
 #pragma unroll
   for (int m = 1; m < 64; m <<= 1) {
@@ -216,7 +261,7 @@ __global__ __launch_bounds__(256) void csv_parse(CsvArgs a) {
           if (digit) {
             m = m * 10ull + (unsigned long long)(ch - '0');
             if (m) ++sig;
-            if (sig > 15) bad = true;
+            if (sig > 19) bad = true;  // 19 digits fit 64 bits
             ++ndig;
             if (st == 1) ++frac;
           } else if (ch == '-' && j == 0) {
@@ -244,11 +289,20 @@ __global__ __launch_bounds__(256) void csv_parse(CsvArgs a) {
       if (start) {
         const int col = nfields + __builtin_popcountll(start_mask & below);
         int e = (eneg ? -e10 : e10) - frac;
-        if (ndig == 0 || st == 2 || (st == 3 && ed == 0) || e < -22 || e > 22) bad = true;
+        if (ndig == 0 || st == 2 || (st == 3 && ed == 0) || e < -44 || e > 44) bad = true;
+        double v = 0.;
+        if (!bad) {
+          if (sig <= 15 && e >= -22 && e <= 22) {
+            v = (double)m;
+            v = e < 0 ? v / kCsvPow10[-e] : v * kCsvPow10[e];
+          } else if (m == 0) {
+            v = 0.;
+          } else if (!csv_scale_dd(m, e, v)) {
+            bad = true;
+          }
+        }
         if (col < a.d) {
           if (!bad) {
-            double v = (double)m;
-            v = e < 0 ? v / kCsvPow10[-e] : v * kCsvPow10[e];
             if (neg) v = -v;
             if (col == a.d - 1) {
               a.y[r] = v;
@@ -258,8 +312,8 @@ __global__ __launch_bounds__(256) void csv_parse(CsvArgs a) {
               a.X[r * a.pitch + col] = v;
             }
           } else {
-            const int k = atomicAdd(a.slow_count, 1);
-            if (k < a.slow_cap) {
+            const unsigned long long k = atomicAdd(a.slow_count, 1ull);
+            if (k < (unsigned long long)a.slow_cap) {
               CsvSlow s;
               s.row = r;
               s.pos = pos + lane;

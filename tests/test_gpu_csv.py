@@ -118,6 +118,56 @@ def test_fields_the_host_converts_and_odd_lines(plr, oracle):
     assert (n, d) == (1, 3) and np.isnan(X[0, 1]) and X[0, 2] == 1.0 and y[0] == 1.0
 
 
+def host_converted(plr):
+    return int(plr.kernel_info().split("parsed from text, ")[1].split(" ")[0])
+
+
+def test_long_mantissas_are_converted_on_the_device_and_still_exact(plr, oracle):
+    # 16..19 significant digits (what "%.17g", repr() and "%.18e" write): scaled in
+    # double-double arithmetic on the device, left to the host only next to a rounding tie
+    rng = np.random.default_rng(77)
+    n, k = 4000, 24
+    vals = rng.normal(size=(n, k)) * 10.0 ** rng.integers(-12, 13, size=(n, k))
+    fmts = ["%.17g", "%.18e", "%.16g", "%.17e", "%r", "%.19g"]
+    lines = []
+    for i in range(n):
+        f = []
+        for j in range(k):
+            fmt = fmts[(i + j) % len(fmts)]
+            f.append(repr(float(vals[i, j])) if fmt == "%r" else fmt % vals[i, j])
+        lines.append(",".join(f) + ",1")
+    check_equal(plr, oracle, "\n".join(lines) + "\n")
+    assert host_converted(plr) <= n * k // 200      # "%.19g" digits beyond 2^64 and the like
+    # integers and decimals of 16..19 random digits, scaled by 10^-44..10^44
+    lines = []
+    for i in range(3000):
+        f = []
+        for j in range(12):
+            nd = int(rng.integers(16, 20))
+            m = "".join(str(int(t)) for t in rng.integers(0, 10, size=nd))
+            m = str(int(rng.integers(1, 10))) + m[1:]
+            cut = int(rng.integers(0, nd + 1))
+            body = (m[:cut] + "." + m[cut:]) if j % 3 else m
+            if j % 4 == 1:
+                body += "e%+d" % int(rng.integers(-30, 31))
+            f.append(("-" if (i + j) % 5 == 0 else "") + body)
+        lines.append(",".join(f) + ",0")
+    check_equal(plr, oracle, "\n".join(lines) + "\n")
+    # a larger sample over 80 decades: 600 000 fields of 17 digits
+    n, k = 3000, 200
+    vals = rng.normal(size=(n, k)) * 10.0 ** rng.integers(-38, 24, size=(n, k))
+    text = "\n".join(",".join("%.17g" % v for v in row) + ",1" for row in vals) + "\n"
+    check_equal(plr, oracle, text)
+    print("600000 fields of 17 digits: %d converted on the host" % host_converted(plr), flush=True)
+    # exact ties and their neighbours: 2^53 + 1 is halfway between two doubles
+    ties = ["9007199254740993", "9007199254740992", "9007199254740994", "9007199254740995",
+            "9007199254740993.0000", "9.007199254740993e15", "4503599627370497.5",
+            "0.50000000000000005551", "1.0000000000000001110", "2.00000000000000022204",
+            "1152921504606846977", "18446744073709551615", "9999999999999999999",
+            "0.9999999999999999444", "1.00000000000000011102230246251565"]
+    check_equal(plr, oracle, "\n".join(t + ",1,1" for t in ties) + "\n")
+
+
 def test_pieces_of_text_and_rows_across_windows(plr, oracle):
     rng = np.random.default_rng(9)
     text = make_text(rng, 333, 12, kinds=[0, 1, 8])
