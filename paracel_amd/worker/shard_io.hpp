@@ -30,6 +30,7 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <cmath>
 #include <stdexcept>
 #include <memory>
 #include <string>
@@ -218,14 +219,57 @@ struct ParsedShard {
   std::vector<double> X, y;      // X: n x d row-major
 };
 
+// m * 10^e for 1 <= m < 2^64 and |e| <= 44, correctly rounded -- or false when
+// 106 bits cannot tell on which side of a rounding boundary the value lies.
+// The integer is split exactly into two doubles and scaled in double-double
+// arithmetic: the quotient (product) of the high part, its exact remainder
+// (error) by FMA, the correction from the low part; the result is good to
+// about 2^-100, and the high word is taken only when the low word is not within
+// 2^-30 of a unit in the last place of the midpoint towards the neighbour on
+// its side (exact ties included).  Every operation below must stay a single
+// IEEE operation: this file is compiled with -ffp-contract=off.  The device
+// parser (csrc/plr_csv.hpp) runs the same sequence.
+inline bool scale_exact_dd(uint64_t m, int e, const double* pow10, double& out) {
+  double h = (double)m;
+  double l = (double)(int64_t)(m - (uint64_t)h);
+  int left = e < 0 ? -e : e;
+  while (left > 0) {
+    const int k = left > 22 ? 22 : left;
+    const double p = pow10[k];
+    left -= k;
+    double a, b;
+    if (e < 0) {
+      a = h / p;
+      const double r = std::fma(-a, p, h) + l;
+      b = r / p;
+    } else {
+      a = h * p;
+      b = std::fma(h, p, -a) + l * p;
+    }
+    h = a + b;
+    l = b + (a - h);
+  }
+  int64_t hb;
+  memcpy(&hb, &h, sizeof hb);
+  hb += l < 0. ? -1 : 1;
+  double nb;
+  memcpy(&nb, &hb, sizeof nb);
+  const double half = 0.5 * std::fabs(nb - h);
+  if (std::fabs(std::fabs(l) - half) <= half * 9.313225746154785e-10) return false;  // 2^-30
+  out = h;
+  return true;
+}
+
 // std::stod's value for one field, without the library call for the common
-// spelling: [-]digits[.digits][e[+-]digits] with at most 15 significant
-// digits and a decimal exponent within +-22.  Then the digits are an exact
-// double, 10^|e| is an exact double, and the one multiplication or division
-// rounds once -- the correctly rounded result, which is what strtod returns
-// (Clinger's fast path).  Every other spelling (more digits, hex floats, inf,
-// nan, leading blanks or '+', trailing garbage) and every error goes through
-// std::stod itself, so the exceptions are the reference's too.
+// spellings [-]digits[.digits][e[+-]digits]:
+//   * at most 15 significant digits and a decimal exponent within +-22: the
+//     digits are an exact double, 10^|e| is an exact double, and the one
+//     multiplication or division rounds once -- the correctly rounded result,
+//     which is what strtod returns (Clinger's fast path);
+//   * up to 19 significant digits and an exponent within +-44: scale_exact_dd.
+// Every other spelling (more digits, hex floats, inf, nan, leading blanks or
+// '+', trailing garbage) and every error goes through std::stod itself, so the
+// exceptions are the reference's too.
 inline double parse_field(const char* p, size_t len) {
   static const double kPow10[23] = {1e0,  1e1,  1e2,  1e3,  1e4,  1e5,  1e6,  1e7,
                                     1e8,  1e9,  1e10, 1e11, 1e12, 1e13, 1e14, 1e15,
@@ -242,14 +286,14 @@ inline double parse_field(const char* p, size_t len) {
   for (; q < end && *q >= '0' && *q <= '9'; ++q, ++ndig) {
     m = m * 10 + (uint64_t)(*q - '0');
     if (m) ++sig;
-    if (sig > 15) goto slow;
+    if (sig > 19) goto slow;
   }
   if (q < end && *q == '.') {
     ++q;
     for (; q < end && *q >= '0' && *q <= '9'; ++q, ++ndig, ++frac) {
       m = m * 10 + (uint64_t)(*q - '0');
       if (m) ++sig;
-      if (sig > 15) goto slow;
+      if (sig > 19) goto slow;
     }
   }
   if (ndig == 0) goto slow;
@@ -269,9 +313,14 @@ inline double parse_field(const char* p, size_t len) {
     }
     if (q != end) goto slow;
     e10 -= frac;
-    if (e10 < -22 || e10 > 22) goto slow;
-    double v = (double)m;
-    v = (e10 < 0) ? v / kPow10[-e10] : v * kPow10[e10];
+    if (e10 < -44 || e10 > 44) goto slow;
+    double v = 0.;
+    if (sig <= 15 && e10 >= -22 && e10 <= 22) {
+      v = (double)m;
+      v = (e10 < 0) ? v / kPow10[-e10] : v * kPow10[e10];
+    } else if (m != 0 && !scale_exact_dd(m, e10, kPow10, v)) {
+      goto slow;
+    }
     return neg ? -v : v;
   }
 slow:

@@ -15,7 +15,7 @@
 #include "shard_io.hpp"
 
 // A random field: mostly decimal spellings around the limits of the fast path
-// (digit counts 1..20, exponents around +-22, zeros, signs), some spellings
+// (digit counts 1..38, exponents around +-22 and +-44, zeros, signs), some spellings
 // only std::stod understands, some it rejects.
 static std::string random_field(std::mt19937_64& rng) {
   auto pick = [&](int n) { return (int)(rng() % (uint64_t)n); };
@@ -25,7 +25,7 @@ static std::string random_field(std::mt19937_64& rng) {
   if (pick(16) == 0) return odd[pick((int)(sizeof odd / sizeof *odd))];
   std::string s;
   if (pick(2)) s += '-';
-  const int ni = pick(12), nf = pick(12);
+  const int ni = pick(3) ? pick(12) : pick(20), nf = pick(3) ? pick(12) : pick(20);
   for (int i = 0; i < ni; ++i) s += (char)('0' + (pick(4) == 0 ? 0 : pick(10)));
   if (nf || pick(3) == 0) {
     s += '.';
@@ -36,7 +36,7 @@ static std::string random_field(std::mt19937_64& rng) {
     const int k = pick(3);
     if (k == 0) s += '-';
     if (k == 1) s += '+';
-    s += std::to_string(pick(3) == 0 ? pick(400) : pick(30));
+    s += std::to_string(pick(3) == 0 ? pick(400) : pick(60));
   }
   return s;
 }
