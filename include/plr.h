@@ -205,6 +205,9 @@ int plr_set_timing(plr_ctx* ctx, int enabled);
  *        have given.  The upload checks the statement row by row and fails
  *        with PLR_ERR_INVALID at the first row that does not start with 1.0.
  *        Applies from the next plr_set_data / plr_alloc_data.  Default 0.
+ *   "csv_lane_per_row"  which kernel plr_set_data_csv parses with: 1 a lane
+ *        per row (64 rows per wave), 0 a wave per row, -1 (default) by the
+ *        number of rows.  Same results either way.
  *   "column_blocks_two_sweeps"  value != 0: rows wider than 19456 columns are
  *        processed in two sweeps over X (dot products, then updates) instead
  *        of once by cooperating workgroups; applies from the next

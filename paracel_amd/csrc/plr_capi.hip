@@ -216,6 +216,7 @@ struct plr_ctx {
   unsigned team_spin_limit = kTeamSpinLimit;
   bool opt_two_sweeps = false;  // plr_set_option("column_blocks_two_sweeps")
   bool synth_first_col = false; // the shard being reserved comes from plr_set_data_csv
+  int opt_csv_lane_rows = -1;   // plr_set_option("csv_lane_per_row"): -1 by row count, 0, 1
   int csv_slow_fields = 0;      // fields of the last plr_set_data_csv the host converted
   bool team_check = false;      // a team pass ran since the status word was last read
   double* d_z = nullptr;        // n: blocked rows only, x.theta accumulated over the blocks
@@ -1086,10 +1087,16 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   ca.slow_cap = slow_cap;
   ca.slow_count = reinterpret_cast<unsigned long long*>(ctl + 2);
   ca.bad_row = reinterpret_cast<long long*>(ctl + 1);
-  const int64_t want = (n + 3) / 4;
-  const unsigned grid = (unsigned)std::min<int64_t>(std::max<int64_t>(want, 1), (int64_t)c->num_cu * 8);
+  ca.flush_at = 52;  // of 64 lanes (sweep: 32..64 within 3 %, 1 is 40 % slower)
+  // many rows: a lane per row (every lane in the character step); few rows: a wave per row
+  const bool lane_rows = c->opt_csv_lane_rows < 0 ? n >= (int64_t)c->num_cu * 4 * 64 * 2
+                                                  : c->opt_csv_lane_rows != 0;
+  const int64_t want = lane_rows ? (n + 255) / 256 : (n + 3) / 4;
+  const unsigned grid = (unsigned)std::min<int64_t>(
+      std::max<int64_t>(want, 1), (int64_t)c->num_cu * 8);
   if (c->timing) PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
-  hipLaunchKernelGGL(plr::csv_parse, dim3(grid), dim3(256), 0, c->stream, ca);
+  hipLaunchKernelGGL(lane_rows ? plr::csv_parse_rows : plr::csv_parse, dim3(grid), dim3(256), 0,
+                     c->stream, ca);
   PLR_HIP(c, hipGetLastError());
   if (c->timing) PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
   int64_t res[3] = {0, 0, 0};
@@ -1160,7 +1167,8 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
     if (rc != PLR_OK) return rc;
   }
   c->csv_slow_fields = nslow;
-  c->info += "; parsed from text, " + std::to_string(nslow) + " fields converted on the host";
+  c->info += std::string("; parsed from text (a ") + (lane_rows ? "lane" : "wave") +
+             " per row), " + std::to_string(nslow) + " fields converted on the host";
   if (c->timing) {  // plr_get_timing's last_ms: the parsing kernel
     float ms = 0.f;
     PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
@@ -1496,6 +1504,10 @@ int plr_set_option(plr_ctx* c, const char* key, int64_t value) {
   }
   if (strcmp(key, "first_column_is_one") == 0) {
     c->opt_first_col_one = value != 0;  // takes effect at the next plr_set_data / plr_alloc_data
+    return PLR_OK;
+  }
+  if (strcmp(key, "csv_lane_per_row") == 0) {
+    c->opt_csv_lane_rows = value < 0 ? -1 : (value != 0);
     return PLR_OK;
   }
   if (strcmp(key, "column_blocks_two_sweeps") == 0) {

@@ -11,11 +11,13 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def plr():
+@pytest.fixture(scope="module", params=["wave per row", "lane per row"])
+def plr(request):
+    # both parsing kernels on every input (the library picks by row count otherwise)
     from paracel_amd import Plr
 
     with Plr(0) as c:
+        c.set_option("csv_lane_per_row", int(request.param == "lane per row"))
         yield c
 
 
@@ -65,6 +67,7 @@ def check_equal(plr, oracle, text, pieces=None, sep=","):
     n, d = plr.set_data_csv(pieces if pieces is not None else data, sep=sep)
     assert (n, d) == Xo.shape
     assert "not stored" in plr.kernel_info()
+    assert ("a lane per row" in plr.kernel_info()) or ("a wave per row" in plr.kernel_info())
     X, y = plr.get_data()
     assert X.tobytes() == Xo.tobytes()
     assert y.tobytes() == yo.tobytes()
@@ -119,7 +122,7 @@ def test_fields_the_host_converts_and_odd_lines(plr, oracle):
 
 
 def host_converted(plr):
-    return int(plr.kernel_info().split("parsed from text, ")[1].split(" ")[0])
+    return int(plr.kernel_info().split("per row), ")[1].split(" ")[0])
 
 
 def test_long_mantissas_are_converted_on_the_device_and_still_exact(plr, oracle):
