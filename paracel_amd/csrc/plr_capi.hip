@@ -993,6 +993,14 @@ int64_t first_line_fields(const char* const* text, const int64_t* len, int nspan
 
 }  // namespace
 
+static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t count);
+struct CopyPiece {  // bytes of pageable host memory and where on the device they go
+  void* dev;
+  const void* src;
+  size_t bytes;
+};
+static int copy_bytes_in(plr_ctx* c, const std::vector<CopyPiece>& pieces);
+
 int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, int nspans,
                      char sep, int64_t* n_out, int64_t* d_out) {
   if (!c) return PLR_ERR_INVALID;
@@ -1030,12 +1038,15 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   }
   unsigned char* dt = static_cast<unsigned char*>(d_text.p);
   std::vector<int64_t> span_at(nspans + 1, 0);  // device offset of every span
+  std::vector<CopyPiece> pieces;
   for (int s = 0; s < nspans; ++s) {
-    if (len[s])
-      PLR_HIP(c, hipMemcpyAsync(dt + span_at[s], text[s], (size_t)len[s], hipMemcpyHostToDevice,
-                                c->stream));
+    if (len[s]) pieces.push_back({dt + span_at[s], text[s], (size_t)len[s]});
     PLR_HIP(c, hipMemsetAsync(dt + span_at[s] + len[s], '\n', 1, c->stream));
     span_at[s + 1] = span_at[s] + len[s] + 1;
+  }
+  {
+    const int rc = copy_bytes_in(c, pieces);
+    if (rc != PLR_OK) return rc;
   }
   PLR_HIP(c, hipMemsetAsync(dt + total, '\n', (size_t)(padded - total), c->stream));
 
@@ -1177,8 +1188,6 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   guard.done = true;
   return PLR_OK;
 }
-
-static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t count);
 
 int plr_get_data(plr_ctx* c, int64_t row0, int64_t nrows, double* X, int64_t ldx, double* y) {
   if (!c) return PLR_ERR_INVALID;
@@ -1393,6 +1402,69 @@ static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t coun
       (void)hipGetLastError();
       return fail(c, PLR_ERR_HIP,
                   std::string("copying the predictions out failed: ") + hipGetErrorString(errs[l]));
+    }
+  return PLR_OK;
+}
+
+// The other direction, for bytes: pieces of pageable host memory into the device through
+// the same pinned lanes.  The pieces are cut into staging-block sized jobs dealt to the lanes
+// in turn; a lane's thread fills one of its two blocks while the other is in flight.
+static int copy_bytes_in(plr_ctx* c, const std::vector<CopyPiece>& pieces) {
+  size_t total = 0;
+  std::vector<CopyPiece> jobs;
+  for (const CopyPiece& p : pieces) {
+    total += p.bytes;
+    for (size_t at = 0; at < p.bytes; at += kCopyBlock)
+      jobs.push_back({static_cast<char*>(p.dev) + at, static_cast<const char*>(p.src) + at,
+                      std::min(kCopyBlock, p.bytes - at)});
+  }
+  if (total < 4 * kCopyBlock) {
+    for (const CopyPiece& p : pieces)
+      if (p.bytes) PLR_HIP(c, hipMemcpy(p.dev, p.src, p.bytes, hipMemcpyHostToDevice));
+    return PLR_OK;
+  }
+  if (!c->out_stage) {
+    PLR_HIP(c, hipHostMalloc(&c->out_stage, 2 * kCopyLanes * kCopyBlock, hipHostMallocDefault));
+    for (int l = 0; l < kCopyLanes; ++l)
+      PLR_HIP(c, hipStreamCreateWithFlags(&c->out_stream[l], hipStreamNonBlocking));
+  }
+  hipError_t errs[kCopyLanes];
+  std::thread th[kCopyLanes];
+  for (int l = 0; l < kCopyLanes; ++l) {
+    errs[l] = hipSuccess;
+    th[l] = std::thread([&, l]() {
+      if (hipSetDevice(c->device) != hipSuccess) {
+        errs[l] = hipErrorInvalidDevice;
+        return;
+      }
+      char* stage = static_cast<char*>(c->out_stage) + (size_t)l * 2 * kCopyBlock;
+      hipStream_t st = c->out_stream[l];
+      hipEvent_t freed[2] = {nullptr, nullptr};
+      if (hipEventCreateWithFlags(&freed[0], hipEventDisableTiming) != hipSuccess ||
+          hipEventCreateWithFlags(&freed[1], hipEventDisableTiming) != hipSuccess)
+        errs[l] = hipErrorOutOfMemory;
+      int slot = 0;
+      size_t round = 0;
+      for (size_t j = l; j < jobs.size() && errs[l] == hipSuccess; j += kCopyLanes, ++round, slot ^= 1) {
+        // the block sent from this slot two rounds ago must have left it
+        if (round >= 2 && hipEventSynchronize(freed[slot]) != hipSuccess) errs[l] = hipErrorUnknown;
+        char* blk = stage + (size_t)slot * kCopyBlock;
+        memcpy(blk, jobs[j].src, jobs[j].bytes);
+        hipError_t e = hipMemcpyAsync(jobs[j].dev, blk, jobs[j].bytes, hipMemcpyHostToDevice, st);
+        if (e == hipSuccess) e = hipEventRecord(freed[slot], st);
+        if (e != hipSuccess) errs[l] = e;
+      }
+      if (hipStreamSynchronize(st) != hipSuccess && errs[l] == hipSuccess) errs[l] = hipErrorUnknown;
+      for (int k = 0; k < 2; ++k)
+        if (freed[k]) (void)hipEventDestroy(freed[k]);
+    });
+  }
+  for (int l = 0; l < kCopyLanes; ++l) th[l].join();
+  for (int l = 0; l < kCopyLanes; ++l)
+    if (errs[l] != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(c, PLR_ERR_HIP, std::string("copying the text to the device failed: ") +
+                                      hipGetErrorString(errs[l]));
     }
   return PLR_OK;
 }
