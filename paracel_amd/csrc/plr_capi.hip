@@ -18,6 +18,14 @@
 #include "plr_kernels.hpp"
 #include "plr_plan.hpp"
 
+struct plr_ctx;
+struct CopyPiece {  // bytes of pageable host memory and where on the device they go
+  void* dev;
+  const void* src;
+  size_t bytes;
+};
+static int copy_bytes_in(plr_ctx* c, const std::vector<CopyPiece>& pieces);
+
 namespace {
 
 using plr::FinishArgs;
@@ -570,9 +578,11 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
       }
   }
   const bool tiled = c->lane != nullptr;
-  if (!tiled && !c->bias && ldx == c->pitch && c->d == c->pitch) {  // same pitch, no pad column: one linear copy
-    PLR_HIP(c, hipMemcpy(c->dX + row0 * c->pitch, X,
-                         (size_t)nrows * c->pitch * sizeof(double), hipMemcpyHostToDevice));
+  if (!tiled && !c->bias && ldx == c->pitch && c->d == c->pitch) {
+    // same pitch, no pad column: one linear stretch, through the pinned lanes
+    const int rc = copy_bytes_in(
+        c, {{c->dX + row0 * c->pitch, X, (size_t)nrows * c->pitch * sizeof(double)}});
+    if (rc != PLR_OK) return rc;
   } else {
     // Different pitches: a strided copy command moves one row per transfer
     // (~1 GB/s).  Repack the rows at the device pitch into two pinned staging
@@ -994,12 +1004,6 @@ int64_t first_line_fields(const char* const* text, const int64_t* len, int nspan
 }  // namespace
 
 static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t count);
-struct CopyPiece {  // bytes of pageable host memory and where on the device they go
-  void* dev;
-  const void* src;
-  size_t bytes;
-};
-static int copy_bytes_in(plr_ctx* c, const std::vector<CopyPiece>& pieces);
 
 int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, int nspans,
                      char sep, int64_t* n_out, int64_t* d_out) {
