@@ -9,6 +9,8 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
+#include <functional>
 #include <mutex>
 #include <string>
 #include <thread>
@@ -25,6 +27,7 @@ struct CopyPiece {  // bytes of pageable host memory and where on the device the
   size_t bytes;
 };
 static int copy_bytes_in(plr_ctx* c, const std::vector<CopyPiece>& pieces);
+static int copy_rows_in(plr_ctx* c, int64_t row0, int64_t nrows, const double* X, int64_t ldx);
 
 namespace {
 
@@ -238,9 +241,6 @@ struct plr_ctx {
   double* h_pred_dev = nullptr;
   void* out_stage = nullptr;    // pinned staging of copy_rows_out, lazily allocated
   hipStream_t out_stream[4] = {nullptr, nullptr, nullptr, nullptr};
-  double* up_stage[2] = {nullptr, nullptr};  // pinned repack buffers for pitched uploads
-  hipEvent_t up_done[2] = {nullptr, nullptr};
-  size_t up_stage_bytes = 0;
   double* d_curve = nullptr;    // per-round losses of plr_train_dgd, lazily allocated
   double* d_train_out = nullptr;  // d + 1: where training rounds put delta (never read back)
   int curve_len = 0;
@@ -278,13 +278,6 @@ int fail(plr_ctx* c, int code, const std::string& msg) {
   } while (0)
 
 void release_upload_staging(plr_ctx* c) {
-  for (int k = 0; k < 2; ++k) {
-    if (c->up_done[k]) (void)hipEventDestroy(c->up_done[k]);
-    if (c->up_stage[k]) (void)hipHostFree(c->up_stage[k]);
-    c->up_done[k] = nullptr;
-    c->up_stage[k] = nullptr;
-  }
-  c->up_stage_bytes = 0;
   if (c->up_dev) (void)hipFree(c->up_dev);
   c->up_dev = nullptr;
 }
@@ -567,92 +560,9 @@ int upload_rows(plr_ctx* c, int64_t row0, int64_t nrows, const double* X,
   if (row0 < 0 || nrows < 0 || row0 + nrows > c->n)
     return fail(c, PLR_ERR_INVALID, "row range outside the reserved shard");
   PLR_HIP(c, hipSetDevice(c->device));
-  const int skip = c->bias ? 1 : 0;  // the constant first column stays on the host
-  if (c->bias) {
-    for (int64_t r = 0; r < nrows; ++r)
-      if (X[r * ldx] != 1.) {
-        char b[160];
-        snprintf(b, sizeof b, "first_column_is_one is set, but row %lld starts with %.17g",
-                 (long long)(row0 + r), X[r * ldx]);
-        return fail(c, PLR_ERR_INVALID, b);
-      }
-  }
-  const bool tiled = c->lane != nullptr;
-  if (!tiled && !c->bias && ldx == c->pitch && c->d == c->pitch) {
-    // same pitch, no pad column: one linear stretch, through the pinned lanes
-    const int rc = copy_bytes_in(
-        c, {{c->dX + row0 * c->pitch, X, (size_t)nrows * c->pitch * sizeof(double)}});
-    if (rc != PLR_OK) return rc;
-  } else {
-    // Different pitches: a strided copy command moves one row per transfer
-    // (~1 GB/s).  Repack the rows at the device pitch into two pinned staging
-    // buffers on the host and send those as linear copies, the packing of one
-    // overlapping the transfer of the other.
-    // Row-tiled shards: the rows go, stored columns only, into a staging
-    // buffer on the device, and tile_rows brings each block into the layout
-    // (same stream: the next block's copy waits for it).  Host rows that are
-    // already dense are sent from where they lie.
-    const int64_t sp = tiled ? c->dcols : c->pitch;  // pitch of the staged rows
-    const bool direct = tiled && !c->bias && ldx == c->dcols;
-    const int64_t chunk_rows = std::max<int64_t>(1, (int64_t)(32u << 20) / (sp * 8));
-    const size_t stage_bytes = (size_t)chunk_rows * sp * sizeof(double);
-    int rc = PLR_OK;
-    if (c->up_stage_bytes < stage_bytes) {  // kept for the shard's lifetime: chunked uploads reuse them
-      release_upload_staging(c);
-      for (int k = 0; k < 2 && rc == PLR_OK; ++k) {
-        if (hipHostMalloc(&c->up_stage[k], stage_bytes, hipHostMallocDefault) != hipSuccess ||
-            hipEventCreate(&c->up_done[k]) != hipSuccess) {
-          (void)hipGetLastError();
-          rc = fail(c, PLR_ERR_NOMEM, "cannot allocate the pinned upload staging buffers");
-        }
-      }
-      if (rc == PLR_OK && tiled && hipMalloc(&c->up_dev, stage_bytes) != hipSuccess) {
-        (void)hipGetLastError();
-        rc = fail(c, PLR_ERR_NOMEM, "cannot allocate the device upload staging buffer");
-      }
-      if (rc != PLR_OK) {
-        release_upload_staging(c);
-        return rc;
-      }
-      c->up_stage_bytes = stage_bytes;
-    }
-    double** stage = c->up_stage;
-    hipEvent_t* done = c->up_done;
-    int k = 0;
-    for (int64_t r0 = 0; r0 < nrows && rc == PLR_OK; r0 += chunk_rows, k ^= 1) {
-      const int64_t m = std::min<int64_t>(chunk_rows, nrows - r0);
-      if (r0 >= 2 * chunk_rows && hipEventSynchronize(done[k]) != hipSuccess)
-        rc = fail(c, PLR_ERR_HIP, "upload: waiting for a staging buffer failed");
-      for (int64_t r = 0; r < m && rc == PLR_OK && !direct; ++r) {
-        double* dst = stage[k] + r * sp;
-        memcpy(dst, X + (r0 + r) * ldx + skip, (size_t)c->dcols * sizeof(double));
-        for (int64_t j = c->dcols; j < sp; ++j) dst[j] = 0.;
-      }
-      const double* src = direct ? X + r0 * ldx : stage[k];
-      double* dst = tiled ? c->up_dev : c->dX + (row0 + r0) * c->pitch;
-      if (rc == PLR_OK && hipMemcpyAsync(dst, src, (size_t)m * sp * sizeof(double),
-                                         hipMemcpyHostToDevice, c->stream) != hipSuccess)
-        rc = fail(c, PLR_ERR_HIP, "upload: host-to-device copy failed");
-      if (rc == PLR_OK && tiled) {
-        const int np = c->lane->np;
-        const int64_t threads = ceil_div(m, plr::kWave) * plr::kWave * np;
-        hipLaunchKernelGGL(plr::tile_rows, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
-                           c->stream, (const double*)c->up_dev, sp, m, (int)c->dcols, c->dX,
-                           row0 + r0, np);
-        if (hipGetLastError() != hipSuccess)
-          rc = fail(c, PLR_ERR_HIP, "upload: launching the tiling kernel failed");
-      }
-      if (rc == PLR_OK && hipEventRecord(done[k], c->stream) != hipSuccess)
-        rc = fail(c, PLR_ERR_HIP, "upload: host-to-device copy failed");
-    }
-    if (hipStreamSynchronize(c->stream) != hipSuccess && rc == PLR_OK)
-      rc = fail(c, PLR_ERR_HIP, "upload: stream synchronisation failed");
-    (void)hipGetLastError();
-    if (rc != PLR_OK) return rc;
-  }
-  PLR_HIP(c, hipMemcpy(c->dy + row0, y, (size_t)nrows * sizeof(double),
-                       hipMemcpyHostToDevice));
-  return PLR_OK;
+  const int rc = copy_rows_in(c, row0, nrows, X, ldx);
+  if (rc != PLR_OK) return rc;
+  return copy_bytes_in(c, {{c->dy + row0, y, (size_t)nrows * sizeof(double)}});
 }
 
 enum PassKind { kPassGrad, kPassDelta, kPassLoss, kPassPredict, kPassPredictLinear };
@@ -1410,67 +1320,194 @@ static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t coun
   return PLR_OK;
 }
 
-// The other direction, for bytes: pieces of pageable host memory into the device through
-// the same pinned lanes.  The pieces are cut into staging-block sized jobs dealt to the lanes
-// in turn; a lane's thread fills one of its two blocks while the other is in flight.
-static int copy_bytes_in(plr_ctx* c, const std::vector<CopyPiece>& pieces) {
-  size_t total = 0;
-  std::vector<CopyPiece> jobs;
-  for (const CopyPiece& p : pieces) {
-    total += p.bytes;
-    for (size_t at = 0; at < p.bytes; at += kCopyBlock)
-      jobs.push_back({static_cast<char*>(p.dev) + at, static_cast<const char*>(p.src) + at,
-                      std::min(kCopyBlock, p.bytes - at)});
-  }
-  if (total < 4 * kCopyBlock) {
-    for (const CopyPiece& p : pieces)
-      if (p.bytes) PLR_HIP(c, hipMemcpy(p.dev, p.src, p.bytes, hipMemcpyHostToDevice));
-    return PLR_OK;
-  }
+// The other direction: pageable host memory into the device through the same pinned lanes.
+// A job is at most one staging block; `fill` writes job j's bytes into the pinned block it
+// is handed (false stops every lane -- the caller has recorded why), the block is sent to
+// jobs[j].dev on the lane's stream, and `sent`, when given, queues more work behind that
+// transfer on the same stream.  Jobs are dealt to the lanes in turn; a lane's thread fills
+// one of its two blocks while the other is in flight.  Job j uses block (j % lanes) * 2 +
+// (j / lanes) % 2 of the staging area.
+struct InJob {
+  void* dev;
+  size_t bytes;
+};
+using FillFn = std::function<bool(size_t job, char* blk)>;
+using SentFn = std::function<hipError_t(size_t job, hipStream_t st)>;
+
+static int lanes_in(plr_ctx* c, const std::vector<InJob>& jobs, const FillFn& fill,
+                    const SentFn& sent, const char* what) {
+  if (jobs.empty()) return PLR_OK;
   if (!c->out_stage) {
     PLR_HIP(c, hipHostMalloc(&c->out_stage, 2 * kCopyLanes * kCopyBlock, hipHostMallocDefault));
     for (int l = 0; l < kCopyLanes; ++l)
       PLR_HIP(c, hipStreamCreateWithFlags(&c->out_stream[l], hipStreamNonBlocking));
   }
   hipError_t errs[kCopyLanes];
-  std::thread th[kCopyLanes];
-  for (int l = 0; l < kCopyLanes; ++l) {
+  std::atomic<bool> stop(false);
+  auto lane = [&](int l) {
     errs[l] = hipSuccess;
-    th[l] = std::thread([&, l]() {
-      if (hipSetDevice(c->device) != hipSuccess) {
-        errs[l] = hipErrorInvalidDevice;
-        return;
+    if (hipSetDevice(c->device) != hipSuccess) {
+      errs[l] = hipErrorInvalidDevice;
+      return;
+    }
+    char* stage = static_cast<char*>(c->out_stage) + (size_t)l * 2 * kCopyBlock;
+    hipStream_t st = c->out_stream[l];
+    hipEvent_t freed[2] = {nullptr, nullptr};
+    if (hipEventCreateWithFlags(&freed[0], hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&freed[1], hipEventDisableTiming) != hipSuccess)
+      errs[l] = hipErrorOutOfMemory;
+    int slot = 0;
+    size_t round = 0;
+    for (size_t j = l; j < jobs.size() && errs[l] == hipSuccess && !stop.load();
+         j += kCopyLanes, ++round, slot ^= 1) {
+      // the block sent from this slot two rounds ago must have left it
+      if (round >= 2 && hipEventSynchronize(freed[slot]) != hipSuccess) errs[l] = hipErrorUnknown;
+      char* blk = stage + (size_t)slot * kCopyBlock;
+      if (!fill(j, blk)) {
+        stop.store(true);
+        break;
       }
-      char* stage = static_cast<char*>(c->out_stage) + (size_t)l * 2 * kCopyBlock;
-      hipStream_t st = c->out_stream[l];
-      hipEvent_t freed[2] = {nullptr, nullptr};
-      if (hipEventCreateWithFlags(&freed[0], hipEventDisableTiming) != hipSuccess ||
-          hipEventCreateWithFlags(&freed[1], hipEventDisableTiming) != hipSuccess)
-        errs[l] = hipErrorOutOfMemory;
-      int slot = 0;
-      size_t round = 0;
-      for (size_t j = l; j < jobs.size() && errs[l] == hipSuccess; j += kCopyLanes, ++round, slot ^= 1) {
-        // the block sent from this slot two rounds ago must have left it
-        if (round >= 2 && hipEventSynchronize(freed[slot]) != hipSuccess) errs[l] = hipErrorUnknown;
-        char* blk = stage + (size_t)slot * kCopyBlock;
-        memcpy(blk, jobs[j].src, jobs[j].bytes);
-        hipError_t e = hipMemcpyAsync(jobs[j].dev, blk, jobs[j].bytes, hipMemcpyHostToDevice, st);
-        if (e == hipSuccess) e = hipEventRecord(freed[slot], st);
-        if (e != hipSuccess) errs[l] = e;
-      }
-      if (hipStreamSynchronize(st) != hipSuccess && errs[l] == hipSuccess) errs[l] = hipErrorUnknown;
-      for (int k = 0; k < 2; ++k)
-        if (freed[k]) (void)hipEventDestroy(freed[k]);
-    });
-  }
-  for (int l = 0; l < kCopyLanes; ++l) th[l].join();
+      hipError_t e = hipMemcpyAsync(jobs[j].dev, blk, jobs[j].bytes, hipMemcpyHostToDevice, st);
+      if (e == hipSuccess && sent) e = sent(j, st);
+      if (e == hipSuccess) e = hipEventRecord(freed[slot], st);
+      if (e != hipSuccess) errs[l] = e;
+    }
+    if (hipStreamSynchronize(st) != hipSuccess && errs[l] == hipSuccess) errs[l] = hipErrorUnknown;
+    for (int k = 0; k < 2; ++k)
+      if (freed[k]) (void)hipEventDestroy(freed[k]);
+  };
+  const int nl = (int)std::min<size_t>(kCopyLanes, jobs.size());
+  for (int l = nl; l < kCopyLanes; ++l) errs[l] = hipSuccess;
+  std::thread th[kCopyLanes];
+  for (int l = 1; l < nl; ++l) th[l] = std::thread(lane, l);
+  lane(0);
+  for (int l = 1; l < nl; ++l) th[l].join();
   for (int l = 0; l < kCopyLanes; ++l)
     if (errs[l] != hipSuccess) {
       (void)hipGetLastError();
-      return fail(c, PLR_ERR_HIP, std::string("copying the text to the device failed: ") +
-                                      hipGetErrorString(errs[l]));
+      return fail(c, PLR_ERR_HIP, std::string(what) + ": " + hipGetErrorString(errs[l]));
     }
   return PLR_OK;
+}
+
+// Bytes as they lie (the sample text, the labels, a shard at the device's own pitch).
+static int copy_bytes_in(plr_ctx* c, const std::vector<CopyPiece>& pieces) {
+  size_t total = 0;
+  std::vector<InJob> jobs;
+  std::vector<const char*> src;
+  for (const CopyPiece& p : pieces) {
+    total += p.bytes;
+    for (size_t at = 0; at < p.bytes; at += kCopyBlock) {
+      jobs.push_back({static_cast<char*>(p.dev) + at, std::min(kCopyBlock, p.bytes - at)});
+      src.push_back(static_cast<const char*>(p.src) + at);
+    }
+  }
+  if (total < 4 * kCopyBlock) {
+    for (const CopyPiece& p : pieces)
+      if (p.bytes) PLR_HIP(c, hipMemcpy(p.dev, p.src, p.bytes, hipMemcpyHostToDevice));
+    return PLR_OK;
+  }
+  return lanes_in(
+      c, jobs,
+      [&](size_t j, char* blk) {
+        memcpy(blk, src[j], jobs[j].bytes);
+        return true;
+      },
+      SentFn(), "copying to the device failed");
+}
+
+// Rows [row0, row0 + nrows) of the caller's row-major X (leading dimension ldx) into the
+// resident shard.  A strided copy command would move one row per transfer (~1 GB/s), so
+// the lanes' threads repack the rows at the pitch they have on the device -- without the
+// constant first column when that is not stored, pad columns zeroed -- into their pinned
+// blocks and send those as linear copies.  Row-tiled shards: a job's rows go, stored
+// columns only, into a block of a staging buffer on the device, and tile_rows, queued
+// behind the transfer on the lane's stream, brings them into the layout.  Rows wider
+// than a staging block are cut by columns.  With first_column_is_one the threads also
+// check the caller's statement; the first row that breaks it is named.
+static int copy_rows_in(plr_ctx* c, int64_t row0, int64_t nrows, const double* X, int64_t ldx) {
+  const bool tiled = c->lane != nullptr;
+  const int skip = c->bias ? 1 : 0;                 // the constant first column stays on the host
+  const int64_t sp = tiled ? c->dcols : c->pitch;   // pitch of the rows as they are sent
+  const int64_t blk_cols = (int64_t)(kCopyBlock / sizeof(double));
+  if (!tiled && !c->bias && ldx == sp && c->dcols == sp)  // as they lie: one linear stretch
+    return copy_bytes_in(c, {{c->dX + row0 * sp, X, (size_t)nrows * sp * sizeof(double)}});
+  if (tiled && !c->up_dev) {
+    if (hipMalloc(&c->up_dev, 2 * kCopyLanes * kCopyBlock) != hipSuccess) {
+      (void)hipGetLastError();
+      c->up_dev = nullptr;
+      return fail(c, PLR_ERR_NOMEM, "cannot allocate the device upload staging buffer");
+    }
+  }
+  struct RowJob {
+    int64_t r0, m;   // rows [r0, r0 + m) of this upload ...
+    int64_t c0, w;   // ... columns [c0, c0 + w) of the sent row (whole rows unless m == 1)
+  };
+  std::vector<RowJob> rj;
+  std::vector<InJob> jobs;
+  if (sp <= blk_cols) {
+    const int64_t per = blk_cols / sp;
+    for (int64_t r0 = 0; r0 < nrows; r0 += per) rj.push_back({r0, std::min(per, nrows - r0), 0, sp});
+  } else {
+    for (int64_t r = 0; r < nrows; ++r)
+      for (int64_t c0 = 0; c0 < sp; c0 += blk_cols) rj.push_back({r, 1, c0, std::min(blk_cols, sp - c0)});
+  }
+  jobs.reserve(rj.size());
+  for (size_t j = 0; j < rj.size(); ++j) {
+    double* dev = tiled ? c->up_dev + ((j % kCopyLanes) * 2 + (j / kCopyLanes) % 2) * (size_t)blk_cols
+                        : c->dX + (row0 + rj[j].r0) * c->pitch + rj[j].c0;
+    jobs.push_back({dev, (size_t)(rj[j].m * rj[j].w) * sizeof(double)});
+  }
+  std::atomic<int64_t> bad_row(INT64_MAX);
+  const int64_t dcols = c->dcols;
+  const bool dense = (skip == 0 && ldx == sp && dcols == sp);  // tiled rows that are already packed
+  auto fill = [&](size_t j, char* blk) {
+    const RowJob& q = rj[j];
+    double* dst = reinterpret_cast<double*>(blk);
+    if (dense) {
+      memcpy(dst, X + q.r0 * ldx, (size_t)(q.m * sp) * sizeof(double));
+      return true;
+    }
+    for (int64_t r = 0; r < q.m; ++r, dst += q.w) {
+      const double* row = X + (q.r0 + r) * ldx;
+      if (skip && q.c0 == 0 && row[0] != 1.) {
+        int64_t seen = bad_row.load();
+        while (q.r0 + r < seen && !bad_row.compare_exchange_weak(seen, q.r0 + r)) {
+        }
+        return false;
+      }
+      const int64_t have = std::max<int64_t>(0, std::min(q.w, dcols - q.c0));  // the rest is padding
+      if (have) memcpy(dst, row + skip + q.c0, (size_t)have * sizeof(double));
+      for (int64_t k = have; k < q.w; ++k) dst[k] = 0.;
+    }
+    return true;
+  };
+  SentFn sent;
+  if (tiled) {
+    const int np = c->lane->np;
+    sent = [&, np](size_t j, hipStream_t st) {
+      const int64_t threads = ceil_div(rj[j].m, plr::kWave) * plr::kWave * np;
+      hipLaunchKernelGGL(plr::tile_rows, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st,
+                         (const double*)jobs[j].dev, sp, rj[j].m, (int)dcols, c->dX,
+                         row0 + rj[j].r0, np);
+      return hipGetLastError();
+    };
+  }
+  const int rc = lanes_in(c, jobs, fill, sent, "upload: host-to-device copy failed");
+  if (bad_row.load() != INT64_MAX) {
+    // lanes run ahead of each other: an earlier row may break the statement too
+    int64_t first = bad_row.load();
+    for (int64_t r = 0; r < first; ++r)
+      if (X[r * ldx] != 1.) {
+        first = r;
+        break;
+      }
+    char b[160];
+    snprintf(b, sizeof b, "first_column_is_one is set, but row %lld starts with %.17g",
+             (long long)(row0 + first), X[first * ldx]);
+    return fail(c, PLR_ERR_INVALID, b);
+  }
+  return rc;
 }
 
 static int predict_rows(plr_ctx* c, PassKind kind, const double* theta, double* out) {

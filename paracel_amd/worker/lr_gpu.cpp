@@ -67,10 +67,14 @@ void logistic_regression_gpu::load_and_parse(const std::string& fn) {
   labels.swap(s.y);
 }
 
-// paracel_load + local_parser on the device (device_load.hpp)
+// the fresh binary cache sent from its mapping, else paracel_load + local_parser
+// on the device (device_load.hpp)
 bool logistic_regression_gpu::load_on_device(const std::string& fn) {
   int64_t n = 0, d = 0;
-  if (!load_shard_on_device(gpu, fn, (int)get_worker_id(), (int)get_worker_size(), n, d))
+  const int rank = (int)get_worker_id(), np = (int)get_worker_size();
+  // the cache's rows start with the bias 1.0 (lr.cpp:83): not kept in HBM
+  check(plr_set_option(gpu, "first_column_is_one", 1), "plr_set_option");
+  if (!upload_cached_shard(gpu, fn, rank, np, n, d) && !load_shard_on_device(gpu, fn, rank, np, n, d))
     return false;
   n_local = n;
   data_dim = d;

@@ -43,7 +43,8 @@ void ridge_regression_gpu::load_and_upload(const std::string& fn) {
   const int rank = (int)get_worker_id(), np = (int)get_worker_size();
   {
     int64_t n = 0, d = 0;
-    if (load_shard_on_device(gpu, fn, rank, np, n, d)) {  // parsed in HBM (device_load.hpp)
+    // the fresh cache from its mapping, else parsed in HBM (device_load.hpp)
+    if (upload_cached_shard(gpu, fn, rank, np, n, d) || load_shard_on_device(gpu, fn, rank, np, n, d)) {
       n_local = n;
       data_dim = d;
       if (kdim == 0 && data_dim > 0) kdim = (int)data_dim - 1;

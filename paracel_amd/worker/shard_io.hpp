@@ -30,6 +30,8 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <stdexcept>
 #include <memory>
@@ -435,6 +437,101 @@ inline bool open_cache(const std::string& input, int rank, int np, ShardCacheHea
     fclose(f);
     f = nullptr;
   }
+  return ok;
+}
+
+// A fresh cache mapped read-only: the rows go to the device straight from the
+// page cache, without a copy of the shard in the process.
+struct MappedShard {
+  void* base = nullptr;
+  size_t bytes = 0;
+  int64_t n = 0, d = 0;
+  MappedShard() {}
+  MappedShard(const MappedShard&) = delete;
+  MappedShard& operator=(const MappedShard&) = delete;
+  ~MappedShard() {
+    if (base) munmap(base, bytes);
+  }
+  const double* X() const {
+    return reinterpret_cast<const double*>(static_cast<const char*>(base) + sizeof(ShardCacheHeader));
+  }
+  const double* y() const { return X() + (size_t)n * d; }
+};
+
+inline bool map_cache(const std::string& input, int rank, int np, MappedShard& m) {
+  ShardCacheHeader h;
+  FILE* f = nullptr;
+  if (!open_cache(input, rank, np, h, f)) return false;
+  struct stat st;
+  const size_t want = sizeof h + ((size_t)h.n * h.d + (size_t)h.n) * sizeof(double);
+  bool ok = fstat(fileno(f), &st) == 0 && (size_t)st.st_size == want;
+  if (ok) {
+    void* p = mmap(nullptr, want, PROT_READ, MAP_PRIVATE, fileno(f), 0);
+    ok = p != MAP_FAILED;
+    if (ok) {
+      m.base = p;
+      m.bytes = want;
+      m.n = h.n;
+      m.d = h.d;
+    }
+  }
+  fclose(f);
+  return ok;
+}
+
+// The cache written slab by slab from rows that live elsewhere (the device):
+// rows(r0, m, X, y) fills rows [r0, r0 + m) into X (m x d, dense) and y; false
+// aborts.  The shard never exists whole in this process.
+template <class Rows>
+inline bool write_cache_rows(const std::string& input, int rank, int np, int64_t n, int64_t d,
+                             Rows rows, size_t slab_bytes = 64u << 20) {
+  ShardCacheHeader h;
+  memset(&h, 0, sizeof h);
+  memcpy(h.magic, "PLRSHARD", 8);
+  h.version = 1;
+  h.n = n;
+  h.d = d;
+  if (!source_stamp(input, h.src_size, h.src_mtime_ns)) return false;
+  const std::string path = cache_path(input, rank, np), tmp = path + ".tmp";
+  const int fd = open(tmp.c_str(), O_WRONLY | O_CREAT | O_TRUNC, 0644);
+  if (fd < 0) return false;  // read-only input directory: run without a cache
+  auto put = [fd](const void* p, size_t bytes, size_t at) {
+    for (size_t lo = 0; lo < bytes;) {
+      const ssize_t w = pwrite(fd, static_cast<const char*>(p) + lo, bytes - lo, (off_t)(at + lo));
+      if (w <= 0) return false;
+      lo += (size_t)w;
+    }
+    return true;
+  };
+  bool ok = put(&h, sizeof h, 0);
+  size_t at = sizeof h;
+  const int64_t slab = std::max<int64_t>(1, (int64_t)slab_bytes / (d * (int64_t)sizeof(double)));
+  // two slab buffers: one is written to the file (a copy into the page cache,
+  // ~10 GB/s, more threads do not help) while the next is fetched
+  std::vector<double> X[2], y((size_t)n);
+  for (auto& x : X) x.resize((size_t)std::min(slab, std::max<int64_t>(n, 1)) * d);
+  std::thread writer;
+  std::atomic<bool> wrote(true);
+  int k = 0;
+  for (int64_t r0 = 0; r0 < n && ok; r0 += slab, k ^= 1) {
+    const int64_t m = std::min(slab, n - r0);
+    const size_t bytes = (size_t)m * d * sizeof(double);
+    ok = rows(r0, m, X[k].data(), y.data() + r0);
+    if (writer.joinable()) writer.join();  // the other buffer is free again
+    ok = ok && wrote.load();
+    if (ok) {
+      const double* src = X[k].data();
+      writer = std::thread([&put, &wrote, src, bytes, at]() {
+        if (!put(src, bytes, at)) wrote = false;
+      });
+    }
+    at += bytes;
+  }
+  if (writer.joinable()) writer.join();
+  ok = ok && wrote.load() && put(y.data(), (size_t)n * sizeof(double), at);
+  ok = (close(fd) == 0) && ok;
+  if (ok) ok = rename(tmp.c_str(), path.c_str()) == 0;
+  if (!ok) remove(tmp.c_str());
   return ok;
 }
 

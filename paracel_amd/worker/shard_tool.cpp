@@ -84,6 +84,28 @@ int main(int argc, char** argv) {
     }
     return 0;
   }
+  if (argc == 6 && std::string(argv[1]) == "recache") {
+    // the fresh cache read through its mapping and written again slab by slab
+    // (slabs of argv[5] bytes): the two routes the GPU workers take
+    const int rank = atoi(argv[3]), np = atoi(argv[4]);
+    plr_ps::MappedShard m;
+    if (!plr_ps::map_cache(argv[2], rank, np, m)) {
+      std::cout << "stale-or-missing\n";
+      return 1;
+    }
+    const int64_t n = m.n, d = m.d;
+    std::vector<double> X(m.X(), m.X() + (size_t)n * d), y(m.y(), m.y() + n);
+    const bool ok = plr_ps::write_cache_rows(
+        argv[2], rank, np, n, d,
+        [&](int64_t r0, int64_t rows, double* Xo, double* yo) {
+          memcpy(Xo, X.data() + (size_t)r0 * d, (size_t)rows * d * sizeof(double));
+          memcpy(yo, y.data() + r0, (size_t)rows * sizeof(double));
+          return true;
+        },
+        (size_t)atoll(argv[5]));
+    std::cout << (ok ? "rewritten " : "failed ") << n << " " << d << "\n";
+    return ok ? 0 : 1;
+  }
   if (argc != 5) {
     std::cerr << "usage: plr_shard_tool parse|info|lines <input> <rank> <np>\n";
     return 2;

@@ -165,8 +165,14 @@ def test_parser_matches_oracle_and_cache_roundtrip(tmp_path, oracle):
     np.testing.assert_array_equal(y, yo)
     assert np.all(X[:, 0] == 1.0)
     assert run("info", f, 0, 1).stdout.split() == ["300", "8"]
+    # the mapped read and the slab-by-slab writer (the GPU workers' routes) keep every byte
+    for slab in (64, 1000, 1 << 26):
+        out = run("recache", f, 0, 1, slab)
+        assert out.returncode == 0 and out.stdout.split() == ["rewritten", "300", "8"], out.stderr
+        assert np.array_equal(np.fromfile(str(f) + ".plrshard.0of1", dtype=np.uint8), raw)
     # touching the source invalidates the cache
     os.utime(f, ns=(1, 1))
+    assert run("recache", f, 0, 1, 4096).returncode == 1
     assert run("info", f, 0, 1).returncode == 1
     # per-rank shards concatenate to the whole
     parts = []
@@ -176,6 +182,19 @@ def test_parser_matches_oracle_and_cache_roundtrip(tmp_path, oracle):
         nn, dd = np.frombuffer(rr[16:32].tobytes(), dtype=np.int64)
         parts.append(np.frombuffer(rr[48:48 + 8 * nn * dd].tobytes(), dtype=np.float64).reshape(nn, dd))
     np.testing.assert_array_equal(np.vstack(parts), Xo)
+
+
+def test_cache_written_in_slabs_while_the_next_is_fetched(tmp_path):
+    # a few slabs and one: the writer thread and the fetch alternate between two buffers
+    f = tmp_path / "big.csv"
+    make_csv(f, 40000, 7, 5, ragged_len=False)
+    assert run("parse", f, 0, 1).stdout.split() == ["40000", "8"]
+    raw = np.fromfile(str(f) + ".plrshard.0of1", dtype=np.uint8)
+    assert raw.size == 48 + 40000 * 9 * 8
+    for slab in (1 << 18, 1 << 20, 1 << 26):
+        out = run("recache", f, 0, 1, slab)
+        assert out.returncode == 0, out.stderr
+        assert np.array_equal(np.fromfile(str(f) + ".plrshard.0of1", dtype=np.uint8), raw)
 
 
 def test_parser_errors(tmp_path):
