@@ -1140,7 +1140,10 @@ enum : int {
 
 template <int NCH, bool GRAD, int LM>
 __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
-  constexpr int D = 3;  // row buffers: rows t - 1, t and t + 1
+  // Row buffers: rows t - 1, t and t + 1.  (A fourth, row t + 2 in flight as well, was
+  // measured at 6 chunks per wave, where it nearly fits the registers: slower at every
+  // width -- the step is not waiting for data any more once the waits below are right.)
+  constexpr int D = 3;
   constexpr unsigned kLoss = LM == kTeamLmReference ? kLossReference
                              : LM == kTeamLmStable  ? kLossStable
                              : LM == kTeamLmSquared ? kLossSquared
@@ -1195,7 +1198,13 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
   const int64_t myrows = a.n > team ? (a.n - team + a.nteams - 1) / a.nteams : 0;
 
   v2d X[D][NCH];
-  auto request = [&](int64_t i, v2d (&buf)[NCH]) {  // row i of this team -> buf
+  // Row i of this team -> buf.  Past the team's last row the last row is asked
+  // for again (and never used): every step then issues the same loads, with no
+  // branch around them, so the wait for row t counts exactly the loads issued
+  // after it -- behind a conditional request the compiler has to wait for
+  // everything outstanding, the row just requested included.
+  auto request = [&](int64_t i, v2d (&buf)[NCH]) {
+    if (i >= myrows) i = myrows - 1;
     const char* rp = xwave + (team + i * a.nteams) * row_bytes;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
@@ -1226,8 +1235,13 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
       w0 = __hip_atomic_load(pslot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       w1 = __hip_atomic_load(pslot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    // the label of row t - 1, for the same reason ahead of the row request: asked
+    // for where it is used, it would come back behind row t + 1 and the update
+    // of row t - 1 would wait for that whole row
+    const int64_t prev_row = team + (have_prev ? t - 1 : 0) * a.nteams;
+    const double yv = *(a.y ? a.y + prev_row : a.zeros);
     asm volatile("" ::: "memory");
-    if (t + 1 < myrows) request(t + 1, X[NEXT]);
+    request(t + 1, X[NEXT]);
     asm volatile("" ::: "memory");
 
     if (have_row) {
@@ -1275,8 +1289,7 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
     }
     __syncthreads();
     if (have_prev) {
-      const int64_t row = team + (t - 1) * a.nteams;
-      const double yv = a.y ? a.y[row] : 0.;
+      const int64_t row = prev_row;
       double z = bias;
       for (int b = 0; b < a.nblk; ++b) z += zp[par][b];
       double h, l;
