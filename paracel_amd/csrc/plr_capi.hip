@@ -112,18 +112,18 @@ struct LaneVariant {
 // columns up; 4 columns 5.9, 2 columns 4.2: one exp/log per 16-32 bytes).
 // From 30 columns on a wave pair per tile is faster than a wave (+1-7 %).
 const LaneVariant kLane[] = {
-    PLR_LANE(1, 2, 2, 3),  // 2 columns
-    PLR_LANE(2, 2, 4, 3),
-    PLR_LANE(3, 4, 4, 1),
-    PLR_LANE(4, 1, 4, 3),
-    PLR_LANE(5, 2, 2, 3),
-    PLR_LANE(6, 2, 4, 3),
-    PLR_LANE(7, 1, 4, 4),
+    PLR_LANE(1, 4, 4, 1),  // 2 columns
+    PLR_LANE(2, 1, 8, 1),
+    PLR_LANE(3, 2, 4, 2),
+    PLR_LANE(4, 1, 8, 1),
+    PLR_LANE(5, 1, 4, 1),
+    PLR_LANE(6, 1, 4, 1),
+    PLR_LANE(7, 1, 4, 1),
     PLR_LANE(8, 1, 4, 2),  // 16 columns
-    PLR_LANE(9, 1, 4, 2),
+    PLR_LANE(9, 1, 4, 1),
     PLR_LANE(10, 1, 4, 2),
-    PLR_LANE(11, 1, 4, 3),
-    PLR_LANE(12, 1, 4, 3),
+    PLR_LANE(11, 1, 4, 1),
+    PLR_LANE(12, 1, 4, 1),
     PLR_LANE(13, 1, 4, 2),
     PLR_LANE(14, 1, 4, 1),
     PLR_LANE2(15, 2, 2),  // 30 columns

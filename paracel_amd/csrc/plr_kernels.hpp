@@ -655,41 +655,33 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void lane_pass(PassArgs a) {
 #pragma unroll
   for (int p = 0; p < NP; ++p) acc[p] = v2d{0., 0.};
   RowSums sums;
-  // a group's predictions are stored after the next group's loads have been
-  // issued (a store in front of them would have to be acknowledged first)
-  double h_keep[U];
-  int64_t h_row0 = -1;
-#pragma unroll
-  for (int u = 0; u < U; ++u) h_keep[u] = 0.;
-  auto store_kept = [&]() {
-    if (a.h_out && h_row0 >= 0) {
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int64_t row = h_row0 + u * kWave;
-        if (row < a.n) store_h(a.h_out + row, h_keep[u]);
-      }
-    }
-  };
 
   constexpr int64_t kGroupRows = (int64_t)kWave * U;
   const int64_t ngroups = (a.n + kGroupRows - 1) / kGroupRows;
   const int64_t stride = (int64_t)gridDim.x * WROW;
-#pragma clang loop unroll(disable)
-  for (int64_t g = (int64_t)blockIdx.x * WROW + wr; g < ngroups; g += stride) {
+  // Software pipeline: the loads of a wave's NEXT group are in flight while it
+  // works on this one (two register buffers, the loop unrolled by two).  Every
+  // load is unconditional -- past the last group the last group is asked for
+  // again and dropped, a row past the end reads the last label -- so the wait
+  // for a buffer counts exactly the loads issued after it.  Without labels
+  // (predict) the first theta entry stands in for the address.
+  const double* ybase = a.y ? a.y : a.theta;
+  auto request = [&](int64_t g, v2d (&x)[U][NP], double (&yv)[U]) {
+    if (g >= ngroups) g = ngroups - 1;
     const v2d* base = reinterpret_cast<const v2d*>(a.X) + g * (U * NP * kWave) + lane;
-    v2d x[U][NP];
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int p = 0; p < NP; ++p) x[u][p] = load_x(base + (u * NP + p) * kWave);
-    const int64_t row0 = g * kGroupRows + lane;
-    double yv[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t row = row0 + u * kWave;
-      yv[u] = (a.y && row < a.n) ? a.y[row] : 0.;
+      int64_t row = g * kGroupRows + lane + u * kWave;
+      if (row >= a.n) row = a.n - 1;
+      yv[u] = ybase[a.y ? row : 0];
     }
-    store_kept();
+  };
+  auto work = [&](int64_t g, v2d (&x)[U][NP], double (&yl)[U]) {
+    const int64_t row0 = g * kGroupRows + lane;
     // keeps the theta reads inside the loop: hoisted, they would occupy
     // 4 * NP registers next to x and acc
     asm volatile("" ::: "memory");
@@ -703,25 +695,43 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void lane_pass(PassArgs a) {
         z = fma(x[u][p].y, th.y, z);
       }
       const bool valid = row0 + u * kWave < a.n;
+      const double yv = a.y ? yl[u] : 0.;
       double h, l;
-      row_terms(z + bias, yv[u], a.loss_mode, a.identity_link, h, l);
-      const double res = valid ? (h - yv[u]) : 0.;
-      h_keep[u] = h;
+      row_terms(z + bias, yv, a.loss_mode, a.identity_link, h, l);
+      const double res = valid ? (h - yv) : 0.;
       if (valid) {
         sums.loss += l;
         sums.res += res;
       }
-      if (GRAD) {
+      if constexpr (GRAD) {
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
           acc[p].x = fma(res, x[u][p].x, acc[p].x);
           acc[p].y = fma(res, x[u][p].y, acc[p].y);
         }
+      } else {
+        // predictions go with the passes that carry no gradient
+        if (a.h_out && valid) store_h(a.h_out + row0 + u * kWave, h);
       }
     }
-    h_row0 = row0;
+  };
+  int64_t g = (int64_t)blockIdx.x * WROW + wr;
+  if (g < ngroups) {
+    v2d xa[U][NP], xb[U][NP];
+    double ya[U], yb[U];
+    request(g, xa, ya);
+#pragma clang loop unroll(disable)
+    for (;;) {
+      request(g + stride, xb, yb);
+      work(g, xa, ya);
+      g += stride;
+      if (g >= ngroups) break;
+      request(g + stride, xa, ya);
+      work(g, xb, yb);
+      g += stride;
+      if (g >= ngroups) break;
+    }
   }
-  store_kept();
 
   if (GRAD) {
     __shared__ v2d gx[(WROW > 1) ? (WROW - 1) * NP : 1];
