@@ -81,7 +81,7 @@ MEASURED_TRAFFIC = {
         "profiles/shard_pass_x_bias_1m_x_2049.md"),
     "x_narrow_30m_x_16": (
         30000000, "lane_pass<NP=8,U=1,WROW=4> row-tiled layout, pitch=16, 64 rows per "
-        "group, grid=768 x 256 threads (occupancy 3 blocks/CU, 256 CUs)", 4080193979,
+        "group, grid=512 x 256 threads (occupancy 2 blocks/CU, 256 CUs)", 4080839161,
         "profiles/lane_pass_x_narrow_30m_x_16.md"),
     "x_narrow_10m_x_41": (
         10000000, "lane2_pass<NP=21,U=2,WROW=1> row-tiled layout, pitch=42, 128 rows per "
