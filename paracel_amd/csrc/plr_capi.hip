@@ -240,7 +240,7 @@ struct plr_ctx {
   double* h_pred = nullptr;     // n, pinned + device-mapped: where wide shards put predictions
   double* h_pred_dev = nullptr;
   void* out_stage = nullptr;    // pinned staging of copy_rows_out, lazily allocated
-  hipStream_t out_stream[4] = {nullptr, nullptr, nullptr, nullptr};
+  hipStream_t out_stream[8] = {};  // one per copy lane (kCopyLanes)
   double* d_curve = nullptr;    // per-round losses of plr_train_dgd, lazily allocated
   double* d_train_out = nullptr;  // d + 1: where training rounds put delta (never read back)
   int curve_len = 0;
@@ -1239,7 +1239,7 @@ int plr_calc_loss(plr_ctx* c, const double* theta, double* loss_sum, int64_t* n_
 // through kCopyLanes independent lanes, each with two pinned staging blocks on
 // a stream of its own: the DMA into one block overlaps the host copy out of
 // the other, and the lanes overlap each other.
-constexpr int kCopyLanes = 4;
+constexpr int kCopyLanes = 8;
 constexpr size_t kCopyBlock = 4u << 20;
 
 // pinned host memory -> the caller's buffer, kCopyLanes threads
