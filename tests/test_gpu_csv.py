@@ -215,7 +215,8 @@ def test_errors_are_the_reference_parsers(plr):
 
 def test_get_data_returns_what_set_data_took(plr):
     rng = np.random.default_rng(3)
-    for n, d in [(100, 7), (130, 64), (77, 66), (50, 300), (10, 20001)]:
+    # (the last shape: a row longer than one 4 MiB block of the upload lanes, cut by columns)
+    for n, d in [(100, 7), (130, 64), (77, 66), (50, 300), (10, 20001), (3, 530001)]:
         X = rng.normal(size=(n, d))
         y = rng.integers(0, 2, size=n).astype(float)
         plr.set_data(X, y)
