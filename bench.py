@@ -68,8 +68,8 @@ MEASURED_TRAFFIC = {
         "threads (occupancy 2 blocks/CU, 256 CUs)", 17582792859,
         "profiles/pair_pass_x_short_30m_x_72.md"),
     "x_c1shape_20m_x_100": (
-        20000000, "shard_pass<NCH=1,R=16,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=1 tail=0 "
-        "pitch=100 grid=512 x 256 threads (occupancy 2 blocks/CU, 256 CUs)", 16453025582,
+        20000000, "shard_pass<NCH=1,R=32,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=1 tail=0 "
+        "pitch=100 grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)", 16355842464,
         "profiles/shard_pass_x_c1shape_20m_x_100.md"),
     "x_bias_10m_x_257": (
         10000000, "shard_pass<NCH=2,R=32,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=2 tail=0 "

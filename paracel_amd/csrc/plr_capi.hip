@@ -329,7 +329,7 @@ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // n x d shard.
 int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   plr_plan::Plan pl;
-  if (!plr_plan::plan_width(d, pl))
+  if (!plr_plan::plan_width(d, pl, n))
     return fail(c, PLR_ERR_UNSUPPORTED, "no kernel variant covers this width");
   c->pitch = pl.pitch;
   c->theta_len = pl.theta_len;
@@ -1704,7 +1704,7 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
   // the row pitch is a whole number of chunks, so the variant is the exact
   // one-wave one for ldx / 128 chunks and no lane reads past a row end
   plr_plan::Plan pl;
-  if (!plr_plan::plan_width(ldx, pl) || pl.path != plr_plan::kPathFused || pl.pitch != ldx ||
+  if (!plr_plan::plan_width(ldx, pl, n) || pl.path != plr_plan::kPathFused || pl.pitch != ldx ||
       !pl.allch || pl.tail_cols != 0 || pl.theta_len > kNaMaxPitch)
     return bad(PLR_ERR_UNSUPPORTED, "no kernel variant covers this pitch");
   const Shape* v = &kShapes[pl.variant];

@@ -57,7 +57,11 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Fills p for a shard of d >= 1 columns; false if no variant covers the width
 // (cannot happen with the table as it is; checked by the host-side test).
-inline bool plan_width(int64_t d, Plan& p) {
+// n: rows of the shard when known (< 0: unknown, taken as large).  Where the
+// variant table has two entries for a shape, shards below kSmallShardBytes
+// take the one with the shorter tiles.
+constexpr int64_t kSmallShardBytes = 1500000000;
+inline bool plan_width(int64_t d, Plan& p, int64_t n = -1) {
   p = Plan();
   p.variant = -1;
   if (d <= kMaxLaneCols) {
@@ -134,10 +138,9 @@ inline bool plan_width(int64_t d, Plan& p) {
       const bool fits = (want_k >= 8 && want_w == 8)
                             ? (k.thl && k.wcol == 8 && k.nch >= want_k)
                             : (!k.thl && k.wcol == want_w && k.nch == want_k);
-      if (fits) {
-        v = i;
-        break;
-      }
+      if (!fits) continue;
+      const bool small = n >= 0 && n * pitch * (int64_t)sizeof(double) < kSmallShardBytes;
+      if (v < 0 || (small && k.R < kShapes[v].R)) v = i;
     }
   }
   if (v < 0) return false;

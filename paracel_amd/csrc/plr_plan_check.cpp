@@ -19,9 +19,9 @@ static int failures = 0;
     }                                                                         \
   } while (0)
 
-static void print_plan(int64_t d) {
+static void print_plan(int64_t d, int64_t n) {
   Plan p;
-  if (!plan_width(d, p)) {
+  if (!plan_width(d, p, n)) {
     printf("d=%lld: no variant\n", (long long)d);
     return;
   }
@@ -39,15 +39,18 @@ static void print_plan(int64_t d) {
 }
 
 int main(int argc, char** argv) {
-  if (argc > 1) {
-    print_plan(atoll(argv[1]));
+  if (argc > 1) {  // plr_plan_check <d> [<n>]
+    print_plan(atoll(argv[1]), argc > 2 ? atoll(argv[2]) : -1);
     return 0;
   }
   std::vector<int64_t> used(kNumShapes, 0);
   const int64_t kMaxD = 140000;
-  for (int64_t d = 1; d <= kMaxD; ++d) {
+  // every width twice: rows unknown (a large shard) and a one-row shard (the
+  // short-tile entries of the table)
+  for (int64_t dn = 2; dn <= 2 * kMaxD + 1; ++dn) {
+    const int64_t d = dn / 2, n = (dn & 1) ? 1 : -1;
     Plan p;
-    if (!plan_width(d, p)) {
+    if (!plan_width(d, p, n)) {
       CHECK(false && "plan_width failed", d);
       continue;
     }

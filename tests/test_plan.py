@@ -17,8 +17,9 @@ def _tool():
                         os.path.join(ROOT, "paracel_amd", "csrc", "plr_plan_check.cpp")], check=True)
 
 
-def plan(d):
-    out = subprocess.run([TOOL, str(d)], capture_output=True, text=True, check=True).stdout
+def plan(d, n=None):
+    args = [TOOL, str(d)] + ([str(n)] if n is not None else [])
+    out = subprocess.run(args, capture_output=True, text=True, check=True).stdout
     return dict(kv.split("=") for kv in out.split()[0:] if "=" in kv)
 
 
@@ -29,8 +30,12 @@ def test_every_width_satisfies_the_kernels_assumptions():
 
 
 def test_the_benchmark_shapes_take_the_intended_variants():
-    p = plan(100)        # config 1: one chunk, 16 rows per tile
+    p = plan(100, 100000)   # config 1 (80 MB): one chunk, 16 rows per tile
     assert (p["path"], p["NCH"], p["R"], p["WCOL"], p["tail"]) == ("fused", "1", "16", "1", "0")
+    p = plan(100, 20000000)  # its shape at 16 GB, and when the rows are not known: 32 rows per tile
+    assert (p["path"], p["NCH"], p["R"], p["WCOL"], p["tail"]) == ("fused", "1", "32", "1", "0")
+    assert plan(100)["R"] == "32" and plan(128, 1000000)["R"] == "16" and plan(128, 1500000)["R"] == "32"
+    assert plan(1000, 1000)["R"] == plan(1000, 1000000)["R"] == "4"   # one entry: no choice
     p = plan(1000)       # config 2: one wave, 8 chunks
     assert (p["NCH"], p["R"], p["WCOL"], p["allch"], p["pitch"]) == ("8", "4", "1", "1", "1000")
     p = plan(256)        # config 3
