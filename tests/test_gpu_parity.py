@@ -257,6 +257,7 @@ def test_constant_first_column_is_not_stored(plr, oracle, gen, n, d):
     # a row that does not start with 1.0 is refused, by row number
     Xb = X.copy()
     Xb[n // 3, 0] = 1.0000001
+    Xb[n - 1, 0] = 0.0      # a later one too (another upload thread may meet it first)
     with pytest.raises(PlrError) as e:
         plr.set_data(Xb, y)
     assert e.value.code == -1 and "row %d" % (n // 3) in str(e.value)
