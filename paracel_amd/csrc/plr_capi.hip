@@ -1241,6 +1241,8 @@ int plr_calc_loss(plr_ctx* c, const double* theta, double* loss_sum, int64_t* n_
 // the other, and the lanes overlap each other.
 constexpr int kCopyLanes = 8;
 constexpr size_t kCopyBlock = 4u << 20;
+static_assert(sizeof(plr_ctx::out_stream) / sizeof(hipStream_t) == kCopyLanes,
+              "one stream per copy lane");
 
 // pinned host memory -> the caller's buffer, kCopyLanes threads
 static void copy_host_parallel(double* out, const double* src, size_t count) {
