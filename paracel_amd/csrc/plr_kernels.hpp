@@ -1151,8 +1151,9 @@ enum : int {
 template <int NCH, bool GRAD, int LM>
 __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
   // Row buffers: rows t - 1, t and t + 1.  (A fourth, row t + 2 in flight as well, was
-  // measured at 6 chunks per wave, where it nearly fits the registers: slower at every
-  // width -- the step is not waiting for data any more once the waits below are right.)
+  // measured at 6 chunks per wave, where the loss-free instance fits the registers
+  // without a spill: 0.5-1 % slower at every width -- the step is not waiting for
+  // data any more once the waits below are right.)
   constexpr int D = 3;
   constexpr unsigned kLoss = LM == kTeamLmReference ? kLossReference
                              : LM == kTeamLmStable  ? kLossStable
