@@ -1317,7 +1317,7 @@ static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t coun
     if (errs[l] != hipSuccess) {
       (void)hipGetLastError();
       return fail(c, PLR_ERR_HIP,
-                  std::string("copying the predictions out failed: ") + hipGetErrorString(errs[l]));
+                  std::string("copying results to the host failed: ") + hipGetErrorString(errs[l]));
     }
   return PLR_OK;
 }
