@@ -43,7 +43,11 @@ def stream_and_reference(plr, cfg, theta, slab_rows=0):
 
 
 FULL = ["c2_headline_1m_x_1000", "c3_tall_10m_x_256", "c4_wide_200k_x_16384",
-        "c4b_wide_200k_x_16385", "c5_e2e_2m_x_512", "x_bias_10m_x_257"]
+        "c4b_wide_200k_x_16385", "c5_e2e_2m_x_512", "x_bias_10m_x_257",
+        # the shapes of the other kernel families, at the sizes bench.py times them:
+        # lane_pass, lane2_pass, pair_pass, the one-chunk shard_pass, team_pass
+        "x_narrow_30m_x_16", "x_narrow_10m_x_41", "x_short_30m_x_66", "x_c1shape_20m_x_100",
+        "x_verywide_100k_x_32768"]
 
 
 @pytest.mark.parametrize("name", FULL)
