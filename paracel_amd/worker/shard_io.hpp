@@ -516,7 +516,14 @@ inline bool write_cache_rows(const std::string& input, int rank, int np, int64_t
   for (int64_t r0 = 0; r0 < n && ok; r0 += slab, k ^= 1) {
     const int64_t m = std::min(slab, n - r0);
     const size_t bytes = (size_t)m * d * sizeof(double);
-    ok = rows(r0, m, X[k].data(), y.data() + r0);
+    try {
+      ok = rows(r0, m, X[k].data(), y.data() + r0);
+    } catch (...) {  // the writer still holds the other buffer and the file
+      if (writer.joinable()) writer.join();
+      close(fd);
+      remove(tmp.c_str());
+      throw;
+    }
     if (writer.joinable()) writer.join();  // the other buffer is free again
     ok = ok && wrote.load();
     if (ok) {
