@@ -201,7 +201,7 @@ void logistic_regression_gpu::predict(const std::string& pred_fn) {
       const size_t en = line.find(',', st);
       const std::string tok = line.substr(st, en == std::string::npos ? en : en - st);
       if (!tok.empty()) {
-        flat.push_back(std::stod(tok));
+        flat.push_back(parse_field(tok.data(), tok.size()));  // std::stod's value and errors
         ++got;
       }
       if (en == std::string::npos) break;
