@@ -1115,7 +1115,7 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
 constexpr int kXcds = 8;        // workgroups are dealt to the XCDs round-robin
 constexpr int kTeamWaves = 8;
 constexpr int kTeamSlots = 4;
-constexpr int kTeamMaxBlocks = 16;
+constexpr int kTeamMaxBlocks = 32;
 
 struct TeamArgs {
   const double* X;
