@@ -392,20 +392,18 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
     c->var = &kBlockShape;
     c->blocked = true;
     if (pl.team_blocks > 0 && !c->opt_two_sweeps) {
-      // one read of X: teams of team_blocks workgroups, all resident at once;
-      // partners share an XCD, so the grid is a whole number of teams per XCD
+      // one read of X: teams of team_blocks workgroups, all resident at once
       int tocc = 0, tocc2 = 0;
       PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
                      &tocc, reinterpret_cast<const void*>(kTeam[1][0]), threads, 0));
       PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
                      &tocc2, reinterpret_cast<const void*>(kTeam[0][0]), threads, 0));
       if (tocc2 < tocc) tocc = tocc2;
-      const int per_xcd = tocc * c->num_cu / plr::kXcds;  // workgroups resident on one XCD
-      const int teams_per_xcd = per_xcd / pl.team_blocks;
-      if (teams_per_xcd >= 1) {
+      const int nteams = tocc * c->num_cu / pl.team_blocks;
+      if (nteams >= 1) {
         c->team_blocks = pl.team_blocks;
         c->team_blk_chunks = pl.team_blk_chunks;
-        c->nteams = teams_per_xcd * plr::kXcds;
+        c->nteams = nteams;
         c->grid = c->grid_nograd = c->nteams * c->team_blocks;
         c->zx_words = (int64_t)c->nteams * plr::kTeamSlots * c->team_blocks * 2;
         char b[256];

@@ -1112,10 +1112,9 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
 // waiting -- the host reports the pass as failed.
 //
 // Same reference loops as shard_pass (lr.cpp:69-72,132-138,322-330,361-363).
-constexpr int kXcds = 8;        // workgroups are dealt to the XCDs round-robin
 constexpr int kTeamWaves = 8;
 constexpr int kTeamSlots = 4;
-constexpr int kTeamMaxBlocks = 32;
+constexpr int kTeamMaxBlocks = 64;
 
 struct TeamArgs {
   const double* X;
@@ -1127,7 +1126,7 @@ struct TeamArgs {
   double* h_out;             // n, or nullptr
   int64_t n, pitch;
   int nblk;                  // B: column blocks = workgroups per team (<= kTeamMaxBlocks)
-  int nteams;                // grid = nteams * nblk, nteams a multiple of kXcds
+  int nteams;                // grid = nteams * nblk
   int blk_chunks;            // 128-column chunks per block (a multiple of 8)
   int nch_rt;                // chunks per wave = blk_chunks / 8  (<= NCH)
   const double* theta_bias;  // as in PassArgs
@@ -1162,11 +1161,14 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
   constexpr int kIdentity = (LM == kTeamLmSquared || LM == kTeamLmLinearNone) ? 1 : 0;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  // partners share an XCD (and with it an L2): consecutive workgroup ids go
-  // to consecutive XCDs, so the team's members are kXcds apart
-  const int xcd = blockIdx.x % kXcds, k = blockIdx.x / kXcds;
-  const int blk = k % a.nblk;
-  const int team = (k / a.nblk) * kXcds + xcd;
+  // A team is nblk consecutive workgroups.  Consecutive workgroup ids go to
+  // consecutive XCDs, so its members sit on different XCDs and meet in memory,
+  // not in an L2 -- the exchange has a whole step to complete, and measured
+  // against teams kept inside one XCD this is faster at every width (+1 % at
+  // 32768 columns, +9 % at 65536 with the same number of teams), besides
+  // leaving no compute unit idle where nblk does not divide an XCD's 32.
+  const int blk = (int)(blockIdx.x % a.nblk);
+  const int team = (int)(blockIdx.x / a.nblk);
 
   const int64_t total_chunks = (a.pitch + kChunkCols - 1) / kChunkCols;
   const int64_t c0 = (int64_t)blk * a.blk_chunks + (int64_t)wave * a.nch_rt;  // my first chunk

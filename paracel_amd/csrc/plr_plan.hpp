@@ -15,7 +15,7 @@ constexpr int64_t kMaxPairPitch = 96;    // up to this pitch: a half-wave per ro
 constexpr int64_t kMaxFusedCols = 19456; // beyond: column blocks, two sweeps over X
 constexpr int kBlkNch = 16, kBlkWcol = 8;
 constexpr int64_t kBlockCols = (int64_t)kBlkNch * kBlkWcol * kChunkCols;  // 16384
-constexpr int kMaxTeamBlocks = 32;       // column blocks a team of workgroups may span
+constexpr int kMaxTeamBlocks = 64;       // column blocks a team of workgroups may span
 constexpr int kTeamNch = 8;              // chunks per wave the team kernel is built for
 constexpr int kAlwaysOneWave = 16;       // up to here no several-waves variant is considered
 constexpr int kMaxRowChunks = 32;        // widest one-wave row

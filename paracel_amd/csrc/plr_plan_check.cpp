@@ -44,7 +44,7 @@ int main(int argc, char** argv) {
     return 0;
   }
   std::vector<int64_t> used(kNumShapes, 0);
-  const int64_t kMaxD = 140000;
+  const int64_t kMaxD = 600000;
   // every width twice: rows unknown (a large shard) and a one-row shard (the
   // short-tile entries of the table)
   for (int64_t dn = 2; dn <= 2 * kMaxD + 1; ++dn) {

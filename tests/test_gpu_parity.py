@@ -184,16 +184,17 @@ def test_linear_model_pieces(plr, oracle, gen, n, d):
 @pytest.mark.parametrize("two_sweeps", [0, 1])
 @pytest.mark.parametrize("n,d", [(19, 19457), (300, 33000), (1030, 20001), (64, 65536),
                                  (700, 32768), (515, 24577), (40, 131072), (12, 140000),
-                                 (9, 262144), (5, 262200), (3, 20000), (2100, 20016)])
+                                 (9, 262144), (5, 262200), (3, 524288), (3, 524300),
+                                 (3, 20000), (2100, 20016)])
 def test_rows_wider_than_the_fused_kernels(plr, oracle, gen, n, d, two_sweeps):
     # past 19456 columns the row is processed in column blocks: by teams of workgroups that
-    # exchange partial dot products (X read once; up to 32 blocks of 8192 columns), or in two
+    # exchange partial dot products (X read once; up to 64 blocks of 8192 columns), or in two
     # sweeps over X
     print("case n=%d d=%d two_sweeps=%d" % (n, d, two_sweeps), flush=True)
     X, y, th = make(gen, n, d)
     plr.set_option("column_blocks_two_sweeps", two_sweeps)
     plr.set_data(X, y)
-    assert ("team_pass" in plr.kernel_info()) == (not two_sweeps and d <= 262144)
+    assert ("team_pass" in plr.kernel_info()) == (not two_sweeps and d <= 524288)
     print(plr.kernel_info(), flush=True)
     g, loss, n_out = plr.loss_grad(th)
     assert n_out == n

@@ -26,7 +26,7 @@ def plan(d, n=None):
 def test_every_width_satisfies_the_kernels_assumptions():
     r = subprocess.run([TOOL], capture_output=True, text=True)
     assert r.returncode == 0, r.stdout
-    assert r.stdout.strip().startswith("ok: 140000 widths")
+    assert r.stdout.strip().startswith("ok: 600000 widths")
 
 
 def test_the_benchmark_shapes_take_the_intended_variants():
