@@ -94,7 +94,7 @@ MEASURED_TRAFFIC = {
         "profiles/lane2_pass_x_narrow_10m_x_41.md"),
     "x_verywide_100k_x_32768": (
         100000, "team_pass<NCH=8> 4 column blocks of 64 chunks, 64 teams, pitch=32768 "
-        "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26309460592,
+        "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)", 26344324303,
         "profiles/team_pass_x_verywide_100k_x_32768.md"),
 }
 
