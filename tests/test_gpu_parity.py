@@ -39,6 +39,11 @@ SHAPES = [
     # several tiles per row group and a partial last tile, for every tile height
     (40003, 256), (20005, 512), (9001, 1000), (6149, 2047), (3077, 4097), (2053, 8193),
     (8195, 100), (515, 16384),
+    # 8 waves side by side with 9..19 chunks each: every count has a variant of its own
+    # (exact multiples of 1024 columns, and rows that leave the last wave short)
+    (70, 9000), (33, 9216), (45, 10000), (40, 11000), (31, 11264), (40, 12288), (36, 13000),
+    (29, 13312), (33, 14000), (30, 15000), (27, 15360), (30, 17000), (25, 18000), (23, 18432),
+    (25, 19000),
     # 65..96 columns: a half-wave per row (pair_pass), 16 rows per tile
     (1, 65), (15, 66), (16, 67), (17, 72), (1000, 80), (4099, 95), (40003, 96), (300, 97),
 ]
