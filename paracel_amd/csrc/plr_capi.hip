@@ -84,16 +84,37 @@ const pass_fn kBlockAxpy[2] = {
 // workgroup of a team owns one column block and the partial dot products are
 // exchanged per row.  [grad]
 typedef void (*team_fn)(plr::TeamArgs);
-// three row buffers per wave: the deepest pipeline that leaves the register file unspilled
-#define PLR_TEAM(GRAD, LM) plr::team_pass<plr_plan::kTeamNch, GRAD, plr::LM>
-// [grad][link / loss formula]
-const team_fn kTeam[2][5] = {
-    {PLR_TEAM(false, kTeamLmReference), PLR_TEAM(false, kTeamLmStable),
-     PLR_TEAM(false, kTeamLmNone), PLR_TEAM(false, kTeamLmSquared),
-     PLR_TEAM(false, kTeamLmLinearNone)},
-    {PLR_TEAM(true, kTeamLmReference), PLR_TEAM(true, kTeamLmStable),
-     PLR_TEAM(true, kTeamLmNone), PLR_TEAM(true, kTeamLmSquared),
-     PLR_TEAM(true, kTeamLmLinearNone)}};
+// [grad][link / loss formula]; a gradient pass with the identity link always
+// carries the squared loss (plr_dgd_delta_linear), so that slot stays empty
+struct TeamFns {
+  team_fn fn[2][5];
+};
+template <int NCH, int LAG>
+TeamFns make_team_fns() {
+  TeamFns f;
+#define PLR_TEAM(GRAD, LM) plr::team_pass<NCH, GRAD, plr::LM, LAG>
+  f.fn[0][0] = PLR_TEAM(false, kTeamLmReference);
+  f.fn[0][1] = PLR_TEAM(false, kTeamLmStable);
+  f.fn[0][2] = PLR_TEAM(false, kTeamLmNone);
+  f.fn[0][3] = PLR_TEAM(false, kTeamLmSquared);
+  f.fn[0][4] = PLR_TEAM(false, kTeamLmLinearNone);
+  f.fn[1][0] = PLR_TEAM(true, kTeamLmReference);
+  f.fn[1][1] = PLR_TEAM(true, kTeamLmStable);
+  f.fn[1][2] = PLR_TEAM(true, kTeamLmNone);
+  f.fn[1][3] = PLR_TEAM(true, kTeamLmSquared);
+  f.fn[1][4] = nullptr;
+#undef PLR_TEAM
+  return f;
+}
+// [chunks per wave - kTeamMinNch][lag - 1]
+const TeamFns kTeam[plr_plan::kTeamNch - plr_plan::kTeamMinNch + 1][2] = {
+    {make_team_fns<5, 1>(), make_team_fns<5, 2>()},
+    {make_team_fns<6, 1>(), make_team_fns<6, 2>()},
+    {make_team_fns<7, 1>(), make_team_fns<7, 2>()},
+    {make_team_fns<8, 1>(), make_team_fns<8, 2>()}};
+static_assert(plr_plan::kTeamMinNch == 5 && plr_plan::kTeamNch == 8 &&
+                  plr_plan::kTeamWaves == plr::kTeamWaves,
+              "one team kernel set per chunk count");
 constexpr int64_t kHostPredictCols = 192;  // from this pitch on predictions go straight to host
 constexpr unsigned kTeamSpinLimit = 1u << 22;  // polls before a wait for a partner gives up
 
@@ -183,6 +204,10 @@ constexpr int kNaMaxDevices = 64;
 std::mutex g_na_mutex;
 unsigned char* g_na_ptr[kNaMaxDevices] = {};
 int g_na_num_cu[kNaMaxDevices] = {};
+// workgroups per compute unit of the variant for a pitch of k chunks, per
+// device (0: not asked yet): the occupancy query runs once per (device, pitch)
+int g_na_occ[kNaMaxDevices][kNaMaxPitch / plr::kChunkCols + 1] = {};
+std::mutex g_err_mutex;  // g_create_error is shared by every context-free call
 
 }  // namespace
 
@@ -220,11 +245,25 @@ struct plr_ctx {
   const PairVariant* pair = nullptr;      // 65..96 columns: half-wave rows
   bool blocked = false;         // rows wider than the widest fused variant: column blocks
   // ... read once by teams of workgroups (team_blocks > 0), else in two sweeps
-  int team_blocks = 0, team_blk_chunks = 0, nteams = 0;
+  int team_blocks = 0, team_blk_chunks = 0, team_blk_extra = 0, team_nch = 0, nteams = 0;
+  const TeamFns* team_fns = nullptr;
+  int opt_team_lag = 1;      // plr_set_option("team_lag")
+  int opt_team_max_nch = 8;  // plr_set_option("team_max_chunks")
   unsigned long long* d_zx = nullptr;  // [nteams][4][team_blocks][2] exchange slots, then the
                                        // status word of the pass
   int64_t zx_words = 0;
   unsigned team_spin_limit = kTeamSpinLimit;
+  // A team pass needs its whole grid resident at once.  When it is not (other
+  // processes or streams holding compute units) a workgroup gives up waiting,
+  // and the pass is run again in two sweeps, which need no residency; after
+  // kTeamGiveUpsAllowed such passes the shard stays on two sweeps.
+  bool opt_team_fallback = true;  // plr_set_option("team_fallback")
+  bool team_off = false;          // team passes switched off for the resident shard
+  int team_giveups = 0;
+  int sweep_grid = 0;             // grid of the two-sweep kernels (0: not sized yet)
+  int64_t part_rows = 0;          // rows of pitch doubles that d_part_g holds
+  int64_t part_len = 0;           // entries of d_part_loss and d_part_res
+  std::string base_info;          // kernel description without the give-up note
   bool opt_two_sweeps = false;  // plr_set_option("column_blocks_two_sweeps")
   bool synth_first_col = false; // the shard being reserved comes from plr_set_data_csv
   int opt_csv_lane_rows = -1;   // plr_set_option("csv_lane_per_row"): -1 by row count, 0, 1
@@ -300,9 +339,15 @@ void free_shape(plr_ctx* c) {
   if (c->d_curve) (void)hipFree(c->d_curve);
   if (c->d_zx) (void)hipFree(c->d_zx);
   c->d_zx = nullptr;
-  c->team_blocks = c->team_blk_chunks = c->nteams = 0;
+  c->team_blocks = c->team_blk_chunks = c->team_blk_extra = c->team_nch = c->nteams = 0;
+  c->team_fns = nullptr;
   c->zx_words = 0;
   c->team_check = false;
+  c->team_off = false;
+  c->team_giveups = 0;
+  c->sweep_grid = 0;
+  c->part_rows = c->part_len = 0;
+  c->base_info.clear();
   if (c->d_z) (void)hipFree(c->d_z);
   if (c->d_res) (void)hipFree(c->d_res);
   if (c->d_train_out) (void)hipFree(c->d_train_out);
@@ -325,11 +370,28 @@ void free_shape(plr_ctx* c) {
 
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Grid of the two-sweep kernels of a column-blocked shard of n rows.
+int size_sweep_grid(plr_ctx* c, int64_t n) {
+  const int threads = plr::kWave * kBlkWcol;
+  int occ = 0, occ2 = 0;
+  PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                 &occ, reinterpret_cast<const void*>(kBlockAxpy[0]), threads, 0));
+  PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                 &occ2, reinterpret_cast<const void*>(kBlockDot[0]), threads, 0));
+  if (occ2 < occ) occ = occ2;
+  if (occ < 1) return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
+  int64_t g = (int64_t)c->num_cu * occ;
+  if (g > n) g = n;
+  if (g < 1) g = 1;
+  c->sweep_grid = (int)g;
+  return PLR_OK;
+}
+
 // Pick the kernel variant (plr_plan.hpp) and the persistent grid for an
 // n x d shard.
 int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   plr_plan::Plan pl;
-  if (!plr_plan::plan_width(d, pl, n))
+  if (!plr_plan::plan_width(d, pl, n, c->opt_team_max_nch))
     return fail(c, PLR_ERR_UNSUPPORTED, "no kernel variant covers this width");
   c->pitch = pl.pitch;
   c->theta_len = pl.theta_len;
@@ -392,41 +454,43 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
     c->var = &kBlockShape;
     c->blocked = true;
     if (pl.team_blocks > 0 && !c->opt_two_sweeps) {
-      // one read of X: teams of team_blocks workgroups, all resident at once
-      int tocc = 0, tocc2 = 0;
-      PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                     &tocc, reinterpret_cast<const void*>(kTeam[1][0]), threads, 0));
-      PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                     &tocc2, reinterpret_cast<const void*>(kTeam[0][0]), threads, 0));
-      if (tocc2 < tocc) tocc = tocc2;
+      // one read of X: teams of team_blocks workgroups, all resident at once.
+      // Any of the instances may be launched on this shard, so the grid is
+      // sized to the one that fits the fewest workgroups on a compute unit.
+      const TeamFns* tf = &kTeam[pl.team_nch - plr_plan::kTeamMinNch][c->opt_team_lag - 1];
+      int tocc = 1 << 30;
+      for (int g = 0; g < 2; ++g)
+        for (int lm = 0; lm < 5; ++lm) {
+          if (!tf->fn[g][lm]) continue;
+          int o = 0;
+          PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                         &o, reinterpret_cast<const void*>(tf->fn[g][lm]), threads, 0));
+          if (o < tocc) tocc = o;
+        }
       const int nteams = tocc * c->num_cu / pl.team_blocks;
       if (nteams >= 1) {
+        c->team_fns = tf;
         c->team_blocks = pl.team_blocks;
         c->team_blk_chunks = pl.team_blk_chunks;
+        c->team_blk_extra = pl.team_blk_extra;
+        c->team_nch = pl.team_nch;
         c->nteams = nteams;
         c->grid = c->grid_nograd = c->nteams * c->team_blocks;
         c->zx_words = (int64_t)c->nteams * plr::kTeamSlots * c->team_blocks * 2;
         char b[256];
         snprintf(b, sizeof b,
-                 "team_pass<NCH=%d> %d column blocks of %d chunks, %d teams, pitch=%lld "
+                 "team_pass<NCH=%d,LAG=%d> %d column blocks of %d%s chunks, %d teams, pitch=%lld "
                  "grid=%d x %d threads (occupancy %d blocks/CU, %d CUs)",
-                 plr_plan::kTeamNch, c->team_blocks, c->team_blk_chunks, c->nteams,
-                 (long long)c->pitch, c->grid, threads, tocc, c->num_cu);
+                 c->team_nch, c->opt_team_lag, c->team_blocks, c->team_blk_chunks,
+                 c->team_blk_extra ? "-" : "", c->nteams, (long long)c->pitch, c->grid, threads,
+                 tocc, c->num_cu);
         c->info = b;
         return PLR_OK;
       }
     }
-    int occ = 0, occ2 = 0;
-    PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                   &occ, reinterpret_cast<const void*>(kBlockAxpy[0]), threads, 0));
-    PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                   &occ2, reinterpret_cast<const void*>(kBlockDot[0]), threads, 0));
-    if (occ2 < occ) occ = occ2;
-    if (occ < 1) return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
-    int64_t g = (int64_t)c->num_cu * occ;
-    if (g > n) g = n;
-    if (g < 1) g = 1;
-    c->grid = c->grid_nograd = (int)g;
+    const int rc = size_sweep_grid(c, n);
+    if (rc != PLR_OK) return rc;
+    c->grid = c->grid_nograd = c->sweep_grid;
     char b[256];
     snprintf(b, sizeof b,
              "column-blocked shard_pass<NCH=%d,R=1,WCOL=%d> two sweeps over %lld blocks of %lld "
@@ -510,11 +574,18 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
   }
   const int gmax = c->grid > c->grid_nograd ? c->grid : c->grid_nograd;
   PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)(c->theta_len + 8) * sizeof(double)));
-  PLR_HIP(c, hipMalloc(&c->d_part_res, (size_t)gmax * sizeof(double)));
-  PLR_HIP(c, hipMalloc(&c->d_part_g, (size_t)c->grid * c->pitch * sizeof(double)));
-  PLR_HIP(c, hipMalloc(&c->d_part_loss, (size_t)gmax * sizeof(double)));
+  // a team shares one row of gradient partials
+  c->part_rows = c->team_blocks > 0 ? c->nteams : c->grid;
+  c->part_len = gmax;
+  PLR_HIP(c, hipMalloc(&c->d_part_res, (size_t)c->part_len * sizeof(double)));
+  PLR_HIP(c, hipMalloc(&c->d_part_g, (size_t)c->part_rows * c->pitch * sizeof(double)));
+  PLR_HIP(c, hipMalloc(&c->d_part_loss, (size_t)c->part_len * sizeof(double)));
   if (c->team_blocks > 0) {
+    // exchange slots, then the status word; the slots are cleared before every
+    // launch, the status word only here and when the host has read a give-up
     PLR_HIP(c, hipMalloc(&c->d_zx, (size_t)(c->zx_words + 1) * sizeof(unsigned long long)));
+    PLR_HIP(c, hipMemsetAsync(c->d_zx, 0, (size_t)(c->zx_words + 1) * sizeof(unsigned long long),
+                              c->stream));
   } else if (c->blocked && n > 0) {
     PLR_HIP(c, hipMalloc(&c->d_z, (size_t)n * sizeof(double)));
     PLR_HIP(c, hipMalloc(&c->d_res, (size_t)n * sizeof(double)));
@@ -534,6 +605,7 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
                                 (size_t)(c->pitch - c->dcols) * sizeof(double), (size_t)n,
                                 c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
+  c->base_info = c->info;
   c->have_data = true;
   return PLR_OK;
 }
@@ -575,7 +647,8 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   const Shape* v = c->var;
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
   const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
-  const int grid = grad ? c->grid : c->grid_nograd;
+  const bool team = c->team_blocks > 0 && !c->team_off;
+  const int grid = (c->blocked && !team) ? c->sweep_grid : grad ? c->grid : c->grid_nograd;
   const int threads = c->lane ? plr::kWave * c->lane->wrow * c->lane->wcol
                       : c->pair ? plr::kWave * c->pair->wrow
                                 : plr::kWave * v->wcol * v->wrow;
@@ -613,10 +686,12 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     hipLaunchKernelGGL(c->fns->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
                        c->stream, pa);
     PLR_HIP(c, hipGetLastError());
-  } else if (c->team_blocks > 0) {
-    // exchange slots and the status word start at zero (sequence number 0 = empty)
+  } else if (team) {
+    // the exchange slots start at zero (sequence number 0 = empty).  The status
+    // word behind them is NOT cleared here: a give-up in any pass of a chain of
+    // passes enqueued back to back must still be there when the host looks.
     hipLaunchKernelGGL(plr::fill_zero, dim3(16), dim3(256), 0, c->stream,
-                       reinterpret_cast<double*>(c->d_zx), c->zx_words + 1);
+                       reinterpret_cast<double*>(c->d_zx), c->zx_words);
     PLR_HIP(c, hipGetLastError());
     plr::TeamArgs ta;
     ta.X = c->dX;
@@ -630,7 +705,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     ta.nblk = c->team_blocks;
     ta.nteams = c->nteams;
     ta.blk_chunks = c->team_blk_chunks;
-    ta.nch_rt = c->team_blk_chunks / plr::kTeamWaves;
+    ta.blk_extra = c->team_blk_extra;
     ta.theta_bias = pa.theta_bias;
     ta.part_res = pa.part_res;
     ta.zeros = c->d_theta + c->theta_len - plr::kChunkCols;  // the padding never changes
@@ -640,7 +715,8 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     const int lm = pa.identity_link ? (pa.loss_mode == plr::kLossSquared ? plr::kTeamLmSquared
                                                                          : plr::kTeamLmLinearNone)
                                     : (int)pa.loss_mode;  // kLossReference/Stable/None = 0/1/2
-    hipLaunchKernelGGL(kTeam[grad ? 1 : 0][lm], dim3(grid), dim3(threads), 0, c->stream, ta);
+    hipLaunchKernelGGL(c->team_fns->fn[grad ? 1 : 0][lm], dim3(grid), dim3(threads), 0, c->stream,
+                       ta);
     PLR_HIP(c, hipGetLastError());
     c->team_check = true;
   } else if (c->n > 0) {
@@ -703,7 +779,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     fa.n = c->n;
     fa.part_res = pa.part_res;
     fa.theta_bias = c->d_theta + c->bias_slot;
-    fa.nparts = c->team_blocks > 0 ? c->nteams : grid;  // a team shares one row of partials
+    fa.nparts = team ? c->nteams : grid;  // a team shares one row of partials
     fa.nparts_loss = fa.nparts;
     fa.delta_mode = (kind == kPassDelta) ? (train_round >= 0 ? 2 : 1) : 0;
     fa.have_grad = grad ? 1 : 0;
@@ -741,16 +817,62 @@ int account_timing(plr_ctx* c) {
 }
 
 // After the stream has drained: did a workgroup of a team pass give up waiting
-// for a partner?  Then the results of that pass are not the shard's.
-int check_team_status(plr_ctx* c) {
-  if (!c->team_check) return PLR_OK;
+// for a partner?  Then the results of every pass since the last look are not
+// the shard's.  Returns 1 if so (the status word is cleared again), 0 if not,
+// a negative status if the look itself failed.
+int team_gave_up(plr_ctx* c) {
+  if (!c->team_check) return 0;
   c->team_check = false;
   unsigned long long st = 0;
   PLR_HIP(c, hipMemcpy(&st, c->d_zx + c->zx_words, sizeof st, hipMemcpyDeviceToHost));
-  if ((unsigned)st != 0u)
+  if ((unsigned)st == 0u) return 0;
+  PLR_HIP(c, hipMemset(c->d_zx + c->zx_words, 0, sizeof st));
+  return 1;
+}
+
+constexpr int kTeamGiveUpsAllowed = 2;  // then the shard stays on two sweeps
+
+// A team pass gave up.  Either report it (fallback switched off), or make the
+// two-sweep path ready -- its grid, z and residual vectors, partials for its
+// grid -- and switch the team path off: for the pass that is run again right
+// away (the caller switches it back on afterwards unless this was the last
+// give-up allowed), or for good.
+int fall_back_to_two_sweeps(plr_ctx* c) {
+  if (!c->opt_team_fallback)
     return fail(c, PLR_ERR_HIP,
                 "team pass: a workgroup gave up waiting for its partners' partial dot products "
                 "(are all workgroups of the grid resident?); results discarded");
+  c->team_giveups += 1;
+  if (c->sweep_grid == 0) {
+    const int rc = size_sweep_grid(c, c->n);
+    if (rc != PLR_OK) return rc;
+  }
+  if (!c->d_z && c->n > 0) {
+    PLR_HIP(c, hipMalloc(&c->d_z, (size_t)c->n * sizeof(double)));
+    PLR_HIP(c, hipMalloc(&c->d_res, (size_t)c->n * sizeof(double)));
+  }
+  if (c->part_rows < c->sweep_grid) {
+    PLR_HIP(c, hipFree(c->d_part_g));
+    c->d_part_g = nullptr;
+    c->part_rows = 0;
+    PLR_HIP(c, hipMalloc(&c->d_part_g, (size_t)c->sweep_grid * c->pitch * sizeof(double)));
+    c->part_rows = c->sweep_grid;
+  }
+  if (c->part_len < c->sweep_grid) {
+    PLR_HIP(c, hipFree(c->d_part_loss));
+    PLR_HIP(c, hipFree(c->d_part_res));
+    c->d_part_loss = c->d_part_res = nullptr;
+    c->part_len = 0;
+    PLR_HIP(c, hipMalloc(&c->d_part_loss, (size_t)c->sweep_grid * sizeof(double)));
+    PLR_HIP(c, hipMalloc(&c->d_part_res, (size_t)c->sweep_grid * sizeof(double)));
+    c->part_len = c->sweep_grid;
+  }
+  c->team_off = true;
+  char b[200];
+  snprintf(b, sizeof b, "; %d team pass%s gave up waiting and ran again in two sweeps%s",
+           c->team_giveups, c->team_giveups == 1 ? "" : "es",
+           c->team_giveups >= kTeamGiveUpsAllowed ? ", team passes now off for this shard" : "");
+  c->info = c->base_info + b;
   return PLR_OK;
 }
 
@@ -783,8 +905,17 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
   if (rc != PLR_OK) return rc;
   // (measured: hipStreamSynchronize returns ~7 us sooner than a hipStreamQuery poll loop)
   PLR_HIP(c, hipStreamSynchronize(c->stream));
-  rc = check_team_status(c);
-  if (rc != PLR_OK) return rc;
+  rc = team_gave_up(c);
+  if (rc < 0) return rc;
+  if (rc == 1) {
+    // theta is still staged; the same pass once more, in two sweeps
+    rc = fall_back_to_two_sweeps(c);
+    if (rc != PLR_OK) return rc;
+    rc = enqueue_pass(c, kind, loss_mode, alpha, beta, c->h_out_dev, -1);
+    if (rc != PLR_OK) return rc;
+    PLR_HIP(c, hipStreamSynchronize(c->stream));
+    if (c->team_giveups < kTeamGiveUpsAllowed) c->team_off = false;
+  }
   return account_timing(c);
 }
 
@@ -793,8 +924,12 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
 extern "C" {
 
 int plr_create(plr_ctx** out, int device_id) {
+  auto set_err = [](const std::string& m) {
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    g_create_error = m;
+  };
   if (!out) {
-    g_create_error = "out must not be NULL";
+    set_err("out must not be NULL");
     return PLR_ERR_INVALID;
   }
   *out = nullptr;
@@ -802,11 +937,11 @@ int plr_create(plr_ctx** out, int device_id) {
   hipError_t e = hipGetDeviceCount(&count);
   if (e != hipSuccess || count < 1) {
     (void)hipGetLastError();
-    g_create_error = std::string("no HIP device available: ") + hipGetErrorString(e);
+    set_err(std::string("no HIP device available: ") + hipGetErrorString(e));
     return PLR_ERR_HIP;
   }
   if (device_id < 0 || device_id >= count) {
-    g_create_error = "device_id out of range";
+    set_err("device_id out of range");
     return PLR_ERR_INVALID;
   }
   plr_ctx* c = new plr_ctx();
@@ -817,14 +952,14 @@ int plr_create(plr_ctx** out, int device_id) {
       (e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking)) != hipSuccess ||
       (e = hipEventCreate(&c->ev0)) != hipSuccess ||
       (e = hipEventCreate(&c->ev1)) != hipSuccess) {
-    g_create_error = std::string("context set-up failed: ") + hipGetErrorString(e);
+    set_err(std::string("context set-up failed: ") + hipGetErrorString(e));
     (void)hipGetLastError();
     plr_destroy(c);
     return PLR_ERR_HIP;
   }
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
-    g_create_error = std::string("device is ") + prop.gcnArchName +
-                     "; this library carries gfx950 code only";
+    set_err(std::string("device is ") + prop.gcnArchName +
+            "; this library carries gfx950 code only");
     plr_destroy(c);
     return PLR_ERR_UNSUPPORTED;
   }
@@ -864,7 +999,15 @@ int plr_set_data(plr_ctx* c, const double* X, int64_t n, int64_t d, int64_t ldx,
   if (ldx < d) return fail(c, PLR_ERR_INVALID, "ldx must be >= d");
   int rc = alloc_shape(c, n, d, /*zero_fill=*/false);  // every row is uploaded right below
   if (rc != PLR_OK) return rc;
-  return upload_rows(c, 0, n, X, ldx, y);
+  rc = upload_rows(c, 0, n, X, ldx, y);
+  if (rc != PLR_OK) {
+    // a shard that was not filled (a refused first column, a failed copy) must
+    // not stay resident: later passes would run on whatever the memory holds
+    const std::string why = c->err;
+    free_shape(c);
+    c->err = why;
+  }
+  return rc;
 }
 
 // ---------------------------------------------------------------------------
@@ -1092,6 +1235,7 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   c->csv_slow_fields = nslow;
   c->info += std::string("; parsed from text (a ") + (lane_rows ? "lane" : "wave") +
              " per row), " + std::to_string(nslow) + " fields converted on the host";
+  c->base_info = c->info;
   if (c->timing) {  // plr_get_timing's last_ms: the parsing kernel
     float ms = 0.f;
     PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
@@ -1194,23 +1338,35 @@ int plr_train_dgd(plr_ctx* c, double* theta, double alpha, double beta, int roun
   }
   if (!c->d_train_out)
     PLR_HIP(c, hipMalloc(&c->d_train_out, (size_t)(c->d + 1) * sizeof(double)));
-  int rc = stage_theta_from_host(c, theta);
-  if (rc != PLR_OK) return rc;
   const unsigned loss_mode = loss_curve ? plr::kLossReference : plr::kLossNone;
-  // every round is enqueued back to back; theta never leaves the device
-  for (int rd = 0; rd < rounds; ++rd) {
-    rc = enqueue_pass(c, kPassDelta, loss_mode, alpha, beta, c->d_train_out, rd);
-    if (rc != PLR_OK) return rc;
-  }
   const int skip = c->bias ? 1 : 0;
-  PLR_HIP(c, hipMemcpyAsync(c->h_theta + skip, c->d_theta, (size_t)c->dcols * sizeof(double),
-                            hipMemcpyDeviceToHost, c->stream));
-  if (c->bias)
-    PLR_HIP(c, hipMemcpyAsync(c->h_theta, c->d_theta + c->bias_slot, sizeof(double),
+  int rc = PLR_OK;
+  for (int attempt = 0;; ++attempt) {
+    rc = stage_theta_from_host(c, theta);
+    if (rc != PLR_OK) return rc;
+    // every round is enqueued back to back; theta never leaves the device
+    for (int rd = 0; rd < rounds; ++rd) {
+      rc = enqueue_pass(c, kPassDelta, loss_mode, alpha, beta, c->d_train_out, rd);
+      if (rc != PLR_OK) return rc;
+    }
+    PLR_HIP(c, hipMemcpyAsync(c->h_theta + skip, c->d_theta, (size_t)c->dcols * sizeof(double),
                               hipMemcpyDeviceToHost, c->stream));
-  PLR_HIP(c, hipStreamSynchronize(c->stream));
-  rc = check_team_status(c);
-  if (rc != PLR_OK) return rc;
+    if (c->bias)
+      PLR_HIP(c, hipMemcpyAsync(c->h_theta, c->d_theta + c->bias_slot, sizeof(double),
+                                hipMemcpyDeviceToHost, c->stream));
+    PLR_HIP(c, hipStreamSynchronize(c->stream));
+    // a give-up in ANY round leaves the status word set (it is not cleared
+    // between rounds) and every later round ran on a theta that is not the
+    // shard's: the whole training is run again from the caller's theta, in two
+    // sweeps
+    rc = team_gave_up(c);
+    if (rc < 0) return rc;
+    if (rc == 0) break;
+    rc = fall_back_to_two_sweeps(c);
+    if (rc != PLR_OK) return rc;
+    if (attempt >= 1) return fail(c, PLR_ERR_HIP, "team pass gave up although switched off");
+  }
+  if (c->team_off && c->team_giveups < kTeamGiveUpsAllowed) c->team_off = false;
   memcpy(theta, c->h_theta, (size_t)c->d * sizeof(double));
   if (loss_curve)
     PLR_HIP(c, hipMemcpy(loss_curve, c->d_curve, (size_t)rounds * sizeof(double),
@@ -1615,6 +1771,21 @@ int plr_set_option(plr_ctx* c, const char* key, int64_t value) {
     c->team_spin_limit = (unsigned)value;
     return PLR_OK;
   }
+  if (strcmp(key, "team_lag") == 0) {
+    if (value < 1 || value > 2) return fail(c, PLR_ERR_INVALID, "team_lag is 1 or 2");
+    c->opt_team_lag = (int)value;  // takes effect at the next plr_set_data / plr_alloc_data
+    return PLR_OK;
+  }
+  if (strcmp(key, "team_max_chunks") == 0) {
+    if (value < plr_plan::kTeamMinNch || value > plr_plan::kTeamNch)
+      return fail(c, PLR_ERR_INVALID, "team_max_chunks out of range");
+    c->opt_team_max_nch = (int)value;  // takes effect at the next plr_set_data / plr_alloc_data
+    return PLR_OK;
+  }
+  if (strcmp(key, "team_fallback") == 0) {
+    c->opt_team_fallback = value != 0;
+    return PLR_OK;
+  }
   if (strcmp(key, "first_column_is_one") == 0) {
     c->opt_first_col_one = value != 0;  // takes effect at the next plr_set_data / plr_alloc_data
     return PLR_OK;
@@ -1647,6 +1818,7 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
                           int64_t n, int64_t d, int64_t ldx, const double* dtheta,
                           double* dout, unsigned flags) {
   auto bad = [](int code, const std::string& msg) {
+    std::lock_guard<std::mutex> lock(g_err_mutex);
     g_create_error = "plr_loss_grad_noalloc: " + msg;
     return code;
   };
@@ -1664,8 +1836,27 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
     return bad(PLR_ERR_INVALID, "n * ldx overflows");
   if ((n > 0 && (!dX || !dy)) || !dtheta || !dout)
     return bad(PLR_ERR_INVALID, "device pointers must not be NULL");
+  // the pass loads X 16 bytes per lane; the other operands are read and written as doubles
+  if ((reinterpret_cast<uintptr_t>(dX) & 15u) != 0)
+    return bad(PLR_ERR_INVALID, "dX must be 16-byte aligned");
+  if (((reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(dtheta) |
+        reinterpret_cast<uintptr_t>(dout)) & 7u) != 0)
+    return bad(PLR_ERR_INVALID, "dy, dtheta and dout must be 8-byte aligned");
   if (flags > plr::kLossSquared) return bad(PLR_ERR_INVALID, "unknown loss flag");
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+
+  // the caller's current device is left as it was found
+  struct DeviceScope {
+    int prev = -1;
+    ~DeviceScope() {
+      if (prev >= 0) (void)hipSetDevice(prev);
+    }
+  } scope;
+  int cur = -1;
+  if (hipGetDevice(&cur) != hipSuccess) {
+    (void)hipGetLastError();
+    cur = -1;
+  }
 
 #define PLR_NA_HIP(call)                                                        \
   do {                                                                          \
@@ -1676,11 +1867,31 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
     }                                                                           \
   } while (0)
 
-  PLR_NA_HIP(hipSetDevice(device_id));
+  if (cur != device_id) {
+    PLR_NA_HIP(hipSetDevice(device_id));
+    scope.prev = cur;  // -1: there was none to go back to
+  }
+
+  // the row pitch is a whole number of chunks, so the variant is the exact
+  // one-wave one for ldx / 128 chunks and no lane reads past a row end
+  plr_plan::Plan pl;
+  if (!plr_plan::plan_width(ldx, pl, n) || pl.path != plr_plan::kPathFused || pl.pitch != ldx ||
+      !pl.allch || pl.tail_cols != 0 || pl.theta_len > kNaMaxPitch)
+    return bad(PLR_ERR_UNSUPPORTED, "no kernel variant covers this pitch");
+  const Shape* v = &kShapes[pl.variant];
+  const bool grad = true;
+  const pass_fn fn = kFns[pl.variant].fn[grad ? 1 : 0][1];
+  if (!fn || v->wcol != 1) return bad(PLR_ERR_UNSUPPORTED, "kernel variant lacks this instance");
+  const int threads = plr::kWave * v->wcol * v->wrow;
+
   unsigned char* base = nullptr;
-  int num_cu = 0;
+  int num_cu = 0, occ = 0;
   {
-    // first call on this device: the device's own address of the static array
+    // First call on this device (and first call with this pitch on it): the
+    // device's own address of the static array, its compute-unit count and the
+    // variant's occupancy are looked up once and kept.  These look-ups are not
+    // stream work; a caller that captures the stream makes one call per pitch
+    // it will use before the capture begins.
     std::lock_guard<std::mutex> lock(g_na_mutex);
     if (!g_na_ptr[device_id]) {
       hipDeviceProp_t prop;
@@ -1694,6 +1905,18 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
       g_na_num_cu[device_id] = prop.multiProcessorCount;
       g_na_ptr[device_id] = ptr;
     }
+    // (a pitch may map to two variants, by shard size: the slot remembers
+    // which one its figure belongs to)
+    int& slot = g_na_occ[device_id][ldx / plr::kChunkCols];
+    const int tag = (pl.variant + 1) << 8;
+    if ((slot & ~0xff) != tag) {
+      int o = 0;
+      PLR_NA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+          &o, reinterpret_cast<const void*>(fn), threads, 0));
+      if (o < 1) return bad(PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
+      slot = tag | (o > 255 ? 255 : o);
+    }
+    occ = slot & 0xff;
     base = g_na_ptr[device_id];
     num_cu = g_na_num_cu[device_id];
   }
@@ -1701,21 +1924,6 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
   double* s_loss = reinterpret_cast<double*>(base + kNaLossOff);
   double* s_part = reinterpret_cast<double*>(base + kNaPartOff);
 
-  // the row pitch is a whole number of chunks, so the variant is the exact
-  // one-wave one for ldx / 128 chunks and no lane reads past a row end
-  plr_plan::Plan pl;
-  if (!plr_plan::plan_width(ldx, pl, n) || pl.path != plr_plan::kPathFused || pl.pitch != ldx ||
-      !pl.allch || pl.tail_cols != 0 || pl.theta_len > kNaMaxPitch)
-    return bad(PLR_ERR_UNSUPPORTED, "no kernel variant covers this pitch");
-  const Shape* v = &kShapes[pl.variant];
-  const bool grad = true;
-  const pass_fn fn = kFns[pl.variant].fn[grad ? 1 : 0][1];
-  if (!fn || v->wcol != 1) return bad(PLR_ERR_UNSUPPORTED, "kernel variant lacks this instance");
-  const int threads = plr::kWave * v->wcol * v->wrow;
-  int occ = 0;
-  PLR_NA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(fn),
-                                                          threads, 0));
-  if (occ < 1) return bad(PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
   const int64_t want = ceil_div(ceil_div(n, v->R), v->wrow);
   int64_t g = std::min<int64_t>((int64_t)num_cu * occ, kNaMaxGrid);
   if (g > want) g = want;

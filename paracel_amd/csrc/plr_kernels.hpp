@@ -1089,23 +1089,24 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
 // all B workgroups add the B partials in block order, so they arrive at the
 // same bits and the team behaves like one very wide workgroup.
 //
-// Software pipeline, per workgroup, at step t:
-//     look for the partners' partials of row t - 1 (published a step ago, so
-//       the first look nearly always finds them)
-//     request row t + 1 into the buffer row t - 2 has left
+// Software pipeline, per workgroup, at step t (LAG = 1 or 2 steps between a
+// row's dot product and its update):
+//     look for the partners' partials of row t - LAG (published LAG steps ago)
+//     request row t + 1 into the buffer row t - LAG - 1 has left
 //     dot product of row t (requested a whole step ago), publish it
-//     residual of row t - 1, rank-1 update from the registers that still hold it
-// so neither the exchange nor HBM latency stalls the stream: three row
+//     residual of row t - LAG, rank-1 update from the registers that still hold it
+// so neither the exchange nor HBM latency stalls the stream: LAG + 2 row
 // buffers of NCH chunks per wave rotate.
 //
 // The exchange needs no fence: a partial travels as two 64-bit words, each
 // carrying 32 bits of the double and the 32-bit sequence number of its row
 // (never 0; the slots are zeroed before every launch), written and read with
 // relaxed device-scope atomics -- a word is valid exactly when its sequence
-// number is the expected one.  Four slots per team rotate: a workgroup that
-// has just published row t + 1 cannot be more than three rows ahead of what a
-// partner still has to read (to get there it needed the partner's row t - 1,
-// which that partner published only after reading row t - 2).  All workgroups
+// number is the expected one.  The slots of a team rotate, and 2 * LAG + 2 of
+// them are enough: a workgroup publishes row t only after it has seen every
+// partner's partial of row t - LAG - 1, and a partner that has published that
+// one still has to read the rows from t - 2 * LAG - 1 on -- so row t may
+// overwrite row t - 2 * LAG - 2 and nothing younger.  All workgroups
 // of the grid must be resident at once (the host sizes the grid to the
 // device); should a partner never show up, the wait gives up after spin_limit
 // polls, raises status[0], and every workgroup then runs to its end without
@@ -1113,7 +1114,7 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
 //
 // Same reference loops as shard_pass (lr.cpp:69-72,132-138,322-330,361-363).
 constexpr int kTeamWaves = 8;
-constexpr int kTeamSlots = 4;
+constexpr int kTeamSlots = 8;  // >= 2 * LAG + 2 for LAG <= 2, a power of two
 constexpr int kTeamMaxBlocks = 64;
 
 struct TeamArgs {
@@ -1127,8 +1128,12 @@ struct TeamArgs {
   int64_t n, pitch;
   int nblk;                  // B: column blocks = workgroups per team (<= kTeamMaxBlocks)
   int nteams;                // grid = nteams * nblk
-  int blk_chunks;            // 128-column chunks per block (a multiple of 8)
-  int nch_rt;                // chunks per wave = blk_chunks / 8  (<= NCH)
+  // The row's chunks are dealt evenly: the first blk_extra blocks own
+  // blk_chunks + 1 of them, the others blk_chunks; inside a block of m chunks
+  // the first m % 8 waves own m / 8 + 1, the others m / 8 -- so no two waves of
+  // a team differ by more than two chunks, and none owns more than NCH.
+  int blk_chunks;
+  int blk_extra;
   const double* theta_bias;  // as in PassArgs
   double* part_res;          // [nteams], or nullptr
   unsigned long long* zx;    // [nteams][kTeamSlots][nblk][2] exchange slots
@@ -1147,13 +1152,14 @@ enum : int {
   kTeamLmLinearNone = 4,  // identity link, no loss
 };
 
-template <int NCH, bool GRAD, int LM>
+template <int NCH, bool GRAD, int LM, int LAG>
 __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
-  // Row buffers: rows t - 1, t and t + 1.  (A fourth, row t + 2 in flight as well, was
-  // measured at 6 chunks per wave, where the loss-free instance fits the registers
-  // without a spill: 0.5-1 % slower at every width -- the step is not waiting for
-  // data any more once the waits below are right.)
-  constexpr int D = 3;
+  static_assert(LAG == 1 || LAG == 2, "a row's update follows its dot product by 1 or 2 steps");
+  static_assert(kTeamSlots >= 2 * LAG + 2 && (kTeamSlots & (kTeamSlots - 1)) == 0, "slot ring");
+  // Row buffers: rows t - LAG .. t + 1.  (With LAG = 1 a fourth buffer -- row
+  // t + 2 in flight as well -- was measured and is 0.5-1 % slower at every
+  // width: the step does not wait for data once the waits below are right.)
+  constexpr int D = LAG + 2;
   constexpr unsigned kLoss = LM == kTeamLmReference ? kLossReference
                              : LM == kTeamLmStable  ? kLossStable
                              : LM == kTeamLmSquared ? kLossSquared
@@ -1170,12 +1176,13 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
   const int blk = (int)(blockIdx.x % a.nblk);
   const int team = (int)(blockIdx.x / a.nblk);
 
+  // my block's chunks, then my wave's share of them
   const int64_t total_chunks = (a.pitch + kChunkCols - 1) / kChunkCols;
-  const int64_t c0 = (int64_t)blk * a.blk_chunks + (int64_t)wave * a.nch_rt;  // my first chunk
-  int64_t blk_end = (int64_t)(blk + 1) * a.blk_chunks;
-  if (blk_end > total_chunks) blk_end = total_chunks;
-  int64_t left = blk_end - c0;
-  const int my_nch = (int)(left < 0 ? 0 : (left > a.nch_rt ? a.nch_rt : left));
+  const int blk_m = a.blk_chunks + (blk < a.blk_extra ? 1 : 0);
+  const int64_t blk_c0 = (int64_t)blk * a.blk_chunks + (blk < a.blk_extra ? blk : a.blk_extra);
+  const int wq = blk_m / kTeamWaves, wrem = blk_m % kTeamWaves;
+  const int my_nch = wq + (wave < wrem ? 1 : 0);                       // <= NCH (host-checked)
+  const int64_t c0 = blk_c0 + (int64_t)wave * wq + (wave < wrem ? wave : wrem);  // my first chunk
   // the row's last chunk may be ragged (the pitch is a multiple of 16, not of 128)
   const int rag_cols = (int)(a.pitch % kChunkCols);
   const int ragged_c =
@@ -1190,8 +1197,8 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     acc[c] = v2d{0., 0.};
-    // (a slot beyond nch_rt reads the page of zeros: a scalar select, no branch)
-    const double* tp = (c < a.nch_rt) ? a.theta + (c0 + c) * kChunkCols : a.zeros;
+    // (a slot this wave does not own reads the page of zeros: a scalar select, no branch)
+    const double* tp = (c < my_nch) ? a.theta + (c0 + c) * kChunkCols : a.zeros;
     thl[c * kWave] = *reinterpret_cast<const v2d*>(tp + 2 * lane);
   }
   double loss_acc = 0., res_acc = 0.;
@@ -1199,11 +1206,10 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
   bool gave_up = false;
 
   // Uniform base + 32-bit lane offset: no address registers per chunk.  A chunk
-  // slot this wave does not own (c >= my_nch: the last block of an uneven
-  // split) reads a page of zeros instead -- a scalar select of the base, so the
-  // loop body has no branch per chunk.  The ragged chunk is loaded whole; its
-  // lanes past the row end (the next row's bytes) are dropped in the dot
-  // product and never stored.
+  // slot this wave does not own (c >= my_nch) reads a page of zeros instead --
+  // a scalar select of the base, so the loop body has no branch per chunk.  The
+  // ragged chunk is loaded whole; its lanes past the row end (the next row's
+  // bytes) are dropped in the dot product and never stored.
   const char* xwave = reinterpret_cast<const char*>(a.X + c0 * kChunkCols);
   const char* zeros = reinterpret_cast<const char*>(a.zeros);
   const uint32_t lane_off = (uint32_t)(lane * sizeof(v2d));
@@ -1227,31 +1233,31 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
   };
 
   auto step = [&](int64_t t, auto phase_tag) {
-    constexpr int PH = decltype(phase_tag)::value;      // t mod 3
-    constexpr int PREV = (PH + 2) % 3;                  // buffer of row t - 1
-    constexpr int NEXT = (PH + 1) % 3;                  // buffer of row t - 2: refilled with t + 1
+    constexpr int PH = decltype(phase_tag)::value;      // t mod D
+    constexpr int PREV = (PH + 2) % D;                  // buffer of row t - LAG
+    constexpr int NEXT = (PH + 1) % D;                  // buffer of row t - LAG - 1: refilled with t + 1
     const int par = (int)(t & 1);
     const bool have_row = t < myrows;                   // uniform
-    const bool have_prev = t >= 1;                      // uniform
+    const bool have_prev = t >= LAG;                    // uniform
 
-    // Wave 0 collects the partials of row t - 1 (its own included: one code
+    // Wave 0 collects the partials of row t - LAG (its own included: one code
     // path) with vector loads, and vector loads return in issue order: the
     // first look is requested BEFORE the next row, so it is not queued behind
     // X; any further look comes after it, at the pace rows arrive.
     const bool poller = have_prev && wave == 0 && lane < a.nblk;
-    const unsigned seq = (unsigned)t;  // sequence number of row t - 1
+    const unsigned seq = (unsigned)(t - LAG + 1);  // sequence number of row t - LAG
     const unsigned long long* pslot =
-        a.zx + ((int64_t)(team * kTeamSlots + (int)((t + kTeamSlots - 1) % kTeamSlots)) * a.nblk +
+        a.zx + ((int64_t)(team * kTeamSlots + (int)((t + kTeamSlots - LAG) % kTeamSlots)) * a.nblk +
                 (poller ? lane : 0)) * 2;
     unsigned long long w0 = 0, w1 = 0;
     if (poller) {
       w0 = __hip_atomic_load(pslot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       w1 = __hip_atomic_load(pslot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    // the label of row t - 1, for the same reason ahead of the row request: asked
-    // for where it is used, it would come back behind row t + 1 and the update
-    // of row t - 1 would wait for that whole row
-    const int64_t prev_row = team + (have_prev ? t - 1 : 0) * a.nteams;
+    // the label of row t - LAG, for the same reason ahead of the row request:
+    // asked for where it is used, it would come back behind row t + 1 and the
+    // update would wait for that whole row
+    const int64_t prev_row = team + (have_prev ? t - LAG : 0) * a.nteams;
     const double yv = *(a.y ? a.y + prev_row : a.zeros);
     asm volatile("" ::: "memory");
     request(t + 1, X[NEXT]);
@@ -1324,19 +1330,32 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
   };
 
   // Row 0 is requested up front; step t requests row t + 1 first thing.
-  // Steps 0 .. myrows: the last one only finishes row myrows - 1.
+  // Steps 0 .. myrows + LAG - 1: the last LAG only finish rows.
   if (myrows > 0) {
     request(0, X[0]);
-    const int64_t nsteps = myrows + 1;
+    const int64_t nsteps = myrows + LAG;
     int64_t t = 0;
+    if constexpr (D == 3) {
 #pragma clang loop unroll(disable)
-    for (; t + 3 <= nsteps; t += 3) {
-      step(t, std::integral_constant<int, 0>{});
-      step(t + 1, std::integral_constant<int, 1>{});
-      step(t + 2, std::integral_constant<int, 2>{});
+      for (; t + 3 <= nsteps; t += 3) {
+        step(t, std::integral_constant<int, 0>{});
+        step(t + 1, std::integral_constant<int, 1>{});
+        step(t + 2, std::integral_constant<int, 2>{});
+      }
+      if (t < nsteps) step(t++, std::integral_constant<int, 0>{});
+      if (t < nsteps) step(t++, std::integral_constant<int, 1>{});
+    } else {
+#pragma clang loop unroll(disable)
+      for (; t + 4 <= nsteps; t += 4) {
+        step(t, std::integral_constant<int, 0>{});
+        step(t + 1, std::integral_constant<int, 1>{});
+        step(t + 2, std::integral_constant<int, 2>{});
+        step(t + 3, std::integral_constant<int, 3>{});
+      }
+      if (t < nsteps) step(t++, std::integral_constant<int, 0>{});
+      if (t < nsteps) step(t++, std::integral_constant<int, 1>{});
+      if (t < nsteps) step(t++, std::integral_constant<int, 2>{});
     }
-    if (t < nsteps) step(t++, std::integral_constant<int, 0>{});
-    if (t < nsteps) step(t++, std::integral_constant<int, 1>{});
   }
 
   if (GRAD) {

@@ -16,7 +16,9 @@ constexpr int64_t kMaxFusedCols = 19456; // beyond: column blocks, two sweeps ov
 constexpr int kBlkNch = 16, kBlkWcol = 8;
 constexpr int64_t kBlockCols = (int64_t)kBlkNch * kBlkWcol * kChunkCols;  // 16384
 constexpr int kMaxTeamBlocks = 64;       // column blocks a team of workgroups may span
-constexpr int kTeamNch = 8;              // chunks per wave the team kernel is built for
+constexpr int kTeamWaves = 8;            // waves of a team's workgroup, side by side
+constexpr int kTeamMinNch = 5;           // chunks per wave the team kernel is built for: from ...
+constexpr int kTeamNch = 8;              // ... to
 constexpr int kAlwaysOneWave = 16;       // up to here no several-waves variant is considered
 constexpr int kMaxRowChunks = 32;        // widest one-wave row
 
@@ -48,9 +50,13 @@ struct Plan {
   bool allch;         // every wave of the row uses exactly NCH chunks
   int tail_cols;      // columns handled by the variant's tail stage (0: none)
   // column-blocked path, one read of X: a team of team_blocks workgroups per
-  // row, each owning team_blk_chunks chunks (0 blocks: too wide, two sweeps)
+  // row (0 blocks: too wide, two sweeps); the first team_blk_extra of them own
+  // team_blk_chunks + 1 chunks, the others team_blk_chunks, and a block's
+  // chunks are dealt the same way to its 8 waves, team_nch at most each
   int team_blocks;
   int team_blk_chunks;
+  int team_blk_extra;
+  int team_nch;
 };
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -60,8 +66,10 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // n: rows of the shard when known (< 0: unknown, taken as large).  Where the
 // variant table has two entries for a shape, shards below kSmallShardBytes
 // take the one with the shorter tiles.
+// team_max_nch: the most chunks a wave of a team pass may own (kTeamMinNch ..
+// kTeamNch); fewer chunks per wave mean more workgroups per row.
 constexpr int64_t kSmallShardBytes = 1500000000;
-inline bool plan_width(int64_t d, Plan& p, int64_t n = -1) {
+inline bool plan_width(int64_t d, Plan& p, int64_t n = -1, int team_max_nch = kTeamNch) {
   p = Plan();
   p.variant = -1;
   if (d <= kMaxLaneCols) {
@@ -85,14 +93,18 @@ inline bool plan_width(int64_t d, Plan& p, int64_t n = -1) {
     // theta padded so that the last (narrower) block still reads whole slabs
     p.theta_len = ceil_div(p.pitch, kBlockCols) * kBlockCols;
     // the row's chunks dealt evenly to the fewest workgroups that can hold
-    // them, each block a whole number of chunks per wave
+    // them, and inside a workgroup evenly to its waves
     const int64_t chunks = ceil_div(p.pitch, kChunkCols);
-    const int64_t blocks = ceil_div(chunks, (int64_t)kBlkWcol * kTeamNch);
+    if (team_max_nch < kTeamMinNch) team_max_nch = kTeamMinNch;
+    if (team_max_nch > kTeamNch) team_max_nch = kTeamNch;
+    const int64_t blocks = ceil_div(chunks, (int64_t)kTeamWaves * team_max_nch);
     if (blocks <= kMaxTeamBlocks) {
       p.team_blocks = (int)blocks;
-      p.team_blk_chunks = (int)(ceil_div(ceil_div(chunks, blocks), kBlkWcol) * kBlkWcol);
-      const int64_t need = blocks * p.team_blk_chunks * kChunkCols;
-      if (need > p.theta_len) p.theta_len = need;
+      p.team_blk_chunks = (int)(chunks / blocks);
+      p.team_blk_extra = (int)(chunks % blocks);
+      const int64_t widest = p.team_blk_chunks + (p.team_blk_extra ? 1 : 0);
+      p.team_nch = (int)ceil_div(widest, kTeamWaves);
+      if (p.team_nch < kTeamMinNch) p.team_nch = kTeamMinNch;
     }
     // one more chunk of padding: the page of zeros an unowned chunk slot reads
     p.theta_len += kChunkCols;

@@ -19,6 +19,36 @@ static int failures = 0;
     }                                                                         \
   } while (0)
 
+// the team split of a column-blocked plan: replays the kernel's own arithmetic
+static void check_team(const Plan& p, int64_t d, int cap) {
+  const int64_t chunks = ceil_div(p.pitch, kChunkCols);
+  if (!p.team_blocks) {
+    CHECK(chunks > (int64_t)kMaxTeamBlocks * kTeamWaves * cap, d);
+    return;
+  }
+  CHECK(p.team_blocks >= 2 && p.team_blocks <= kMaxTeamBlocks, d);
+  CHECK(p.team_blk_extra >= 0 && p.team_blk_extra < p.team_blocks, d);
+  // the blocks cover the row exactly, and no wave owns more chunks than the kernel holds
+  CHECK((int64_t)p.team_blocks * p.team_blk_chunks + p.team_blk_extra == chunks, d);
+  CHECK(p.team_nch >= kTeamMinNch && p.team_nch <= cap, d);
+  CHECK(ceil_div(p.team_blk_chunks + (p.team_blk_extra ? 1 : 0), kTeamWaves) <= p.team_nch, d);
+  CHECK(p.team_blk_chunks >= kTeamWaves, d);  // every wave owns a chunk
+  int64_t next = 0;
+  for (int b = 0; b < p.team_blocks; ++b) {
+    const int bm = p.team_blk_chunks + (b < p.team_blk_extra ? 1 : 0);
+    const int64_t b0 = (int64_t)b * p.team_blk_chunks + (b < p.team_blk_extra ? b : p.team_blk_extra);
+    const int wq = bm / kTeamWaves, wrem = bm % kTeamWaves;
+    for (int w = 0; w < kTeamWaves; ++w) {
+      const int m = wq + (w < wrem ? 1 : 0);
+      const int64_t c0 = b0 + (int64_t)w * wq + (w < wrem ? w : wrem);
+      CHECK(c0 == next && m >= 1 && m <= p.team_nch, d);
+      next = c0 + m;
+    }
+  }
+  CHECK(next == chunks, d);
+  CHECK(p.theta_len >= chunks * kChunkCols + kChunkCols, d);
+}
+
 static void print_plan(int64_t d, int64_t n) {
   Plan p;
   if (!plan_width(d, p, n)) {
@@ -35,6 +65,9 @@ static void print_plan(int64_t d, int64_t n) {
            p.variant, s.nch, s.R, s.wcol, s.wrow, (int)s.thl, s.tl, (long long)p.chunks, p.nch_rt,
            (int)p.allch, p.tail_cols);
   }
+  if (p.path == kPathBlocked)
+    printf(" team_blocks=%d blk_chunks=%d(+1 in the first %d) nch=%d", p.team_blocks,
+           p.team_blk_chunks, p.team_blk_extra, p.team_nch);
   printf("\n");
 }
 
@@ -50,6 +83,14 @@ int main(int argc, char** argv) {
   for (int64_t dn = 2; dn <= 2 * kMaxD + 1; ++dn) {
     const int64_t d = dn / 2, n = (dn & 1) ? 1 : -1;
     Plan p;
+    if (d > kMaxFusedCols && n < 0) {
+      // the team split for every cap on the chunks per wave
+      for (int cap = kTeamMinNch; cap < kTeamNch; ++cap) {
+        Plan q;
+        CHECK(plan_width(d, q, n, cap), d);
+        check_team(q, d, cap);
+      }
+    }
     if (!plan_width(d, p, n)) {
       CHECK(false && "plan_width failed", d);
       continue;
@@ -67,13 +108,7 @@ int main(int argc, char** argv) {
       CHECK(d > kMaxFusedCols && p.pitch % 16 == 0 && p.pitch - d < 16, d);
       CHECK(p.theta_len >= p.pitch + kChunkCols, d);  // a whole chunk of zeros behind theta
       if (p.team_blocks) {
-        const int64_t chunks = ceil_div(p.pitch, kChunkCols);
-        CHECK(p.team_blocks >= 2 && p.team_blocks <= kMaxTeamBlocks, d);
-        CHECK(p.team_blk_chunks % kBlkWcol == 0 && p.team_blk_chunks / kBlkWcol <= kTeamNch, d);
-        CHECK((int64_t)p.team_blocks * p.team_blk_chunks >= chunks, d);            // covers the row
-        CHECK((int64_t)(p.team_blocks - 1) * p.team_blk_chunks < chunks, d);       // no empty block
-        CHECK(p.theta_len >=
-                  (int64_t)p.team_blocks * p.team_blk_chunks * kChunkCols + kChunkCols, d);
+        check_team(p, d, kTeamNch);
       } else {
         CHECK(ceil_div(p.pitch, kChunkCols) > (int64_t)kMaxTeamBlocks * kBlkWcol * kTeamNch, d);
       }

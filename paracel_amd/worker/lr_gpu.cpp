@@ -26,6 +26,11 @@ logistic_regression_gpu::logistic_regression_gpu(
       beta(_beta),
       debug(_debug) {
   check(plr_create(&gpu, device_id), "plr_create");
+  // Several workers on one GPU: the one-read pass over rows wider than 19456
+  // columns needs its whole grid resident at once, which processes that share
+  // the compute units cannot count on; such shards take the two-sweep pass.
+  if (get_worker_size() > 1)
+    check(plr_set_option(gpu, "column_blocks_two_sweeps", 1), "plr_set_option");
 }
 
 logistic_regression_gpu::~logistic_regression_gpu() { plr_destroy(gpu); }
@@ -140,6 +145,7 @@ void logistic_regression_gpu::solve() {
     load_and_parse(input);
     upload();
   }
+  std::cout << "shard on the device: " << plr_kernel_info(gpu) << std::endl;
   paracel_sync();
   if (learning_method == "dgd") {
     dgd_learning();

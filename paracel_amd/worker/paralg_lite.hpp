@@ -9,22 +9,34 @@
 // MPI_Barrier, ps.hpp:890-892; Comm::allreduce = MPI_Allreduce(SUM),
 // utils/comm.hpp:629-636).  Here the workers are plain processes (one shard
 // each, sharing the GPU of the box), so the same two collectives run over what
-// every worker already has a connection to -- server 0's tables:
-//   barrier    every worker adds 1 to the integer "plr_sync_<k>" (incr_int on
-//              the ssp port) and waits until it reads worker_sz (pull_int);
-//              k counts this worker's barriers, and all workers call them in
-//              the same order, as MPI requires too
-//   allreduce  every worker pushes its value under "plr_ar_<k>_<rank>",
-//              barrier, then pulls all worker_sz values and adds them in rank
-//              order -- the same bits on every worker
-// With one worker both are no-ops.
+// every worker already has a connection to -- server 0's key-value table, with
+// push and pull only (the two ops whose behaviour on a missing key is the
+// same on the reference's server: push creates it, pull answers "nokey"):
+//   barrier    worker r pushes the number k of the barrier it has reached
+//              under "plr_sync_<r>" (k = 1, 2, ...: all workers call their
+//              barriers in the same order, as MPI requires too) and waits
+//              until every worker's key reads k or more.  The counters only
+//              grow, so nothing has to be removed and the table holds
+//              worker_sz such keys however long the job runs.
+//   allreduce  worker r pushes its value under "plr_ar_<k mod 2>_<r>", barrier,
+//              then pulls all worker_sz values and adds them in rank order --
+//              the same bits on every worker.  Two slots suffice: slot k mod 2
+//              is written again in call k + 2, behind the barrier of call
+//              k + 1, which nobody passes before every worker has read call k.
+// A worker that waits longer than sync_timeout_s (PLR_SYNC_TIMEOUT_S in the
+// environment, default 1800) for a barrier throws, naming the workers that
+// did not arrive: a crashed peer ends the job instead of hanging it.
+// A server carries one job at a time (a second job's barriers would find the
+// first one's counters).  With one worker both collectives are no-ops.
 #pragma once
 
 #include <stdio.h>
+#include <stdlib.h>
 #include <sys/stat.h>
 #include <unistd.h>
 #include <zmq.h>
 
+#include <chrono>
 #include <fstream>
 #include <iostream>
 #include <memory>
@@ -249,20 +261,38 @@ class paralg {
   // ps.hpp:890-892 (MPI_Barrier there): returns once every worker has arrived
   void paracel_sync() {
     if (nworker_ <= 1) return;
-    const std::string key = "plr_sync_" + std::to_string(sync_count_++);
-    if (!kvm_[0]->incr_int(key, 1)) throw std::runtime_error("paracel_sync: incr_int failed");
-    int arrived = 0;
-    for (unsigned spins = 0;; ++spins) {
-      if (kvm_[0]->pull_int(key, arrived) && arrived >= nworker_) break;
-      usleep(spins < 64 ? 20 : 200);
+    const int k = ++sync_count_;
+    if (!kvm_[0]->push(sync_key(rank_), k)) throw std::runtime_error("paracel_sync: push failed");
+    const auto deadline =
+        std::chrono::steady_clock::now() + std::chrono::duration<double>(sync_timeout_s_);
+    int next = 0;  // workers [0, next) have been seen at barrier k
+    for (unsigned spins = 0; next < nworker_;) {
+      int at = 0;
+      if (next == rank_ || (kvm_[0]->pull(sync_key(next), at) && at >= k)) {
+        ++next;
+        continue;
+      }
+      if (std::chrono::steady_clock::now() > deadline) {
+        std::string missing;
+        for (int r = next; r < nworker_; ++r) {
+          at = 0;
+          if (r != rank_ && !(kvm_[0]->pull(sync_key(r), at) && at >= k))
+            missing += (missing.empty() ? "" : ", ") + std::to_string(r);
+        }
+        throw std::runtime_error("paracel_sync: barrier " + std::to_string(k) + ": worker(s) " +
+                                 missing + " did not arrive within " +
+                                 std::to_string(sync_timeout_s_) + " s");
+      }
+      usleep(spins++ < 64 ? 20 : 200);
     }
   }
+  void set_sync_timeout(double seconds) { sync_timeout_s_ = seconds; }
   size_t get_worker_id() const { return rank_; }
   size_t get_worker_size() const { return nworker_; }
   // comm.hpp:629-636 (MPI_Allreduce, MPI_SUM): v becomes the sum over all workers
   void allreduce(double& v) {
     if (nworker_ <= 1) return;
-    const std::string base = "plr_ar_" + std::to_string(reduce_count_++) + "_";
+    const std::string base = "plr_ar_" + std::to_string(reduce_count_++ & 1) + "_";
     if (!kvm_[0]->push(base + std::to_string(rank_), v))
       throw std::runtime_error("allreduce: push failed");
     paracel_sync();
@@ -314,8 +344,16 @@ class paralg {
   kvclt& srv(const std::string& key) {
     return *kvm_[kvm_.size() == 1 ? 0 : std::hash<std::string>()(key) % kvm_.size()];
   }
+  static std::string sync_key(int r) { return "plr_sync_" + std::to_string(r); }
+  static double default_sync_timeout() {
+    const char* e = getenv("PLR_SYNC_TIMEOUT_S");
+    const double v = e ? atof(e) : 0.;
+    return v > 0. ? v : 1800.;
+  }
   int rank_, nworker_;
-  long sync_count_ = 0, reduce_count_ = 0;
+  int sync_count_ = 0;
+  long reduce_count_ = 0;
+  double sync_timeout_s_ = default_sync_timeout();
   void* zctx_ = nullptr;
   std::vector<std::unique_ptr<kvclt> > kvm_;
 };

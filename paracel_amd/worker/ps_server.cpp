@@ -138,6 +138,28 @@ static void op_thread(void* sock) {
           }
           reply(sock, it->second);  // the new value
         }
+      } else if (op == "pullall") {
+        // server.hpp:261-264: the whole table as one packed map of key -> stored bytes
+        std::lock_guard<std::mutex> g(store_mutex);
+        std::string body;
+        const size_t n = tbl_store.size();
+        if (n < 16) {
+          body.push_back((char)(0x80 | n));
+        } else if (n < 65536) {
+          body.push_back((char)0xde);
+          detail::put_be(body, n, 2);
+        } else {
+          body.push_back((char)0xdf);
+          detail::put_be(body, n, 4);
+        }
+        for (const auto& kv : tbl_store) {
+          detail::enc(body, kv.first);
+          detail::enc(body, kv.second);
+        }
+        const size_t len = body.size();
+        std::string out((const char*)&len, sizeof len);
+        out.append(body);
+        reply(sock, out);
       } else if (op == "remove") {
         std::lock_guard<std::mutex> g(store_mutex);
         reply(sock, pack<bool>(tbl_store.erase(unpack<std::string>(msg.at(1).str())) != 0));
@@ -172,8 +194,11 @@ static void ssp_thread(void* sock) {
         if (it == ssp_tbl.end()) reply(sock, "nokey");
         else reply(sock, pack<int>(it->second));
       } else if (op == "incr_int") {
+        // kv.hpp:108-112: a missing key is not created; server.hpp:136-153
+        // answers true either way
         std::lock_guard<std::mutex> g(store_mutex);
-        ssp_tbl[unpack<std::string>(msg.at(1))] += unpack<int>(msg.at(2));
+        auto it = ssp_tbl.find(unpack<std::string>(msg.at(1)));
+        if (it != ssp_tbl.end()) it->second += unpack<int>(msg.at(2));
         reply(sock, pack<bool>(true));
       } else {
         reply(sock, pack<bool>(false));

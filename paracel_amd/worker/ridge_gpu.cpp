@@ -24,6 +24,11 @@ ridge_regression_gpu::ridge_regression_gpu(const std::string& hosts_dct_str,
       alpha(_alpha),
       beta(_beta) {
   check(plr_create(&gpu, device_id), "plr_create");
+  // Several workers on one GPU: the one-read pass over rows wider than 19456
+  // columns needs its whole grid resident at once, which processes that share
+  // the compute units cannot count on; such shards take the two-sweep pass.
+  if (get_worker_size() > 1)
+    check(plr_set_option(gpu, "column_blocks_two_sweeps", 1), "plr_set_option");
   // every shard this worker uploads starts its rows with the bias 1.0
   // (ridge.hpp:149,168): that column need not be kept in HBM
   check(plr_set_option(gpu, "first_column_is_one", 1), "plr_set_option");
@@ -88,6 +93,7 @@ void ridge_regression_gpu::batch_learning() {
 
 void ridge_regression_gpu::solve() {
   load_and_upload(input);
+  std::cout << "shard on the device: " << plr_kernel_info(gpu) << std::endl;
   paracel_sync();
   batch_learning();
   paracel_sync();

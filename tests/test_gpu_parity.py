@@ -186,6 +186,55 @@ def test_linear_model_pieces(plr, oracle, gen, n, d):
     assert abs(loss2 - want) <= 1e-12 * want
 
 
+# one shape per kernel family: lane_pass, lane2_pass, pair_pass, one-chunk shard_pass, tail
+# stage, one wave per row, several waves side by side, theta in LDS + tail, and the two
+# wide-row paths (team_pass, two sweeps)
+LINEAR_SHAPES = [(3000, 16, 0), (2500, 41, 0), (1500, 70, 0), (1000, 100, 0), (333, 257, 0),
+                 (2051, 1000, 0), (130, 4097, 0), (37, 16385, 0), (300, 20001, 0),
+                 (300, 20001, 1), (64, 65536, 0), (64, 65536, 1)]
+
+
+@pytest.mark.parametrize("first_col_one", [0, 1])
+@pytest.mark.parametrize("n,d,two_sweeps", LINEAR_SHAPES)
+def test_linear_delta_matches_oracle(plr, oracle, gen, n, d, two_sweeps, first_col_one):
+    # the identity link in every kernel family: the ridge worker's batch step
+    # (alg/regression/ridge/ridge.hpp:79-84 summed at a fixed theta), its loss (:103-109)
+    # and its prediction (:130-139), with the constant first column stored and not
+    print("case n=%d d=%d two_sweeps=%d first_col_one=%d" % (n, d, two_sweeps, first_col_one),
+          flush=True)
+    X, _, th = make(gen, n, d, seed=0x1D + d)
+    if first_col_one:
+        X[:, 0] = 1.0
+    y = X @ gen.gen_vec(7, gen.STREAM_THETA_STAR, d) + 0.3 * gen.gen_vec(99, gen.STREAM_THETA, n)
+    plr.set_option("column_blocks_two_sweeps", two_sweeps)
+    plr.set_option("first_column_is_one", first_col_one)
+    plr.set_data(X, y)
+    info = plr.kernel_info()
+    print(info, flush=True)
+    assert ("not stored" in info) == bool(first_col_one)
+    if d > 19456:
+        assert ("team_pass" in info) == (not two_sweeps)
+    alpha, beta = 0.1 / n, 0.005
+    delta, loss = plr.dgd_delta_linear(th, alpha, beta)
+    assert rel(delta, oracle.ridge_delta(X, y, th, alpha, beta)) <= GRAD_TOL
+    # the textbook form of the same step
+    assert rel(delta, alpha * (X.T @ (y - X @ th)) - 2 * alpha * beta * n * th) <= 1e-11
+    want = oracle.ridge_loss_sum(X, y, th)
+    assert abs(loss - want) <= 1e-12 * want
+    g, loss2, n_out = plr.loss_grad(th, 3)
+    assert n_out == n and rel(g, oracle.lsq_gsum(X, y, th)) <= GRAD_TOL
+    assert abs(loss2 - want) <= 1e-12 * want
+    l3, _ = plr.calc_loss(th, 3)
+    assert abs(l3 - want) <= 1e-12 * want
+    np.testing.assert_allclose(plr.predict_linear(th), oracle.predict_linear(X, th), rtol=0,
+                               atol=1e-12)
+    # the reference's own knobs (ridge README: alpha=0.01, beta=0.01 scale) and repeatability
+    d2, _ = plr.dgd_delta_linear(th, 0.01, 0.01)
+    assert rel(d2, oracle.ridge_delta(X, y, th, 0.01, 0.01)) <= GRAD_TOL
+    d3, _ = plr.dgd_delta_linear(th, 0.01, 0.01)
+    np.testing.assert_array_equal(d2, d3)
+
+
 @pytest.mark.parametrize("two_sweeps", [0, 1])
 @pytest.mark.parametrize("n,d", [(19, 19457), (300, 33000), (1030, 20001), (64, 65536),
                                  (700, 32768), (515, 24577), (40, 131072), (12, 140000),
@@ -216,6 +265,15 @@ def test_rows_wider_than_the_fused_kernels(plr, oracle, gen, n, d, two_sweeps):
     assert np.max(np.abs(plr.predict(th) - oracle.predict(X, th))) <= 1e-14
     t5 = plr.train_dgd(np.zeros(d), 0.1 / n, 0.005, 5)
     assert rel(t5, oracle.train_dgd(X, y, np.zeros(d), 0.1 / n, 0.005, 5)) <= 1e-10
+    # the identity link on the same shard: squared loss, least-squares gradient, x.theta
+    wq = oracle.ridge_loss_sum(X, y, th)
+    gq, lq, _ = plr.loss_grad(th, 3)
+    assert rel(gq, oracle.lsq_gsum(X, y, th)) <= GRAD_TOL
+    assert abs(lq - wq) <= 1e-12 * wq
+    lq2, _ = plr.calc_loss(th, 3)
+    assert abs(lq2 - wq) <= 1e-12 * wq
+    np.testing.assert_allclose(plr.predict_linear(th), oracle.predict_linear(X, th), rtol=0,
+                               atol=1e-12)
 
 
 @pytest.mark.parametrize("n,d", [(300, 2), (1000, 3), (4099, 17), (2051, 65), (2000, 66), (999, 98),
@@ -267,6 +325,11 @@ def test_constant_first_column_is_not_stored(plr, oracle, gen, n, d):
     with pytest.raises(PlrError) as e:
         plr.set_data(Xb, y)
     assert e.value.code == -1 and "row %d" % (n // 3) in str(e.value)
+    # the refused shard does not stay resident, half uploaded
+    assert plr.shape == (0, 0)
+    with pytest.raises(PlrError) as e:
+        plr.loss_grad(th)
+    assert e.value.code == -4  # PLR_ERR_NODATA
     # switched off again: the column is stored, same results to rounding
     plr.set_option("first_column_is_one", 0)
     plr.set_data(X, y)
@@ -278,19 +341,30 @@ def test_constant_first_column_is_not_stored(plr, oracle, gen, n, d):
 def test_wide_row_exchange_gives_up_instead_of_hanging(plr, oracle, gen):
     # a workgroup that never hears from its partners must not spin for ever: with the poll
     # limit at 0 every wait that does not find its partial at the first look gives up, the
-    # kernel runs to its end and the call reports the failure (a pass in which every first
-    # look happens to succeed is correct and also accepted)
+    # kernel runs to its end and -- with the fallback switched off -- the call reports the
+    # failure (a pass in which every first look happens to succeed is correct and also accepted)
     from paracel_amd import PlrError
 
     X, y, th = make(gen, 600, 20001)
     plr.set_data(X, y)
     assert "team_pass" in plr.kernel_info()
     g_ref = oracle.gsum(X, y, th)
+    plr.set_option("team_fallback", 0)
     plr.set_option("team_spin_limit", 0)
     try:
         g, _, _ = plr.loss_grad(th)
         assert rel(g, g_ref) <= GRAD_TOL
         print("every first look succeeded", flush=True)
+    except PlrError as e:
+        assert e.code == -2 and "gave up waiting" in str(e)
+    # several rounds enqueued back to back: a give-up in ANY of them must surface -- what may
+    # never come back is success with a theta that later rounds built on a discarded pass
+    alpha, beta = 0.1 / 600, 0.005
+    t_ref = oracle.train_dgd(X, y, np.zeros(20001), alpha, beta, 8)
+    try:
+        t8 = plr.train_dgd(np.zeros(20001), alpha, beta, 8)
+        assert rel(t8, t_ref) <= 1e-8
+        print("every first look of 8 rounds succeeded", flush=True)
     except PlrError as e:
         assert e.code == -2 and "gave up waiting" in str(e)
     # the context is usable again once the limit is back
@@ -299,6 +373,37 @@ def test_wide_row_exchange_gives_up_instead_of_hanging(plr, oracle, gen):
     assert rel(g, g_ref) <= GRAD_TOL
     with pytest.raises(PlrError):
         plr.set_option("no_such_option", 1)
+
+
+def test_a_wide_row_pass_that_gives_up_runs_again_in_two_sweeps(plr, oracle, gen):
+    # the default: a team pass whose workgroups are not all resident (other processes or
+    # streams on the compute units) is run again in two sweeps, which need no residency; the
+    # caller gets the shard's results either way, and after two such passes the shard stays on
+    # two sweeps.  Forced here from the host with the poll limit at 0.
+    X, y, th = make(gen, 600, 20001, seed=0xFA11)
+    plr.set_data(X, y)
+    assert "team_pass" in plr.kernel_info() and "gave up" not in plr.kernel_info()
+    g_ref = oracle.gsum(X, y, th)
+    l_ref = oracle.calc_loss_sum(X, y, th)
+    alpha, beta = 0.1 / 600, 0.005
+    t_ref = oracle.train_dgd(X, y, np.zeros(20001), alpha, beta, 8)
+    plr.set_option("team_spin_limit", 0)
+    for _ in range(3):
+        g, loss, _ = plr.loss_grad(th)
+        assert rel(g, g_ref) <= GRAD_TOL and abs(loss - l_ref) <= LOSS_TOL * l_ref
+        t8 = plr.train_dgd(np.zeros(20001), alpha, beta, 8)
+        assert rel(t8, t_ref) <= 1e-8
+        h = plr.predict(th)
+        assert np.max(np.abs(h - oracle.predict(X, th))) <= 1e-14
+    print(plr.kernel_info(), flush=True)
+    plr.set_option("team_spin_limit", 1 << 22)
+    g, loss, _ = plr.loss_grad(th)
+    assert rel(g, g_ref) <= GRAD_TOL and abs(loss - l_ref) <= LOSS_TOL * l_ref
+    # a fresh shard starts on the team path again
+    plr.set_data(X, y)
+    assert "team_pass" in plr.kernel_info() and "gave up" not in plr.kernel_info()
+    g, _, _ = plr.loss_grad(th)
+    assert rel(g, g_ref) <= GRAD_TOL
 
 
 NARROW = [(n, d) for d in (1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 48, 63, 64)

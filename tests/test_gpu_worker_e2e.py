@@ -213,6 +213,53 @@ def test_several_workers_share_the_gpu_and_the_server(server_info, oracle, tmp_p
     assert got_lines == n
 
 
+def test_two_workers_with_rows_wider_than_one_workgroup_holds(server_info, oracle, tmp_path):
+    # 20 000 features + bias: past 19 456 stored columns a row is shared by several
+    # workgroups.  The one-read pass needs its whole grid resident, which two processes on
+    # one GPU cannot count on, so workers that are not alone take the two-sweep pass
+    # (lr.cpp:143-145, update.cpp:26-32, prun.py:169-172: mpirun -n W)
+    W, n, k, rounds = 2, 600, 20000, 20
+    rng = np.random.default_rng(2026)
+    F = np.round(rng.normal(size=(n, k)) / np.sqrt(k), 6)
+    lab = (rng.random(n) < 0.5).astype(int)
+    train = tmp_path / "wide.csv"
+    np.savetxt(train, np.hstack([F, lab[:, None]]), fmt=["%.6f"] * k + ["%d"], delimiter=",")
+    cfgf = tmp_path / "cfg.json"
+    cfgf.write_text(json.dumps({
+        "training_input": str(train), "test_input": "", "predict_input": "",
+        "output": str(tmp_path / "out") + "/", "update_file": os.path.join(PKG, "liblr_update.so"),
+        "update_func": "lr_theta_update", "method": "dgd", "rounds": rounds,
+        "alpha": 0.5 / n, "beta": 0.005, "debug": False}))
+    procs = []
+    for r in range(W):
+        cmd = [os.path.join(PKG, "plr_lr_worker"), "--server_info", server_info, "--cfg_file",
+               str(cfgf), "--theta0", "zero", "--worker_id", str(r), "--worker_sz", str(W),
+               "--theta_out", str(tmp_path / "theta.bin")]
+        procs.append(subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                                      text=True))
+    outs = []
+    for p in procs:
+        try:
+            o, e = p.communicate(timeout=100)
+        except subprocess.TimeoutExpired:
+            for q in procs:
+                q.kill()
+            raise
+        assert p.returncode == 0, e
+        outs.append(o)
+    X = np.hstack([np.ones((n, 1)), F])
+    y = lab.astype(float)
+    theta_ref = oracle.train_dgd_workers(X, y, np.zeros(k + 1), 0.5 / n, 0.005, rounds, W)
+    theta = np.fromfile(tmp_path / "theta.bin")
+    assert theta.shape == (k + 1,) and rel(theta, theta_ref) <= 1e-8
+    want = oracle.calc_loss(X, y, theta_ref)
+    for o in outs:
+        assert "two sweeps" in o, o[-2000:]
+        loss_line = [ln for ln in o.splitlines() if ln.startswith("final loss:")][0]
+        assert abs(float(loss_line.split(":")[1]) - want) <= 1e-10
+        assert o.count("finished round:") == rounds
+
+
 def test_ridge_worker_end_to_end(server_info, oracle, tmp_path):
     # cfg keys and call order of ridge_driver.cpp:29-73; the batch trainer against the
     # oracle's batch form of ridge.hpp:79-84, loss / predictions against ridge.hpp:103-139

@@ -42,6 +42,13 @@ def unfield(b):
     return msgpack.unpackb(b[8:], raw=False)
 
 
+def unfield_raw(b):
+    """a framed field whose strings are byte blobs (stored values), left as bytes"""
+    (n,) = struct.unpack("=Q", b[:8])
+    assert len(b) == 8 + n
+    return msgpack.unpackb(b[8:], raw=True)
+
+
 class Zmq:
     def __init__(self):
         self.lib = C.CDLL("/opt/conda/lib/libzmq.so.5")
@@ -262,6 +269,46 @@ def test_worker_collectives_over_the_server_tables(W):
             out, err = q.communicate(timeout=60)
             assert q.returncode == 0, err
             assert out.strip() == "ok %d" % r
+        # 30 rounds = 91 barriers and 60 all-reduces per worker: the collectives' keys are
+        # per-worker counters and two value slots, so their number does not depend on how
+        # long the job ran (server.hpp:261-264 pullall: the whole table as one packed map)
+        host, ports = info.split(":")
+        z = Zmq()
+        try:
+            table = unfield_raw(z.req(host, ports.split(",")[0], field("pullall")))
+        finally:
+            z.close()
+        ours = sorted(k.decode() for k in table if k.startswith(b"plr_"))
+        want = [] if W == 1 else sorted(["plr_sync_%d" % r for r in range(W)] +
+                                        ["plr_ar_%d_%d" % (s, r) for s in (0, 1) for r in range(W)])
+        assert ours == want
     finally:
         p.kill()
         p.wait()
+
+
+def test_a_barrier_names_the_workers_that_never_arrive():
+    # a crashed or missing peer must end the job, not hang it: worker 0 of 3 alone
+    _need_host_binaries()
+    p, info = _start_server(True)
+    try:
+        env = dict(os.environ, PLR_SYNC_TIMEOUT_S="0.5")
+        r = subprocess.run([os.path.join(PKG, "plr_comm_check"), "--server_info", info,
+                            "--worker_id", "0", "--worker_sz", "3"], env=env,
+                           capture_output=True, text=True, timeout=60)
+        assert r.returncode == 1
+        assert "worker(s) 1, 2 did not arrive" in r.stderr, r.stderr
+    finally:
+        p.kill()
+        p.wait()
+
+
+def test_incr_int_does_not_create_a_key(server):
+    # kv.hpp:108-112 / server.hpp:136-153: incr on a missing key changes nothing (and is
+    # still answered with true); on an existing key it adds
+    z, host, ports, _ = server
+    assert unfield(z.req(host, ports[4], SEP.join([field("incr_int"), field("ghost"), field(1)]))) is True
+    assert z.req(host, ports[4], SEP.join([field("pull_int"), field("ghost")])) == b"nokey"
+    z.req(host, ports[4], SEP.join([field("push_int"), field("clock"), field(5)]))
+    z.req(host, ports[4], SEP.join([field("incr_int"), field("clock"), field(2)]))
+    assert unfield(z.req(host, ports[4], SEP.join([field("pull_int"), field("clock")]))) == 7
