@@ -105,7 +105,8 @@ PER_CONFIG = ["c1_dense_100k_x_100", "c3_tall_10m_x_256", "c4_wide_200k_x_16384"
 # Shapes beyond the five configurations, one per kernel family and layout, timed last in
 # a default run (GPU only) and reported under other_shapes.
 OTHER_SHAPES = ["x_narrow_30m_x_16", "x_narrow_10m_x_41", "x_short_30m_x_66",
-                "x_c1shape_20m_x_100", "x_bias_10m_x_257", "x_verywide_100k_x_32768"]
+                "x_c1shape_20m_x_100", "x_bias_10m_x_257", "x_verywide_100k_x_32768",
+                "x_wide_75k_x_20000", "x_wide_30k_x_50000"]
 
 # A one-GPU box gives a job 16 CPUs whatever os.cpu_count() shows there.
 CPU_SHARE = 16

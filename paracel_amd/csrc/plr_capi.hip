@@ -84,35 +84,19 @@ const pass_fn kBlockAxpy[2] = {
 // workgroup of a team owns one column block and the partial dot products are
 // exchanged per row.  [grad]
 typedef void (*team_fn)(plr::TeamArgs);
-// [grad][link / loss formula]; a gradient pass with the identity link always
-// carries the squared loss (plr_dgd_delta_linear), so that slot stays empty
 struct TeamFns {
-  team_fn fn[2][5];
+  team_fn grad[2];  // team_pass: [identity link]
+  team_fn dot;      // team_dot: the passes without a gradient
 };
 template <int NCH, int LAG>
 TeamFns make_team_fns() {
-  TeamFns f;
-#define PLR_TEAM(GRAD, LM) plr::team_pass<NCH, GRAD, plr::LM, LAG>
-  f.fn[0][0] = PLR_TEAM(false, kTeamLmReference);
-  f.fn[0][1] = PLR_TEAM(false, kTeamLmStable);
-  f.fn[0][2] = PLR_TEAM(false, kTeamLmNone);
-  f.fn[0][3] = PLR_TEAM(false, kTeamLmSquared);
-  f.fn[0][4] = PLR_TEAM(false, kTeamLmLinearNone);
-  f.fn[1][0] = PLR_TEAM(true, kTeamLmReference);
-  f.fn[1][1] = PLR_TEAM(true, kTeamLmStable);
-  f.fn[1][2] = PLR_TEAM(true, kTeamLmNone);
-  f.fn[1][3] = PLR_TEAM(true, kTeamLmSquared);
-  f.fn[1][4] = nullptr;
-#undef PLR_TEAM
-  return f;
+  return {{plr::team_pass<NCH, false, LAG>, plr::team_pass<NCH, true, LAG>}, plr::team_dot<NCH>};
 }
 // [chunks per wave - kTeamMinNch][lag - 1]
 const TeamFns kTeam[plr_plan::kTeamNch - plr_plan::kTeamMinNch + 1][2] = {
-    {make_team_fns<5, 1>(), make_team_fns<5, 2>()},
-    {make_team_fns<6, 1>(), make_team_fns<6, 2>()},
     {make_team_fns<7, 1>(), make_team_fns<7, 2>()},
     {make_team_fns<8, 1>(), make_team_fns<8, 2>()}};
-static_assert(plr_plan::kTeamMinNch == 5 && plr_plan::kTeamNch == 8 &&
+static_assert(plr_plan::kTeamMinNch == 7 && plr_plan::kTeamNch == 8 &&
                   plr_plan::kTeamWaves == plr::kTeamWaves,
               "one team kernel set per chunk count");
 constexpr int64_t kHostPredictCols = 192;  // from this pitch on predictions go straight to host
@@ -247,8 +231,8 @@ struct plr_ctx {
   // ... read once by teams of workgroups (team_blocks > 0), else in two sweeps
   int team_blocks = 0, team_blk_chunks = 0, team_blk_extra = 0, team_nch = 0, nteams = 0;
   const TeamFns* team_fns = nullptr;
-  int opt_team_lag = 1;      // plr_set_option("team_lag")
-  int opt_team_max_nch = 8;  // plr_set_option("team_max_chunks")
+  int opt_team_lag = 0;      // plr_set_option("team_lag"): 0 = by shape
+  int team_lag = 0;          // in force for the resident shard
   unsigned long long* d_zx = nullptr;  // [nteams][4][team_blocks][2] exchange slots, then the
                                        // status word of the pass
   int64_t zx_words = 0;
@@ -270,6 +254,9 @@ struct plr_ctx {
   int csv_slow_fields = 0;      // fields of the last plr_set_data_csv the host converted
   bool team_check = false;      // a team pass ran since the status word was last read
   double* d_z = nullptr;        // n: blocked rows only, x.theta accumulated over the blocks
+  double* d_zparts = nullptr;   // [team_blocks * 8][n]: team_dot's partial dot products
+  int64_t zstride = 0;          // entries per (wave, team) in d_zparts
+  int res_grid = 1;             // workgroups of residual_pass behind a team pass
   double* d_res = nullptr;      // n: blocked rows only, residual per row
   int64_t theta_len = 0;
   double* d_theta = nullptr;    // theta_len doubles, zero padded
@@ -349,6 +336,8 @@ void free_shape(plr_ctx* c) {
   c->part_rows = c->part_len = 0;
   c->base_info.clear();
   if (c->d_z) (void)hipFree(c->d_z);
+  if (c->d_zparts) (void)hipFree(c->d_zparts);
+  c->d_zparts = nullptr;
   if (c->d_res) (void)hipFree(c->d_res);
   if (c->d_train_out) (void)hipFree(c->d_train_out);
   if (c->h_theta) (void)hipHostFree(c->h_theta);
@@ -391,7 +380,7 @@ int size_sweep_grid(plr_ctx* c, int64_t n) {
 // n x d shard.
 int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   plr_plan::Plan pl;
-  if (!plr_plan::plan_width(d, pl, n, c->opt_team_max_nch))
+  if (!plr_plan::plan_width(d, pl, n))
     return fail(c, PLR_ERR_UNSUPPORTED, "no kernel variant covers this width");
   c->pitch = pl.pitch;
   c->theta_len = pl.theta_len;
@@ -457,16 +446,16 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
       // one read of X: teams of team_blocks workgroups, all resident at once.
       // Any of the instances may be launched on this shard, so the grid is
       // sized to the one that fits the fewest workgroups on a compute unit.
-      const TeamFns* tf = &kTeam[pl.team_nch - plr_plan::kTeamMinNch][c->opt_team_lag - 1];
+      const int lag = c->opt_team_lag ? c->opt_team_lag : pl.team_lag;
+      const TeamFns* tf = &kTeam[pl.team_nch - plr_plan::kTeamMinNch][lag - 1];
+      // (team_dot needs no residency; it runs on the same grid)
       int tocc = 1 << 30;
-      for (int g = 0; g < 2; ++g)
-        for (int lm = 0; lm < 5; ++lm) {
-          if (!tf->fn[g][lm]) continue;
-          int o = 0;
-          PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                         &o, reinterpret_cast<const void*>(tf->fn[g][lm]), threads, 0));
-          if (o < tocc) tocc = o;
-        }
+      for (int k = 0; k < 2; ++k) {
+        int o = 0;
+        PLR_HIP(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                       &o, reinterpret_cast<const void*>(tf->grad[k]), threads, 0));
+        if (o < tocc) tocc = o;
+      }
       const int nteams = tocc * c->num_cu / pl.team_blocks;
       if (nteams >= 1) {
         c->team_fns = tf;
@@ -474,6 +463,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
         c->team_blk_chunks = pl.team_blk_chunks;
         c->team_blk_extra = pl.team_blk_extra;
         c->team_nch = pl.team_nch;
+        c->team_lag = lag;
         c->nteams = nteams;
         c->grid = c->grid_nograd = c->nteams * c->team_blocks;
         c->zx_words = (int64_t)c->nteams * plr::kTeamSlots * c->team_blocks * 2;
@@ -481,7 +471,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
         snprintf(b, sizeof b,
                  "team_pass<NCH=%d,LAG=%d> %d column blocks of %d%s chunks, %d teams, pitch=%lld "
                  "grid=%d x %d threads (occupancy %d blocks/CU, %d CUs)",
-                 c->team_nch, c->opt_team_lag, c->team_blocks, c->team_blk_chunks,
+                 c->team_nch, c->team_lag, c->team_blocks, c->team_blk_chunks,
                  c->team_blk_extra ? "-" : "", c->nteams, (long long)c->pitch, c->grid, threads,
                  tocc, c->num_cu);
         c->info = b;
@@ -576,7 +566,9 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
   PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)(c->theta_len + 8) * sizeof(double)));
   // a team shares one row of gradient partials
   c->part_rows = c->team_blocks > 0 ? c->nteams : c->grid;
-  c->part_len = gmax;
+  // behind a team pass residual_pass folds the row terms: a thread per row
+  c->res_grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n, 256), 2 * c->num_cu));
+  c->part_len = std::max(gmax, c->res_grid);
   PLR_HIP(c, hipMalloc(&c->d_part_res, (size_t)c->part_len * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_g, (size_t)c->part_rows * c->pitch * sizeof(double)));
   PLR_HIP(c, hipMalloc(&c->d_part_loss, (size_t)c->part_len * sizeof(double)));
@@ -586,6 +578,11 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
     PLR_HIP(c, hipMalloc(&c->d_zx, (size_t)(c->zx_words + 1) * sizeof(unsigned long long)));
     PLR_HIP(c, hipMemsetAsync(c->d_zx, 0, (size_t)(c->zx_words + 1) * sizeof(unsigned long long),
                               c->stream));
+    // z per row (team_pass), and every wave's partial of it (team_dot)
+    PLR_HIP(c, hipMalloc(&c->d_z, (size_t)std::max<int64_t>(n, 1) * sizeof(double)));
+    c->zstride = ceil_div(ceil_div(std::max<int64_t>(n, 1), c->nteams), plr::kWave) * plr::kWave;
+    PLR_HIP(c, hipMalloc(&c->d_zparts, (size_t)c->zstride * c->nteams * c->team_blocks *
+                                           plr::kTeamWaves * sizeof(double)));
   } else if (c->blocked && n > 0) {
     PLR_HIP(c, hipMalloc(&c->d_z, (size_t)n * sizeof(double)));
     PLR_HIP(c, hipMalloc(&c->d_res, (size_t)n * sizeof(double)));
@@ -647,8 +644,13 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   const Shape* v = c->var;
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
   const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
-  const bool team = c->team_blocks > 0 && !c->team_off;
-  const int grid = (c->blocked && !team) ? c->sweep_grid : grad ? c->grid : c->grid_nograd;
+  // rows shared by a team of workgroups: with a gradient the one-read pass with
+  // its exchange (unless switched off), without one the exchange-free team_dot
+  const bool team = c->team_blocks > 0 && !c->team_off && grad;
+  const bool team_dot = c->team_blocks > 0 && !grad;
+  const int grid = (c->blocked && !team && !team_dot) ? c->sweep_grid
+                   : grad                             ? c->grid
+                                                      : c->grid_nograd;
   const int threads = c->lane ? plr::kWave * c->lane->wrow * c->lane->wcol
                       : c->pair ? plr::kWave * c->pair->wrow
                                 : plr::kWave * v->wcol * v->wrow;
@@ -686,20 +688,12 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     hipLaunchKernelGGL(c->fns->fn[grad ? 1 : 0][c->allch ? 1 : 0], dim3(grid), dim3(threads), 0,
                        c->stream, pa);
     PLR_HIP(c, hipGetLastError());
-  } else if (team) {
-    // the exchange slots start at zero (sequence number 0 = empty).  The status
-    // word behind them is NOT cleared here: a give-up in any pass of a chain of
-    // passes enqueued back to back must still be there when the host looks.
-    hipLaunchKernelGGL(plr::fill_zero, dim3(16), dim3(256), 0, c->stream,
-                       reinterpret_cast<double*>(c->d_zx), c->zx_words);
-    PLR_HIP(c, hipGetLastError());
+  } else if (team || team_dot) {
     plr::TeamArgs ta;
     ta.X = c->dX;
     ta.y = pa.y;
     ta.theta = c->d_theta;
     ta.part_g = c->d_part_g;
-    ta.part_loss = c->d_part_loss;
-    ta.h_out = pa.h_out;
     ta.n = c->n;
     ta.pitch = c->pitch;
     ta.nblk = c->team_blocks;
@@ -707,18 +701,38 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     ta.blk_chunks = c->team_blk_chunks;
     ta.blk_extra = c->team_blk_extra;
     ta.theta_bias = pa.theta_bias;
-    ta.part_res = pa.part_res;
     ta.zeros = c->d_theta + c->theta_len - plr::kChunkCols;  // the padding never changes
     ta.zx = c->d_zx;
     ta.status = reinterpret_cast<unsigned*>(c->d_zx + c->zx_words);
     ta.spin_limit = c->team_spin_limit;
-    const int lm = pa.identity_link ? (pa.loss_mode == plr::kLossSquared ? plr::kTeamLmSquared
-                                                                         : plr::kTeamLmLinearNone)
-                                    : (int)pa.loss_mode;  // kLossReference/Stable/None = 0/1/2
-    hipLaunchKernelGGL(c->team_fns->fn[grad ? 1 : 0][lm], dim3(grid), dim3(threads), 0, c->stream,
-                       ta);
+    int zparts = 0;
+    if (grad) {
+      // the exchange slots start at zero (sequence number 0 = empty).  The status
+      // word behind them is NOT cleared here: a give-up in any pass of a chain of
+      // passes enqueued back to back must still be there when the host looks.
+      hipLaunchKernelGGL(plr::fill_zero, dim3(16), dim3(256), 0, c->stream,
+                         reinterpret_cast<double*>(c->d_zx), c->zx_words);
+      PLR_HIP(c, hipGetLastError());
+      ta.z_out = c->d_z;
+      ta.zstride = 0;
+      hipLaunchKernelGGL(c->team_fns->grad[pa.identity_link], dim3(c->grid), dim3(threads), 0,
+                         c->stream, ta);
+      PLR_HIP(c, hipGetLastError());
+      c->team_check = true;
+    } else {
+      // no gradient: every wave's partial dot products, no exchange
+      ta.z_out = c->d_zparts;
+      ta.zstride = c->zstride;
+      zparts = c->team_blocks;
+      hipLaunchKernelGGL(c->team_fns->dot, dim3(c->grid), dim3(threads), 0, c->stream, ta);
+      PLR_HIP(c, hipGetLastError());
+    }
+    // z -> loss terms, predictions, sum of the residuals
+    hipLaunchKernelGGL(plr::residual_pass, dim3(c->res_grid), dim3(256), 0, c->stream,
+                       (const double*)ta.z_out, (const double*)pa.y, (double*)nullptr, pa.h_out,
+                       c->d_part_loss, c->n, pa.loss_mode, pa.identity_link, pa.theta_bias,
+                       pa.part_res, zparts, c->nteams, c->zstride);
     PLR_HIP(c, hipGetLastError());
-    c->team_check = true;
   } else if (c->n > 0) {
     // sweep 1: z = x.theta, one launch per column block, accumulated in d_z
     pa.z_buf = c->d_z;
@@ -740,7 +754,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     hipLaunchKernelGGL(plr::residual_pass, dim3(grid), dim3(256), 0, c->stream,
                        (const double*)c->d_z, (const double*)pa.y, grad ? c->d_res : nullptr,
                        pred_out, c->d_part_loss, c->n, pa.loss_mode,
-                       pa.identity_link, pa.theta_bias, pa.part_res);
+                       pa.identity_link, pa.theta_bias, pa.part_res, 0, 0, (int64_t)0);
     PLR_HIP(c, hipGetLastError());
     // sweep 2: rank-1 updates, block by block
     if (grad) {
@@ -780,7 +794,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     fa.part_res = pa.part_res;
     fa.theta_bias = c->d_theta + c->bias_slot;
     fa.nparts = team ? c->nteams : grid;  // a team shares one row of partials
-    fa.nparts_loss = fa.nparts;
+    fa.nparts_loss = (team || team_dot) ? c->res_grid : grid;
     fa.delta_mode = (kind == kPassDelta) ? (train_round >= 0 ? 2 : 1) : 0;
     fa.have_grad = grad ? 1 : 0;
     fa.alpha = alpha;
@@ -847,10 +861,8 @@ int fall_back_to_two_sweeps(plr_ctx* c) {
     const int rc = size_sweep_grid(c, c->n);
     if (rc != PLR_OK) return rc;
   }
-  if (!c->d_z && c->n > 0) {
-    PLR_HIP(c, hipMalloc(&c->d_z, (size_t)c->n * sizeof(double)));
+  if (!c->d_res && c->n > 0)  // (d_z exists: the team pass stores z there too)
     PLR_HIP(c, hipMalloc(&c->d_res, (size_t)c->n * sizeof(double)));
-  }
   if (c->part_rows < c->sweep_grid) {
     PLR_HIP(c, hipFree(c->d_part_g));
     c->d_part_g = nullptr;
@@ -1772,14 +1784,8 @@ int plr_set_option(plr_ctx* c, const char* key, int64_t value) {
     return PLR_OK;
   }
   if (strcmp(key, "team_lag") == 0) {
-    if (value < 1 || value > 2) return fail(c, PLR_ERR_INVALID, "team_lag is 1 or 2");
+    if (value < 0 || value > 2) return fail(c, PLR_ERR_INVALID, "team_lag is 0 (by shape), 1 or 2");
     c->opt_team_lag = (int)value;  // takes effect at the next plr_set_data / plr_alloc_data
-    return PLR_OK;
-  }
-  if (strcmp(key, "team_max_chunks") == 0) {
-    if (value < plr_plan::kTeamMinNch || value > plr_plan::kTeamNch)
-      return fail(c, PLR_ERR_INVALID, "team_max_chunks out of range");
-    c->opt_team_max_nch = (int)value;  // takes effect at the next plr_set_data / plr_alloc_data
     return PLR_OK;
   }
   if (strcmp(key, "team_fallback") == 0) {

@@ -1112,6 +1112,14 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void pair_pass(PassArgs a) {
 // polls, raises status[0], and every workgroup then runs to its end without
 // waiting -- the host reports the pass as failed.
 //
+// What leaves the kernel besides the gradient partials is z = x.theta of every
+// row (z_out): the loss terms, the predictions and the sum of the residuals are
+// produced from z by residual_pass, which costs 16 bytes per row against the
+// row's 8 * d -- so the kernel carries no log, no loss formula and no
+// prediction store, only the link (the sigmoid's exp and division, or
+// nothing).  The passes without a gradient need no exchange at all: team_dot
+// below.
+//
 // Same reference loops as shard_pass (lr.cpp:69-72,132-138,322-330,361-363).
 constexpr int kTeamWaves = 8;
 constexpr int kTeamSlots = 8;  // >= 2 * LAG + 2 for LAG <= 2, a power of two
@@ -1123,8 +1131,10 @@ struct TeamArgs {
   const double* theta;       // zero-padded to nblk * blk_chunks * 128 entries
   const double* zeros;       // 128 doubles of zeros (what an unowned chunk slot reads)
   double* part_g;            // [nteams][pitch]
-  double* part_loss;         // [nteams]
-  double* h_out;             // n, or nullptr
+  double* z_out;             // team_pass: n, x.theta per row (without theta_bias);
+                             // team_dot: [nblk * 8][nteams][zstride], every wave's
+                             // partial of it, a team's rows side by side
+  int64_t zstride;           // team_dot: entries per (wave, team), a multiple of 64
   int64_t n, pitch;
   int nblk;                  // B: column blocks = workgroups per team (<= kTeamMaxBlocks)
   int nteams;                // grid = nteams * nblk
@@ -1135,24 +1145,12 @@ struct TeamArgs {
   int blk_chunks;
   int blk_extra;
   const double* theta_bias;  // as in PassArgs
-  double* part_res;          // [nteams], or nullptr
   unsigned long long* zx;    // [nteams][kTeamSlots][nblk][2] exchange slots
   unsigned* status;          // [0]: set when a wait gave up
   unsigned spin_limit;
 };
 
-// the link / loss formula as a compile-time constant: the loop then carries
-// the polynomial coefficients of one formula instead of all of them (they are
-// hoisted into registers, two per coefficient)
-enum : int {
-  kTeamLmReference = 0,   // sigmoid, -log h / -log(1-h)
-  kTeamLmStable = 1,      // sigmoid, log1p(exp(-|z|)) form
-  kTeamLmNone = 2,        // sigmoid, no loss
-  kTeamLmSquared = 3,     // identity link, (z - y)^2
-  kTeamLmLinearNone = 4,  // identity link, no loss
-};
-
-template <int NCH, bool GRAD, int LM, int LAG>
+template <int NCH, bool IDENT, int LAG>
 __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
   static_assert(LAG == 1 || LAG == 2, "a row's update follows its dot product by 1 or 2 steps");
   static_assert(kTeamSlots >= 2 * LAG + 2 && (kTeamSlots & (kTeamSlots - 1)) == 0, "slot ring");
@@ -1160,11 +1158,6 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
   // t + 2 in flight as well -- was measured and is 0.5-1 % slower at every
   // width: the step does not wait for data once the waits below are right.)
   constexpr int D = LAG + 2;
-  constexpr unsigned kLoss = LM == kTeamLmReference ? kLossReference
-                             : LM == kTeamLmStable  ? kLossStable
-                             : LM == kTeamLmSquared ? kLossSquared
-                                                    : kLossNone;
-  constexpr int kIdentity = (LM == kTeamLmSquared || LM == kTeamLmLinearNone) ? 1 : 0;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   // A team is nblk consecutive workgroups.  Consecutive workgroup ids go to
@@ -1201,7 +1194,6 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
     const double* tp = (c < my_nch) ? a.theta + (c0 + c) * kChunkCols : a.zeros;
     thl[c * kWave] = *reinterpret_cast<const v2d*>(tp + 2 * lane);
   }
-  double loss_acc = 0., res_acc = 0.;
   const double bias = a.theta_bias ? *a.theta_bias : 0.;
   bool gave_up = false;
 
@@ -1308,23 +1300,17 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
     }
     __syncthreads();
     if (have_prev) {
-      const int64_t row = prev_row;
-      double z = bias;
+      double z = 0.;
       for (int b = 0; b < a.nblk; ++b) z += zp[par][b];
-      double h, l;
-      row_terms(z, yv, kLoss, kIdentity, h, l);
+      if (blk == 0 && threadIdx.x == 0) a.z_out[prev_row] = z;
+      // lr.cpp:69-72 / ridge.hpp:79: the model's output, then the residual
+      double h = z + bias;
+      if (!IDENT) h = 1. / (1. + exp(-h));
       const double res = h - yv;
-      if (blk == 0 && threadIdx.x == 0) {
-        loss_acc += l;
-        res_acc += res;
-        if (a.h_out) store_h(a.h_out + row, h);
-      }
-      if (GRAD) {
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) {
-          acc[c].x = fma(res, X[PREV][c].x, acc[c].x);
-          acc[c].y = fma(res, X[PREV][c].y, acc[c].y);
-        }
+      for (int c = 0; c < NCH; ++c) {
+        acc[c].x = fma(res, X[PREV][c].x, acc[c].x);
+        acc[c].y = fma(res, X[PREV][c].y, acc[c].y);
       }
     }
   };
@@ -1358,16 +1344,99 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
     }
   }
 
-  if (GRAD) {
-    double* out = a.part_g + (int64_t)team * a.pitch + c0 * kChunkCols + 2 * lane;
+  double* out = a.part_g + (int64_t)team * a.pitch + c0 * kChunkCols + 2 * lane;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c)
-      if (c < my_nch && (c != ragged_c || lane_in_ragged))
-        *reinterpret_cast<v2d*>(out + (int64_t)c * kChunkCols) = acc[c];
+  for (int c = 0; c < NCH; ++c)
+    if (c < my_nch && (c != ragged_c || lane_in_ragged))
+      *reinterpret_cast<v2d*>(out + (int64_t)c * kChunkCols) = acc[c];
+}
+
+// The passes over such rows that carry no gradient (loss only, predictions)
+// need nothing from a row but z = x.theta, and no workgroup needs another
+// one's share of it: same split of the row over teams of workgroups and their
+// waves, but every wave just streams its chunks of its team's rows and stores
+// its partial dot products -- kept in the lanes for 64 rows, then written as one
+// dense 512-byte store to z_out[((blk * 8 + wave) * nteams + team) * zstride + i],
+// i counting the team's rows.  No exchange, no barrier, no residency
+// requirement.  residual_pass adds a row's partials --
+// first over the waves of a block, then over the blocks, the order team_pass
+// adds them in, so both give the same bits -- and turns z into loss terms and
+// predictions.  Three row buffers rotate: rows t + 1 and t + 2 are in flight
+// while row t is summed.
+template <int NCH>
+__global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_dot(TeamArgs a) {
+  constexpr int D = 3;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int blk = (int)(blockIdx.x % a.nblk);
+  const int team = (int)(blockIdx.x / a.nblk);
+  const int64_t total_chunks = (a.pitch + kChunkCols - 1) / kChunkCols;
+  const int blk_m = a.blk_chunks + (blk < a.blk_extra ? 1 : 0);
+  const int64_t blk_c0 = (int64_t)blk * a.blk_chunks + (blk < a.blk_extra ? blk : a.blk_extra);
+  const int wq = blk_m / kTeamWaves, wrem = blk_m % kTeamWaves;
+  const int my_nch = wq + (wave < wrem ? 1 : 0);
+  const int64_t c0 = blk_c0 + (int64_t)wave * wq + (wave < wrem ? wave : wrem);
+  const int rag_cols = (int)(a.pitch % kChunkCols);
+  const int ragged_c =
+      (rag_cols != 0 && my_nch > 0 && c0 + my_nch == total_chunks) ? my_nch - 1 : -1;
+  const bool lane_in_ragged = 2 * lane < rag_cols;
+
+  v2d th[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const double* tp = (c < my_nch) ? a.theta + (c0 + c) * kChunkCols : a.zeros;
+    th[c] = *reinterpret_cast<const v2d*>(tp + 2 * lane);
+    if (c == ragged_c && !lane_in_ragged) th[c] = v2d{0., 0.};
   }
-  if (blk == 0 && threadIdx.x == 0) {
-    a.part_loss[team] = loss_acc;
-    if (a.part_res) a.part_res[team] = res_acc;
+  const char* xwave = reinterpret_cast<const char*>(a.X + c0 * kChunkCols);
+  const char* zeros = reinterpret_cast<const char*>(a.zeros);
+  const uint32_t lane_off = (uint32_t)(lane * sizeof(v2d));
+  const int64_t row_bytes = a.pitch * (int64_t)sizeof(double);
+  const int64_t myrows = a.n > team ? (a.n - team + a.nteams - 1) / a.nteams : 0;
+  double* zmine = a.z_out + ((int64_t)(blk * kTeamWaves + wave) * a.nteams + team) * a.zstride;
+  double keep = 0.;  // lane j: this wave's partial of the team's row 64 * (t / 64) + j
+
+  v2d X[D][NCH];
+  // unconditional loads, as in team_pass: past the last row the last row again
+  auto request = [&](int64_t i, v2d (&buf)[NCH]) {
+    if (i >= myrows) i = myrows - 1;
+    const char* rp = xwave + (team + i * a.nteams) * row_bytes;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const char* base = (c < my_nch) ? rp + c * (int)(kChunkCols * sizeof(double)) : zeros;
+      buf[c] = load_x(reinterpret_cast<const v2d*>(base + lane_off));
+    }
+  };
+  auto step = [&](int64_t t, auto phase_tag) {
+    constexpr int PH = decltype(phase_tag)::value;  // t mod 3
+    request(t + 2, X[(PH + 2) % D]);
+    asm volatile("" ::: "memory");
+    // the ragged chunk's lanes past the row end hold the next row's bytes: their
+    // theta is zero, but a non-finite neighbour must not turn 0 * x into NaN
+    double s0 = 0., s1 = 0.;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const bool drop = (c == ragged_c) && !lane_in_ragged;
+      s0 = fma(drop ? 0. : X[PH][c].x, th[c].x, s0);
+      s1 = fma(drop ? 0. : X[PH][c].y, th[c].y, s1);
+    }
+    const double wsum = wave_sum(s0 + s1);
+    if (lane == (int)(t & (kWave - 1))) keep = wsum;
+    if ((t & (kWave - 1)) == kWave - 1 || t == myrows - 1)  // uniform; zstride covers whole groups
+      zmine[(t & ~(int64_t)(kWave - 1)) + lane] = keep;
+  };
+  if (myrows > 0) {
+    request(0, X[0]);
+    request(1, X[1]);
+    int64_t t = 0;
+#pragma clang loop unroll(disable)
+    for (; t + 3 <= myrows; t += 3) {
+      step(t, std::integral_constant<int, 0>{});
+      step(t + 1, std::integral_constant<int, 1>{});
+      step(t + 2, std::integral_constant<int, 2>{});
+    }
+    if (t < myrows) step(t++, std::integral_constant<int, 0>{});
+    if (t < myrows) step(t++, std::integral_constant<int, 1>{});
   }
 }
 
@@ -1392,10 +1461,16 @@ __global__ __launch_bounds__(256) void read_probe(const v2d* base, int64_t ntile
   if (acc.x + acc.y == 1.2345e300) sink[0] = acc.x;  // keeps the loads alive
 }
 
-// Between the two sweeps of a column-blocked row: z (complete dot products)
-// -> h, residual and loss per row.  One thread per row, grid-stride; each
-// thread adds its rows' loss terms in row order, the workgroup folds them in
-// a fixed order into part_loss[block].
+// z = x.theta of every row -> h, residual, loss term, prediction.  Runs between
+// the two sweeps of a column-blocked row and behind a team pass.  One thread
+// per row, grid-stride; each thread adds its rows' loss terms in the order it
+// meets them, the workgroup folds them in a fixed order into part_loss[block]
+// (and the residuals into part_res[block]: the gradient of a constant first
+// column that is not stored).
+// zparts > 0: z[] holds team_dot's partial dot products, [zparts * 8][nteams]
+// [zstride], entry i of team m belonging to row m + i * nteams; the threads then
+// walk (team, i) so that their reads of z are dense, and a row's z is the sum
+// over the zparts groups of the sums over each group's 8 waves, in that order.
 __global__ __launch_bounds__(256) void residual_pass(const double* __restrict__ z,
                                                      const double* __restrict__ y,
                                                      double* __restrict__ res,
@@ -1403,14 +1478,32 @@ __global__ __launch_bounds__(256) void residual_pass(const double* __restrict__ 
                                                      double* __restrict__ part_loss, int64_t n,
                                                      unsigned loss_mode, int identity_link,
                                                      const double* __restrict__ theta_bias,
-                                                     double* __restrict__ part_res) {
+                                                     double* __restrict__ part_res, int zparts,
+                                                     int nteams, int64_t zstride) {
   const double bias = theta_bias ? *theta_bias : 0.;
   RowSums sums;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
-       i += (int64_t)gridDim.x * blockDim.x) {
+  const int64_t count = zparts > 0 ? (int64_t)nteams * zstride : n;
+  for (int64_t q = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; q < count;
+       q += (int64_t)gridDim.x * blockDim.x) {
+    int64_t i = q;
+    double zi;
+    if (zparts > 0) {
+      i = q / zstride + (q % zstride) * nteams;
+      if (i >= n) continue;
+      zi = 0.;
+      for (int b = 0; b < zparts; ++b) {
+        const double* zp = z + (int64_t)b * kTeamWaves * count + q;
+        double zb = 0.;
+#pragma unroll
+        for (int w = 0; w < kTeamWaves; ++w) zb += zp[(int64_t)w * count];
+        zi += zb;
+      }
+    } else {
+      zi = z[i];
+    }
     const double yv = y ? y[i] : 0.;
     double h, l;
-    row_terms(z[i] + bias, yv, loss_mode, identity_link, h, l);
+    row_terms(zi + bias, yv, loss_mode, identity_link, h, l);
     if (res) res[i] = h - yv;
     if (h_out) store_h(h_out + i, h);
     sums.loss += l;

@@ -17,8 +17,8 @@ constexpr int kBlkNch = 16, kBlkWcol = 8;
 constexpr int64_t kBlockCols = (int64_t)kBlkNch * kBlkWcol * kChunkCols;  // 16384
 constexpr int kMaxTeamBlocks = 64;       // column blocks a team of workgroups may span
 constexpr int kTeamWaves = 8;            // waves of a team's workgroup, side by side
-constexpr int kTeamMinNch = 5;           // chunks per wave the team kernel is built for: from ...
-constexpr int kTeamNch = 8;              // ... to
+constexpr int kTeamMinNch = 7;           // chunks per wave the team kernels are built for: from ...
+constexpr int kTeamNch = 8;              // ... to (rows past 19456 columns never need fewer than 7)
 constexpr int kAlwaysOneWave = 16;       // up to here no several-waves variant is considered
 constexpr int kMaxRowChunks = 32;        // widest one-wave row
 
@@ -57,6 +57,7 @@ struct Plan {
   int team_blk_chunks;
   int team_blk_extra;
   int team_nch;
+  int team_lag;       // steps between a row's dot product and its update (1 or 2)
 };
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -66,10 +67,8 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // n: rows of the shard when known (< 0: unknown, taken as large).  Where the
 // variant table has two entries for a shape, shards below kSmallShardBytes
 // take the one with the shorter tiles.
-// team_max_nch: the most chunks a wave of a team pass may own (kTeamMinNch ..
-// kTeamNch); fewer chunks per wave mean more workgroups per row.
 constexpr int64_t kSmallShardBytes = 1500000000;
-inline bool plan_width(int64_t d, Plan& p, int64_t n = -1, int team_max_nch = kTeamNch) {
+inline bool plan_width(int64_t d, Plan& p, int64_t n = -1) {
   p = Plan();
   p.variant = -1;
   if (d <= kMaxLaneCols) {
@@ -95,16 +94,21 @@ inline bool plan_width(int64_t d, Plan& p, int64_t n = -1, int team_max_nch = kT
     // the row's chunks dealt evenly to the fewest workgroups that can hold
     // them, and inside a workgroup evenly to its waves
     const int64_t chunks = ceil_div(p.pitch, kChunkCols);
-    if (team_max_nch < kTeamMinNch) team_max_nch = kTeamMinNch;
-    if (team_max_nch > kTeamNch) team_max_nch = kTeamNch;
-    const int64_t blocks = ceil_div(chunks, (int64_t)kTeamWaves * team_max_nch);
+    const int64_t blocks = ceil_div(chunks, (int64_t)kTeamWaves * kTeamNch);
     if (blocks <= kMaxTeamBlocks) {
       p.team_blocks = (int)blocks;
       p.team_blk_chunks = (int)(chunks / blocks);
       p.team_blk_extra = (int)(chunks % blocks);
       const int64_t widest = p.team_blk_chunks + (p.team_blk_extra ? 1 : 0);
-      p.team_nch = (int)ceil_div(widest, kTeamWaves);
+      p.team_nch = (int)ceil_div(widest, kTeamWaves);  // 7 or 8: more than 152 chunks in >= 3 blocks
       if (p.team_nch < kTeamMinNch) p.team_nch = kTeamMinNch;
+      // How many steps a row's update trails its dot product.  Two steps hide the
+      // exchange of the partial dots better (measured on 12 GB shards: +1-3 % up
+      // to 8 blocks, +6-10 % from 10 blocks on) but cost a fourth row buffer;
+      // where every wave owns all 8 chunks and the team is small that buffer
+      // fills the register file and one step is 2 % faster.
+      const bool full = chunks == blocks * kTeamWaves * kTeamNch;
+      p.team_lag = (full && blocks <= 8) ? 1 : 2;
     }
     // one more chunk of padding: the page of zeros an unowned chunk slot reads
     p.theta_len += kChunkCols;

@@ -31,6 +31,7 @@ static void check_team(const Plan& p, int64_t d, int cap) {
   // the blocks cover the row exactly, and no wave owns more chunks than the kernel holds
   CHECK((int64_t)p.team_blocks * p.team_blk_chunks + p.team_blk_extra == chunks, d);
   CHECK(p.team_nch >= kTeamMinNch && p.team_nch <= cap, d);
+  CHECK(p.team_lag == 1 || p.team_lag == 2, d);
   CHECK(ceil_div(p.team_blk_chunks + (p.team_blk_extra ? 1 : 0), kTeamWaves) <= p.team_nch, d);
   CHECK(p.team_blk_chunks >= kTeamWaves, d);  // every wave owns a chunk
   int64_t next = 0;
@@ -66,8 +67,8 @@ static void print_plan(int64_t d, int64_t n) {
            (int)p.allch, p.tail_cols);
   }
   if (p.path == kPathBlocked)
-    printf(" team_blocks=%d blk_chunks=%d(+1 in the first %d) nch=%d", p.team_blocks,
-           p.team_blk_chunks, p.team_blk_extra, p.team_nch);
+    printf(" team_blocks=%d blk_chunks=%d(+1 in the first %d) nch=%d lag=%d", p.team_blocks,
+           p.team_blk_chunks, p.team_blk_extra, p.team_nch, p.team_lag);
   printf("\n");
 }
 
@@ -83,14 +84,6 @@ int main(int argc, char** argv) {
   for (int64_t dn = 2; dn <= 2 * kMaxD + 1; ++dn) {
     const int64_t d = dn / 2, n = (dn & 1) ? 1 : -1;
     Plan p;
-    if (d > kMaxFusedCols && n < 0) {
-      // the team split for every cap on the chunks per wave
-      for (int cap = kTeamMinNch; cap < kTeamNch; ++cap) {
-        Plan q;
-        CHECK(plan_width(d, q, n, cap), d);
-        check_team(q, d, cap);
-      }
-    }
     if (!plan_width(d, p, n)) {
       CHECK(false && "plan_width failed", d);
       continue;

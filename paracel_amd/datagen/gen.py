@@ -178,6 +178,11 @@ def configs():
         # wider than the widest one-workgroup kernel: column blocks, a team of workgroups per row
         "x_verywide_100k_x_32768": Config("x_verywide_100k_x_32768", 100_000, 32768, 0x5EED0006,
                                           NORMAL, 1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),
+        # ... on dense data, at widths that do not fill the workgroups of a team evenly
+        "x_wide_75k_x_20000": Config("x_wide_75k_x_20000", 75_000, 20000, 0x5EED000E, NORMAL,
+                                     1.0 / np.sqrt(20000), lam=0.01),
+        "x_wide_30k_x_50000": Config("x_wide_30k_x_50000", 30_000, 50000, 0x5EED000F, NORMAL,
+                                     1.0 / np.sqrt(50000), lam=0.01),
         # end-to-end through the host parameter server
         "c5_e2e_2m_x_512": Config("c5_e2e_2m_x_512", 2_000_000, 512, 0x5EED0005, NORMAL,
                                   1.0 / np.sqrt(512), lam=0.01, theta0_zero=True),

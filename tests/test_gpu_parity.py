@@ -328,7 +328,7 @@ def test_constant_first_column_is_not_stored(plr, oracle, gen, n, d):
     # the refused shard does not stay resident, half uploaded
     assert plr.shape == (0, 0)
     with pytest.raises(PlrError) as e:
-        plr.loss_grad(th)
+        plr.loss_grad(np.zeros(0))
     assert e.value.code == -4  # PLR_ERR_NODATA
     # switched off again: the column is stored, same results to rounding
     plr.set_option("first_column_is_one", 0)
