@@ -10,6 +10,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <functional>
 #include <mutex>
 #include <string>
@@ -26,6 +27,16 @@ struct CopyPiece {  // bytes of pageable host memory and where on the device the
   const void* src;
   size_t bytes;
 };
+// Host memory moves to and from the device through kCopyLanes lanes of pinned
+// staging blocks (see lanes_in / copy_rows_out below).
+constexpr int kCopyLanes = 8;
+constexpr size_t kCopyBlock = 4u << 20;
+struct InJob {  // one staging block's worth of bytes and where on the device they go
+  void* dev;
+  size_t bytes;
+};
+using FillFn = std::function<bool(size_t job, char* blk)>;
+using SentFn = std::function<hipError_t(size_t job, hipStream_t st)>;
 static int copy_bytes_in(plr_ctx* c, const std::vector<CopyPiece>& pieces);
 static int copy_rows_in(plr_ctx* c, int64_t row0, int64_t nrows, const double* X, int64_t ldx);
 
@@ -249,6 +260,7 @@ struct plr_ctx {
   int64_t part_len = 0;           // entries of d_part_loss and d_part_res
   std::string base_info;          // kernel description without the give-up note
   bool opt_two_sweeps = false;  // plr_set_option("column_blocks_two_sweeps")
+  bool opt_csv_overlap = false;  // plr_set_option("csv_overlap")
   bool synth_first_col = false; // the shard being reserved comes from plr_set_data_csv
   int opt_csv_lane_rows = -1;   // plr_set_option("csv_lane_per_row"): -1 by row count, 0, 1
   int csv_slow_fields = 0;      // fields of the last plr_set_data_csv the host converted
@@ -523,7 +535,9 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
   return PLR_OK;
 }
 
-int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
+// The rows of an n x d shard: layout and kernel variant for that shape, then X
+// (with the slack the kernels may read past the last row) and y.
+int alloc_rows(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
   c->bias = (c->opt_first_col_one || c->synth_first_col) && d >= 2;
   c->dcols = d - (c->bias ? 1 : 0);
   int rc = plan_shape(c, n, c->dcols);
@@ -561,7 +575,18 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
       PLR_HIP(c, hipMemsetAsync(c->dX, 0, xbytes, c->stream));
       PLR_HIP(c, hipMemsetAsync(c->dy, 0, (size_t)n * sizeof(double), c->stream));
     }
+    if (c->pitch != c->dcols && !c->lane)  // the pad column must read as zero
+      PLR_HIP(c, hipMemset2DAsync(c->dX + c->dcols, (size_t)c->pitch * sizeof(double), 0,
+                                  (size_t)(c->pitch - c->dcols) * sizeof(double), (size_t)n,
+                                  c->stream));
   }
+  return PLR_OK;
+}
+
+// Everything else a pass over the resident rows needs: theta and result
+// staging, the per-workgroup partials of the variant chosen for (c->n, c->d).
+int alloc_workspace(plr_ctx* c) {
+  const int64_t n = c->n, d = c->d;
   const int gmax = c->grid > c->grid_nograd ? c->grid : c->grid_nograd;
   PLR_HIP(c, hipMalloc(&c->d_theta, (size_t)(c->theta_len + 8) * sizeof(double)));
   // a team shares one row of gradient partials
@@ -597,14 +622,15 @@ int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
   PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_out_dev), c->h_out, 0));
   memset(c->h_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double));
   PLR_HIP(c, hipMemsetAsync(c->d_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double), c->stream));
-  if (n > 0 && c->pitch != c->dcols && !c->lane)  // the pad column must read as zero
-    PLR_HIP(c, hipMemset2DAsync(c->dX + c->dcols, (size_t)c->pitch * sizeof(double), 0,
-                                (size_t)(c->pitch - c->dcols) * sizeof(double), (size_t)n,
-                                c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
   c->base_info = c->info;
   c->have_data = true;
   return PLR_OK;
+}
+
+int alloc_shape_buffers(plr_ctx* c, int64_t n, int64_t d, bool zero_fill) {
+  const int rc = alloc_rows(c, n, d, zero_fill);
+  return rc != PLR_OK ? rc : alloc_workspace(c);
 }
 
 // Drop the resident shard (if any) and reserve an n x d one.  On failure the
@@ -1068,54 +1094,146 @@ int64_t first_line_fields(const char* const* text, const int64_t* len, int nspan
 
 static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t count);
 
-int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, int nspans,
-                     char sep, int64_t* n_out, int64_t* d_out) {
-  if (!c) return PLR_ERR_INVALID;
-  if (nspans < 0 || (nspans > 0 && (!text || !len)))
-    return fail(c, PLR_ERR_INVALID, "text and len must not be NULL");
-  if (sep == '\n' || sep == '\0') return fail(c, PLR_ERR_INVALID, "bad separator");
-  int64_t total = 0;
-  for (int s = 0; s < nspans; ++s) {
-    if (len[s] < 0 || (len[s] > 0 && !text[s]))
-      return fail(c, PLR_ERR_INVALID, "bad text span");
-    total += len[s] + 1;  // a newline behind every span keeps their lines apart
-  }
-  const int64_t d = first_line_fields(text, len, nspans, sep);
-  if (n_out) *n_out = 0;
-  if (d_out) *d_out = d;
-  if (d == 0) {  // no sample line at all: an empty shard
-    PLR_HIP(c, hipSetDevice(c->device));
-    free_shape(c);
-    return PLR_OK;
-  }
-  if (d < 2)
-    return fail(c, PLR_ERR_UNSUPPORTED, "lines of one field (a label and no feature) are not "
-                                        "parsed on the device");
-  if (d > (int64_t)INT32_MAX) return fail(c, PLR_ERR_INVALID, "too many fields in a line");
-  PLR_HIP(c, hipSetDevice(c->device));
-  free_shape(c);
-  ShardGuard guard{c};
+// The sample text as it lies on the device: the spans back to back, a newline
+// behind each (it keeps their lines apart), then kCsvPadBytes of newlines.
+struct CsvText {
+  const char* const* text;
+  const int64_t* len;
+  int nspans;
+  int64_t total = 0;             // bytes with the newline behind every span
+  int64_t padded = 0;            // bytes of the device buffer
+  std::vector<int64_t> span_at;  // device offset of every span
+};
 
-  // the text, spans back to back, padded with newlines
+// Fields the device left to the host (longer digit strings, inf, nan, hex, ...):
+// std::stod on the host's copy of the text, then patched into the shard.
+static int resolve_slow_fields(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int nslow,
+                               const void* d_slow) {
+  if (nslow <= 0) return PLR_OK;
+  std::vector<plr::CsvSlow> slow(nslow);
+  PLR_HIP(c, hipMemcpy(slow.data(), d_slow, (size_t)nslow * sizeof(plr::CsvSlow),
+                       hipMemcpyDeviceToHost));
+  std::vector<int64_t> xi, yi;
+  std::vector<double> xv, yv;
+  for (const plr::CsvSlow& f : slow) {
+    int s = 0;
+    while (s + 1 < ct.nspans && f.pos >= ct.span_at[s + 1]) ++s;
+    const char* p = ct.text[s] + (f.pos - ct.span_at[s]);
+    const char* const end = ct.text[s] + ct.len[s];
+    int64_t flen = f.len;
+    if (flen < 0) {
+      flen = 0;
+      while (p + flen < end && p[flen] != sep && p[flen] != '\n') ++flen;
+    }
+    double v;
+    try {
+      v = std::stod(std::string(p, (size_t)flen));
+    } catch (const std::exception& e) {  // what the reference's parser would have thrown
+      return fail(c, PLR_ERR_INVALID, std::string(e.what()) + ": field " + std::to_string(f.col) +
+                                          " of sample line " + std::to_string(f.row));
+    }
+    if (f.col == d - 1) {
+      yi.push_back(f.row);
+      yv.push_back(v);
+    } else if (c->lane) {
+      const int64_t np = c->lane->np;
+      xi.push_back(((((f.row >> 6) * np + (f.col >> 1)) << 6) + (f.row & 63)) * 2 + (f.col & 1));
+      xv.push_back(v);
+    } else {
+      xi.push_back(f.row * c->pitch + f.col);
+      xv.push_back(v);
+    }
+  }
+  auto patch = [&](double* base, const std::vector<int64_t>& idx,
+                   const std::vector<double>& val) -> int {
+    if (idx.empty()) return PLR_OK;
+    DevBuf di, dv;
+    PLR_HIP(c, hipMalloc(&di.p, idx.size() * sizeof(int64_t)));
+    PLR_HIP(c, hipMalloc(&dv.p, val.size() * sizeof(double)));
+    PLR_HIP(c, hipMemcpy(di.p, idx.data(), idx.size() * sizeof(int64_t), hipMemcpyHostToDevice));
+    PLR_HIP(c, hipMemcpy(dv.p, val.data(), val.size() * sizeof(double), hipMemcpyHostToDevice));
+    hipLaunchKernelGGL(plr::csv_patch, dim3((unsigned)((idx.size() + 255) / 256)), dim3(256), 0,
+                       c->stream, base, static_cast<const int64_t*>(di.p),
+                       static_cast<const double*>(dv.p), (int64_t)idx.size());
+    PLR_HIP(c, hipGetLastError());
+    PLR_HIP(c, hipStreamSynchronize(c->stream));
+    return PLR_OK;
+  };
+  int rc = patch(c->dX, xi, xv);
+  if (rc == PLR_OK) rc = patch(c->dy, yi, yv);
+  return rc;
+}
+
+constexpr int kCsvSlowCap = 1 << 20;
+constexpr int kCsvRetrySerial = 1;  // the pipelined parse leaves the input to the serial one
+
+static plr::CsvArgs csv_args(plr_ctx* c, const unsigned char* dt, int64_t total,
+                             const int64_t* rows, int64_t n, int64_t d, char sep,
+                             plr::CsvSlow* slow, int64_t* ctl) {
+  plr::CsvArgs ca;
+  ca.text = dt;
+  ca.len = total;
+  ca.row_start = rows;
+  ca.n = n;
+  ca.row_range = nullptr;
+  ca.d = (int)d;
+  ca.sep = (unsigned char)sep;
+  ca.X = c->dX;
+  ca.y = c->dy;
+  ca.pitch = c->pitch;
+  ca.np = c->lane ? c->lane->np : 0;
+  ca.slow = slow;
+  ca.slow_cap = kCsvSlowCap;
+  ca.slow_count = reinterpret_cast<unsigned long long*>(ctl + 2);
+  ca.bad_row = reinterpret_cast<long long*>(ctl + 1);
+  ca.flush_at = 52;  // of 64 lanes (sweep: 32..64 within 3 %, 1 is 40 % slower)
+  return ca;
+}
+
+// What both parses end with: the parser's verdict, the fields left to the
+// host, the description.
+static int finish_csv(plr_ctx* c, const CsvText& ct, int64_t d, char sep, const int64_t res[3],
+                      const void* d_slow, bool lane_rows, const char* how) {
+  if (res[1] != INT64_MAX)  // parse_lines' message for the same input
+    return fail(c, PLR_ERR_INVALID, "ragged sample line " + std::to_string(res[1]));
+  if (res[2] > (int64_t)kCsvSlowCap)
+    return fail(c, PLR_ERR_UNSUPPORTED,
+                "more than 2^20 fields need the host's number parser: parse this input there");
+  const int nslow = (int)res[2];
+  const int rc = resolve_slow_fields(c, ct, d, sep, nslow, d_slow);
+  if (rc != PLR_OK) return rc;
+  c->csv_slow_fields = nslow;
+  c->info += std::string("; parsed from text") + how + " (a " + (lane_rows ? "lane" : "wave") +
+             " per row), " + std::to_string(nslow) + " fields converted on the host";
+  c->base_info = c->info;
+  if (c->timing) {  // plr_get_timing's last_ms: the parsing kernel(s)
+    float ms = 0.f;
+    PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
+    c->last_ms = ms;
+  }
+  return PLR_OK;
+}
+
+// Transfer, then parse: the whole text goes to the device, the rows are counted
+// (the host learns n and reserves exactly that shard), then located and parsed.
+static int csv_serial(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int64_t* n_out) {
   DevBuf d_text, d_counts, d_first, d_rows, d_slow, d_ctl;
-  const int64_t padded = (total + 15) / 16 * 16 + plr::kCsvPadBytes;
-  if (hipMalloc(&d_text.p, (size_t)padded) != hipSuccess) {
+  const int64_t total = ct.total;
+  if (hipMalloc(&d_text.p, (size_t)ct.padded) != hipSuccess) {
     (void)hipGetLastError();
     return fail(c, PLR_ERR_NOMEM, "cannot allocate the device copy of the sample text");
   }
   unsigned char* dt = static_cast<unsigned char*>(d_text.p);
-  std::vector<int64_t> span_at(nspans + 1, 0);  // device offset of every span
   std::vector<CopyPiece> pieces;
-  for (int s = 0; s < nspans; ++s) {
-    if (len[s]) pieces.push_back({dt + span_at[s], text[s], (size_t)len[s]});
-    PLR_HIP(c, hipMemsetAsync(dt + span_at[s] + len[s], '\n', 1, c->stream));
-    span_at[s + 1] = span_at[s] + len[s] + 1;
+  for (int s = 0; s < ct.nspans; ++s) {
+    if (ct.len[s]) pieces.push_back({dt + ct.span_at[s], ct.text[s], (size_t)ct.len[s]});
+    PLR_HIP(c, hipMemsetAsync(dt + ct.span_at[s] + ct.len[s], '\n', 1, c->stream));
   }
   {
     const int rc = copy_bytes_in(c, pieces);
     if (rc != PLR_OK) return rc;
   }
-  PLR_HIP(c, hipMemsetAsync(dt + total, '\n', (size_t)(padded - total), c->stream));
+  PLR_HIP(c, hipMemsetAsync(dt + total, '\n', (size_t)(ct.padded - total), c->stream));
 
   // rows: count, running sum, offsets
   const int64_t nblocks = (total + plr::kCsvBlockBytes - 1) / plr::kCsvBlockBytes;
@@ -1124,48 +1242,36 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   PLR_HIP(c, hipMalloc(&d_first.p, (size_t)nblocks * sizeof(int64_t)));
   PLR_HIP(c, hipMalloc(&d_ctl.p, 4 * sizeof(int64_t)));  // [0] rows, [1] bad row, [2] slow fields
   int64_t* ctl = static_cast<int64_t*>(d_ctl.p);
+  PLR_HIP(c, hipMemsetAsync(ctl, 0, 4 * sizeof(int64_t), c->stream));
   hipLaunchKernelGGL(plr::csv_count_rows, dim3((unsigned)nblocks), dim3(plr::kCsvThreads), 0,
-                     c->stream, dt, total, static_cast<int*>(d_counts.p));
+                     c->stream, dt, total, static_cast<int*>(d_counts.p), (int64_t)0);
   hipLaunchKernelGGL(plr::csv_scan_counts, dim3(1), dim3(1024), 0, c->stream,
                      static_cast<const int*>(d_counts.p), nblocks,
-                     static_cast<int64_t*>(d_first.p), ctl);
+                     static_cast<int64_t*>(d_first.p), ctl, static_cast<int64_t*>(nullptr));
   PLR_HIP(c, hipGetLastError());
   int64_t n = 0;
   PLR_HIP(c, hipMemcpyAsync(&n, ctl, sizeof n, hipMemcpyDeviceToHost, c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
   if (n_out) *n_out = n;
 
-  // the shard: k = d - 1 feature columns; the sample's constant first column is not stored
+  // the shard: k = d - 1 feature columns; the sample's constant first column is
+  // not stored.  Every field of every row is written by the parser (a line with
+  // another number of fields fails the call), so only the padding is cleared.
   c->synth_first_col = true;
-  int rc = alloc_shape_buffers(c, n, d, /*zero_fill=*/true);
+  int rc = alloc_shape_buffers(c, n, d, /*zero_fill=*/false);
   c->synth_first_col = false;
   if (rc != PLR_OK) return rc;
   PLR_HIP(c, hipMalloc(&d_rows.p, (size_t)std::max<int64_t>(n, 1) * sizeof(int64_t)));
   hipLaunchKernelGGL(plr::csv_row_starts, dim3((unsigned)nblocks), dim3(plr::kCsvThreads), 0,
                      c->stream, dt, total, static_cast<const int64_t*>(d_first.p),
-                     static_cast<int64_t*>(d_rows.p));
+                     static_cast<int64_t*>(d_rows.p), (int64_t)0, n);
   PLR_HIP(c, hipGetLastError());
 
-  const int slow_cap = 1 << 20;
-  PLR_HIP(c, hipMalloc(&d_slow.p, (size_t)slow_cap * sizeof(plr::CsvSlow)));
+  PLR_HIP(c, hipMalloc(&d_slow.p, (size_t)kCsvSlowCap * sizeof(plr::CsvSlow)));
   const int64_t ctl_init[3] = {n, INT64_MAX, 0};
   PLR_HIP(c, hipMemcpyAsync(ctl, ctl_init, sizeof ctl_init, hipMemcpyHostToDevice, c->stream));
-  plr::CsvArgs ca;
-  ca.text = dt;
-  ca.len = total;
-  ca.row_start = static_cast<const int64_t*>(d_rows.p);
-  ca.n = n;
-  ca.d = (int)d;
-  ca.sep = (unsigned char)sep;
-  ca.X = c->dX;
-  ca.y = c->dy;
-  ca.pitch = c->pitch;
-  ca.np = c->lane ? c->lane->np : 0;
-  ca.slow = static_cast<plr::CsvSlow*>(d_slow.p);
-  ca.slow_cap = slow_cap;
-  ca.slow_count = reinterpret_cast<unsigned long long*>(ctl + 2);
-  ca.bad_row = reinterpret_cast<long long*>(ctl + 1);
-  ca.flush_at = 52;  // of 64 lanes (sweep: 32..64 within 3 %, 1 is 40 % slower)
+  const plr::CsvArgs ca = csv_args(c, dt, total, static_cast<const int64_t*>(d_rows.p), n, d, sep,
+                                   static_cast<plr::CsvSlow*>(d_slow.p), ctl);
   // many rows: a lane per row (every lane in the character step); few rows: a wave per row
   const bool lane_rows = c->opt_csv_lane_rows < 0 ? n >= (int64_t)c->num_cu * 4 * 64 * 2
                                                   : c->opt_csv_lane_rows != 0;
@@ -1180,81 +1286,295 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
   int64_t res[3] = {0, 0, 0};
   PLR_HIP(c, hipMemcpyAsync(res, ctl, sizeof res, hipMemcpyDeviceToHost, c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
+  return finish_csv(c, ct, d, sep, res, d_slow.p, lane_rows, "");
+}
 
-  auto give_up = [&](int code, const std::string& msg) { return fail(c, code, msg); };
-  if (res[1] != INT64_MAX)  // parse_lines' message for the same input
-    return give_up(PLR_ERR_INVALID, "ragged sample line " + std::to_string(res[1]));
-  if (res[2] > (int64_t)slow_cap)
-    return give_up(PLR_ERR_UNSUPPORTED,
-                   "more than 2^20 fields need the host's number parser: parse this input there");
-  const int nslow = (int)res[2];
-  if (nslow > 0) {
-    // spellings the device does not convert: std::stod on the host's copy of the text
-    std::vector<plr::CsvSlow> slow(nslow);
-    PLR_HIP(c, hipMemcpy(slow.data(), d_slow.p, (size_t)nslow * sizeof(plr::CsvSlow),
-                         hipMemcpyDeviceToHost));
-    std::vector<int64_t> xi, yi;
-    std::vector<double> xv, yv;
-    for (const plr::CsvSlow& f : slow) {
-      int s = 0;
-      while (s + 1 < nspans && f.pos >= span_at[s + 1]) ++s;
-      const char* p = text[s] + (f.pos - span_at[s]);
-      const char* const end = text[s] + len[s];
-      int64_t flen = f.len;
-      if (flen < 0) {
-        flen = 0;
-        while (p + flen < end && p[flen] != sep && p[flen] != '\n') ++flen;
-      }
-      double v;
-      try {
-        v = std::stod(std::string(p, (size_t)flen));
-      } catch (const std::exception& e) {  // what the reference's parser would have thrown
-        return give_up(PLR_ERR_INVALID, std::string(e.what()) + ": field " +
-                                            std::to_string(f.col) + " of sample line " +
-                                            std::to_string(f.row));
-      }
-      if (f.col == d - 1) {
-        yi.push_back(f.row);
-        yv.push_back(v);
-      } else if (c->lane) {
-        const int64_t np = c->lane->np;
-        xi.push_back(((((f.row >> 6) * np + (f.col >> 1)) << 6) + (f.row & 63)) * 2 + (f.col & 1));
-        xv.push_back(v);
-      } else {
-        xi.push_back(f.row * c->pitch + f.col);
-        xv.push_back(v);
-      }
+// Lines per byte from a sample of the text: the lengths of up to 256 lines at
+// evenly spaced places.  0 when no line was found.
+static double sampled_line_bytes(const CsvText& ct) {
+  double sum = 0.;
+  int64_t cnt = 0;
+  const int kSamples = 256;
+  for (int i = 0; i < kSamples; ++i) {
+    const int64_t off = (int64_t)((double)ct.total * i / kSamples);
+    int s = 0;
+    while (s + 1 < ct.nspans && off >= ct.span_at[s + 1]) ++s;
+    const char* t = ct.text[s];
+    const int64_t L = ct.len[s];
+    int64_t p = std::min<int64_t>(off - ct.span_at[s], L);
+    if (i > 0 || p > 0) {  // the line in progress at `off` is skipped
+      const void* nl = p < L ? memchr(t + p, '\n', (size_t)(L - p)) : nullptr;
+      if (!nl) continue;
+      p = static_cast<const char*>(nl) - t + 1;
     }
-    auto patch = [&](double* base, const std::vector<int64_t>& idx,
-                     const std::vector<double>& val) -> int {
-      if (idx.empty()) return PLR_OK;
-      DevBuf di, dv;
-      PLR_HIP(c, hipMalloc(&di.p, idx.size() * sizeof(int64_t)));
-      PLR_HIP(c, hipMalloc(&dv.p, val.size() * sizeof(double)));
-      PLR_HIP(c, hipMemcpy(di.p, idx.data(), idx.size() * sizeof(int64_t), hipMemcpyHostToDevice));
-      PLR_HIP(c, hipMemcpy(dv.p, val.data(), val.size() * sizeof(double), hipMemcpyHostToDevice));
-      hipLaunchKernelGGL(plr::csv_patch, dim3((unsigned)((idx.size() + 255) / 256)), dim3(256), 0,
-                         c->stream, base, static_cast<const int64_t*>(di.p),
-                         static_cast<const double*>(dv.p), (int64_t)idx.size());
-      PLR_HIP(c, hipGetLastError());
-      PLR_HIP(c, hipStreamSynchronize(c->stream));
+    while (p < L && t[p] == '\n') ++p;  // empty lines are no rows
+    if (p >= L) continue;
+    const void* e = memchr(t + p, '\n', (size_t)(L - p));
+    const int64_t end = e ? static_cast<const char*>(e) - t : L;
+    sum += (double)(end - p + 1);
+    ++cnt;
+  }
+  return cnt ? sum / (double)cnt : 0.;
+}
+
+// Device offset of the first newline at or behind device offset `off`.
+static int64_t newline_at_or_after(const CsvText& ct, int64_t off) {
+  int s = 0;
+  while (s + 1 < ct.nspans && off >= ct.span_at[s + 1]) ++s;
+  const int64_t p = off - ct.span_at[s];
+  if (p < ct.len[s]) {
+    const void* nl = memchr(ct.text[s] + p, '\n', (size_t)(ct.len[s] - p));
+    if (nl) return ct.span_at[s] + (static_cast<const char*>(nl) - ct.text[s]);
+  }
+  return ct.span_at[s] + ct.len[s];  // the newline behind the span
+}
+
+struct LaneProgress;
+static int lanes_in(plr_ctx* c, const std::vector<InJob>& jobs, const FillFn& fill,
+                    const SentFn& sent, const char* what, LaneProgress* prog,
+                    const std::function<int()>* conductor);
+
+// Parse while the text arrives.  The text crosses the host link in 4 MiB blocks
+// on the copy lanes; cut into stretches, every stretch is counted, located and
+// parsed on the context's stream as soon as it and the end of its last row
+// are on the device -- so the parser works in the shadow of the transfer and
+// only the last stretch's kernels are left when the last byte has arrived.
+// A wave of the lane-per-row parser walks 64 whole rows in lockstep, which on
+// rows of kilobytes takes it milliseconds however few rows there are; it pays
+// when some thousands of waves are in flight -- 262144 rows or more.  A stretch
+// (64 MiB, the last one 16 MiB) with fewer rows goes to the wave-per-row
+// parser, whose waves are done with a row in tens of microseconds and which
+// still parses faster than the host link delivers (measured on rows of 512
+// six-decimal fields: 62 GB/s of text against 50).
+// The shard has to exist before the number of rows is known: it is reserved
+// for an estimate from the lengths of sampled lines plus 1/64 and 4096 rows;
+// the few rows reserved in excess stay allocated.  Whenever that does not work
+// out -- more rows than reserved, no memory for the generous shard -- the call
+// falls back to csv_serial (kCsvRetrySerial; nothing is left behind).
+// Off unless plr_set_option("csv_overlap", 1).  Measured on 1.96 GB of text
+// (rows of 512 six-decimal fields): the kernels do keep pace -- the stream has
+// drained 0.03 ms after the last block has landed -- but the transfer itself
+// takes 41-63 ms beside them instead of the 36-41 ms it takes alone (the copy
+// lanes' streams and the kernels' stream share the device's few hardware
+// queues, and a block queued behind a kernel waits for it; with the kernels
+// dealt over the lanes' own streams, or the lanes sharing two or three
+// streams, 41-61 ms), so that the whole call is 44-62 ms against 48-53 ms for
+// transfer-then-parse: no gain that could be relied on.
+constexpr int64_t kCsvStretch = 64ll << 20, kCsvLastStretch = 16ll << 20;
+constexpr int64_t kCsvLaneRowsMin = 4 * 1024 * 64;  // rows that fill the device's SIMDs 4 deep
+static_assert(kCsvLastStretch % (int64_t)kCopyBlock == 0 &&
+                  (int64_t)kCopyBlock % plr::kCsvBlockBytes == 0,
+              "a stretch is whole copy blocks and whole counting blocks");
+
+struct LaneProgress {
+  std::vector<hipEvent_t> done;            // per job: recorded behind its transfer
+  std::atomic<size_t> issued[kCopyLanes];  // jobs lane l has issued (its k-th job is l + 8 k)
+  std::atomic<bool> failed{false};
+  ~LaneProgress() {
+    for (hipEvent_t e : done)
+      if (e) (void)hipEventDestroy(e);
+  }
+};
+
+static int csv_pipelined(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int64_t* n_out) {
+  const int64_t total = ct.total;
+  const double line_bytes = sampled_line_bytes(ct);
+  if (line_bytes <= 0.) return kCsvRetrySerial;
+  const int64_t n_est = (int64_t)((double)total / line_bytes);
+  const int64_t cap = n_est + n_est / 64 + 4096;
+  const int64_t nblocks = ceil_div(total, (int64_t)plr::kCsvBlockBytes);
+  if (nblocks > (int64_t)INT32_MAX) return kCsvRetrySerial;
+  // stretch boundaries (multiples of the copy block, so of the counting block)
+  std::vector<int64_t> bound(1, 0);
+  {
+    const int64_t S = kCsvStretch;
+    const int64_t last = (total - kCsvLastStretch) / (int64_t)kCopyBlock * (int64_t)kCopyBlock;
+    for (int64_t b = S; b + S / 2 < last; b += S) bound.push_back(b);
+    if (last > bound.back()) bound.push_back(last);
+    bound.push_back(total);
+  }
+  const int64_t nslabs = (int64_t)bound.size() - 1;
+  DevBuf d_text, d_counts, d_first, d_rows, d_slow, d_ctl;
+  auto no_room = [&]() {
+    (void)hipGetLastError();
+    return kCsvRetrySerial;
+  };
+  if (hipMalloc(&d_text.p, (size_t)ct.padded) != hipSuccess) return no_room();
+  unsigned char* dt = static_cast<unsigned char*>(d_text.p);
+  for (int s = 0; s < ct.nspans; ++s)
+    PLR_HIP(c, hipMemsetAsync(dt + ct.span_at[s] + ct.len[s], '\n', 1, c->stream));
+  PLR_HIP(c, hipMemsetAsync(dt + total, '\n', (size_t)(ct.padded - total), c->stream));
+
+  // the transfer's jobs, in text order
+  std::vector<InJob> jobs;
+  std::vector<const char*> src;
+  std::vector<int64_t> job_end;  // device offset behind every job
+  for (int s = 0; s < ct.nspans; ++s)
+    for (int64_t at = 0; at < ct.len[s]; at += (int64_t)kCopyBlock) {
+      const size_t m = (size_t)std::min<int64_t>((int64_t)kCopyBlock, ct.len[s] - at);
+      jobs.push_back({dt + ct.span_at[s] + at, m});
+      src.push_back(ct.text[s] + at);
+      job_end.push_back(ct.span_at[s] + at + (int64_t)m);
+    }
+  LaneProgress prog;
+  prog.done.assign(jobs.size(), nullptr);
+  for (size_t j = 0; j < jobs.size(); ++j)
+    PLR_HIP(c, hipEventCreateWithFlags(&prog.done[j], hipEventDisableTiming));
+  for (int l = 0; l < kCopyLanes; ++l) prog.issued[l].store(0);
+
+  int64_t res[3] = {0, INT64_MAX, 0};
+  bool lane_rows = false, any_by_lane = false;
+  int fallback = 0;  // set by the conductor: leave the input to csv_serial
+  const std::function<int()> conductor = [&]() -> int {
+    // (runs on the calling thread while the lanes move the text)
+    c->synth_first_col = true;
+    int rc = alloc_rows(c, cap, d, /*zero_fill=*/false);
+    c->synth_first_col = false;
+    if (rc == PLR_ERR_NOMEM) {
+      fallback = 1;
       return PLR_OK;
-    };
-    rc = patch(c->dX, xi, xv);
-    if (rc == PLR_OK) rc = patch(c->dy, yi, yv);
+    }
     if (rc != PLR_OK) return rc;
+    if (hipMalloc(&d_counts.p, (size_t)nblocks * sizeof(int)) != hipSuccess ||
+        hipMalloc(&d_first.p, (size_t)nblocks * sizeof(int64_t)) != hipSuccess ||
+        hipMalloc(&d_rows.p, (size_t)cap * sizeof(int64_t)) != hipSuccess ||
+        hipMalloc(&d_slow.p, (size_t)kCsvSlowCap * sizeof(plr::CsvSlow)) != hipSuccess ||
+        hipMalloc(&d_ctl.p, (size_t)(4 + 2 * nslabs) * sizeof(int64_t)) != hipSuccess) {
+      (void)hipGetLastError();
+      fallback = 1;
+      return PLR_OK;
+    }
+    int64_t* ctl = static_cast<int64_t*>(d_ctl.p);  // [0] rows so far, [1] bad row, [2] slow fields
+    int64_t* ranges = ctl + 4;                       // [stretch][2]: its rows
+    const int64_t ctl_init[4] = {0, INT64_MAX, 0, 0};
+    PLR_HIP(c, hipMemcpyAsync(ctl, ctl_init, sizeof ctl_init, hipMemcpyHostToDevice, c->stream));
+    plr::CsvArgs ca = csv_args(c, dt, total, static_cast<const int64_t*>(d_rows.p), cap, d, sep,
+                               static_cast<plr::CsvSlow*>(d_slow.p), ctl);
+    lane_rows = c->opt_csv_lane_rows > 0;  // forced; otherwise by the rows of a stretch
+    size_t ready = 0;  // jobs [0, ready) are behind the context's stream already
+    for (int64_t s = 0; s < nslabs; ++s) {
+      hipStream_t cs = c->stream;
+      // what this stretch needs on the device: itself, and the row that starts
+      // last in it to its end, plus what the parser reads ahead
+      const int64_t need = std::min<int64_t>(
+          total, newline_at_or_after(ct, bound[s + 1] - 1) + 1 + plr::kCsvPadBytes);
+      size_t upto = ready;
+      while (upto < jobs.size() && job_end[upto] - (int64_t)jobs[upto].bytes < need) ++upto;
+      for (int l = 0; l < kCopyLanes; ++l) {
+        // lane l's jobs below `upto`: l, l + 8, ...
+        const size_t mine = upto > (size_t)l ? (upto - l + kCopyLanes - 1) / kCopyLanes : 0;
+        while (prog.issued[l].load(std::memory_order_acquire) < mine) {
+          if (prog.failed.load()) return PLR_OK;  // the lanes report the error
+          std::this_thread::sleep_for(std::chrono::microseconds(20));
+        }
+        if (mine > 0 && (size_t)l + (mine - 1) * kCopyLanes >= ready)
+          PLR_HIP(c, hipStreamWaitEvent(cs, prog.done[l + (mine - 1) * kCopyLanes], 0));
+      }
+      ready = upto;
+      const int64_t b0 = bound[s] / plr::kCsvBlockBytes;
+      const int64_t nb = ceil_div(bound[s + 1], (int64_t)plr::kCsvBlockBytes) - b0;
+      if (s == 0 && c->timing) PLR_HIP(c, hipEventRecord(c->ev0, cs));
+      hipLaunchKernelGGL(plr::csv_count_rows, dim3((unsigned)nb), dim3(plr::kCsvThreads), 0,
+                         cs, dt, total, static_cast<int*>(d_counts.p), b0);
+      hipLaunchKernelGGL(plr::csv_scan_counts, dim3(1), dim3(1024), 0, cs,
+                         static_cast<const int*>(d_counts.p) + b0, nb,
+                         static_cast<int64_t*>(d_first.p) + b0, ctl, ranges + 2 * s);
+      hipLaunchKernelGGL(plr::csv_row_starts, dim3((unsigned)nb), dim3(plr::kCsvThreads), 0,
+                         cs, dt, total, static_cast<const int64_t*>(d_first.p),
+                         static_cast<int64_t*>(d_rows.p), b0, cap);
+      ca.row_range = ranges + 2 * s;
+      // rows of this stretch, roughly
+      const int64_t rows = std::max<int64_t>(
+          1, (int64_t)((double)(bound[s + 1] - bound[s]) / line_bytes));
+      const bool by_lane = c->opt_csv_lane_rows < 0 ? rows >= kCsvLaneRowsMin : lane_rows;
+      any_by_lane = any_by_lane || by_lane;
+      const int64_t want = by_lane ? (rows + 255) / 256 : (rows + 3) / 4;
+      const unsigned pgrid = (unsigned)std::min<int64_t>(std::max<int64_t>(want, 1),
+                                                         (int64_t)c->num_cu * 8);
+      hipLaunchKernelGGL(by_lane ? plr::csv_parse_rows : plr::csv_parse, dim3(pgrid), dim3(256), 0,
+                         cs, ca);
+      PLR_HIP(c, hipGetLastError());
+    }
+    if (c->timing) PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
+    PLR_HIP(c, hipMemcpyAsync(res, ctl, sizeof res, hipMemcpyDeviceToHost, c->stream));
+    return PLR_OK;
+  };
+  int rc = lanes_in(
+      c, jobs,
+      [&](size_t j, char* blk) {
+        memcpy(blk, src[j], jobs[j].bytes);
+        return true;
+      },
+      SentFn(), "copying the sample text to the device failed", &prog, &conductor);
+  if (rc != PLR_OK) return rc;
+  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  if (fallback || res[0] > cap) return kCsvRetrySerial;
+
+  // the exact shape: n rows of the cap reserved; variant, grid and workspace for n
+  const int64_t n = res[0];
+  if (n_out) *n_out = n;
+  if (c->lane && n < c->n_alloc) {
+    // the row-tiled layout's last group: its rows past n must read as zeros
+    const int64_t group = (int64_t)plr::kWave * c->lane->U;
+    const int64_t hi = std::min(c->n_alloc, ceil_div(std::max<int64_t>(n, 1), group) * group);
+    if (hi > n) {
+      hipLaunchKernelGGL(plr::zero_tiled_rows, dim3((unsigned)ceil_div((hi - n) * c->lane->np, 256)),
+                         dim3(256), 0, c->stream, c->dX, c->lane->np, n, hi);
+      PLR_HIP(c, hipGetLastError());
+    }
   }
-  c->csv_slow_fields = nslow;
-  c->info += std::string("; parsed from text (a ") + (lane_rows ? "lane" : "wave") +
-             " per row), " + std::to_string(nslow) + " fields converted on the host";
-  c->base_info = c->info;
-  if (c->timing) {  // plr_get_timing's last_ms: the parsing kernel
-    float ms = 0.f;
-    PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
-    c->last_ms = ms;
+  c->n = n;
+  rc = plan_shape(c, n, c->dcols);
+  if (rc != PLR_OK) return rc;
+  if (c->bias) c->info += "; first column constant 1, not stored";
+  c->bias_slot = c->theta_len;
+  rc = alloc_workspace(c);
+  if (rc != PLR_OK) return rc;
+  return finish_csv(c, ct, d, sep, res, d_slow.p, any_by_lane, " while it arrived");
+}
+
+int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, int nspans,
+                     char sep, int64_t* n_out, int64_t* d_out) {
+  if (!c) return PLR_ERR_INVALID;
+  if (nspans < 0 || (nspans > 0 && (!text || !len)))
+    return fail(c, PLR_ERR_INVALID, "text and len must not be NULL");
+  if (sep == '\n' || sep == '\0') return fail(c, PLR_ERR_INVALID, "bad separator");
+  CsvText ct;
+  ct.text = text;
+  ct.len = len;
+  ct.nspans = nspans;
+  ct.span_at.assign(nspans + 1, 0);
+  for (int s = 0; s < nspans; ++s) {
+    if (len[s] < 0 || (len[s] > 0 && !text[s]))
+      return fail(c, PLR_ERR_INVALID, "bad text span");
+    ct.span_at[s + 1] = ct.span_at[s] + len[s] + 1;  // a newline behind every span
   }
-  guard.done = true;
-  return PLR_OK;
+  ct.total = ct.span_at[nspans];
+  ct.padded = (ct.total + 15) / 16 * 16 + plr::kCsvPadBytes;
+  const int64_t d = first_line_fields(text, len, nspans, sep);
+  if (n_out) *n_out = 0;
+  if (d_out) *d_out = d;
+  if (d == 0) {  // no sample line at all: an empty shard
+    PLR_HIP(c, hipSetDevice(c->device));
+    free_shape(c);
+    return PLR_OK;
+  }
+  if (d < 2)
+    return fail(c, PLR_ERR_UNSUPPORTED, "lines of one field (a label and no feature) are not "
+                                        "parsed on the device");
+  if (d > (int64_t)INT32_MAX) return fail(c, PLR_ERR_INVALID, "too many fields in a line");
+  PLR_HIP(c, hipSetDevice(c->device));
+  free_shape(c);
+  if (c->opt_csv_overlap && ct.total >= 4 * kCsvStretch) {
+    ShardGuard guard{c};
+    const int rc = csv_pipelined(c, ct, d, sep, n_out);
+    if (rc == PLR_OK) guard.done = true;
+    if (rc != kCsvRetrySerial) return rc;
+  }
+  ShardGuard guard{c};
+  const int rc = csv_serial(c, ct, d, sep, n_out);
+  if (rc == PLR_OK) guard.done = true;
+  return rc;
 }
 
 int plr_get_data(plr_ctx* c, int64_t row0, int64_t nrows, double* X, int64_t ldx, double* y) {
@@ -1405,8 +1725,6 @@ int plr_calc_loss(plr_ctx* c, const double* theta, double* loss_sum, int64_t* n_
 // through kCopyLanes independent lanes, each with two pinned staging blocks on
 // a stream of its own: the DMA into one block overlaps the host copy out of
 // the other, and the lanes overlap each other.
-constexpr int kCopyLanes = 8;
-constexpr size_t kCopyBlock = 4u << 20;
 static_assert(sizeof(plr_ctx::out_stream) / sizeof(hipStream_t) == kCopyLanes,
               "one stream per copy lane");
 
@@ -1495,15 +1813,9 @@ static int copy_rows_out(plr_ctx* c, double* out, const double* dev, size_t coun
 // transfer on the same stream.  Jobs are dealt to the lanes in turn; a lane's thread fills
 // one of its two blocks while the other is in flight.  Job j uses block (j % lanes) * 2 +
 // (j / lanes) % 2 of the staging area.
-struct InJob {
-  void* dev;
-  size_t bytes;
-};
-using FillFn = std::function<bool(size_t job, char* blk)>;
-using SentFn = std::function<hipError_t(size_t job, hipStream_t st)>;
-
 static int lanes_in(plr_ctx* c, const std::vector<InJob>& jobs, const FillFn& fill,
-                    const SentFn& sent, const char* what) {
+                    const SentFn& sent, const char* what, LaneProgress* prog,
+                    const std::function<int()>* conductor) {
   if (jobs.empty()) return PLR_OK;
   if (!c->out_stage) {
     PLR_HIP(c, hipHostMalloc(&c->out_stage, 2 * kCopyLanes * kCopyBlock, hipHostMallocDefault));
@@ -1516,6 +1828,7 @@ static int lanes_in(plr_ctx* c, const std::vector<InJob>& jobs, const FillFn& fi
     errs[l] = hipSuccess;
     if (hipSetDevice(c->device) != hipSuccess) {
       errs[l] = hipErrorInvalidDevice;
+      if (prog) prog->failed.store(true);
       return;
     }
     char* stage = static_cast<char*>(c->out_stage) + (size_t)l * 2 * kCopyBlock;
@@ -1538,8 +1851,15 @@ static int lanes_in(plr_ctx* c, const std::vector<InJob>& jobs, const FillFn& fi
       hipError_t e = hipMemcpyAsync(jobs[j].dev, blk, jobs[j].bytes, hipMemcpyHostToDevice, st);
       if (e == hipSuccess && sent) e = sent(j, st);
       if (e == hipSuccess) e = hipEventRecord(freed[slot], st);
+      if (e == hipSuccess && prog) {
+        // whoever waits for this job's bytes waits for this event; the count is
+        // published only once the record has been issued
+        e = hipEventRecord(prog->done[j], st);
+        if (e == hipSuccess) prog->issued[l].store(round + 1, std::memory_order_release);
+      }
       if (e != hipSuccess) errs[l] = e;
     }
+    if (prog && (errs[l] != hipSuccess || stop.load())) prog->failed.store(true);
     if (hipStreamSynchronize(st) != hipSuccess && errs[l] == hipSuccess) errs[l] = hipErrorUnknown;
     for (int k = 0; k < 2; ++k)
       if (freed[k]) (void)hipEventDestroy(freed[k]);
@@ -1547,9 +1867,15 @@ static int lanes_in(plr_ctx* c, const std::vector<InJob>& jobs, const FillFn& fi
   const int nl = (int)std::min<size_t>(kCopyLanes, jobs.size());
   for (int l = nl; l < kCopyLanes; ++l) errs[l] = hipSuccess;
   std::thread th[kCopyLanes];
-  for (int l = 1; l < nl; ++l) th[l] = std::thread(lane, l);
-  lane(0);
-  for (int l = 1; l < nl; ++l) th[l].join();
+  // with a conductor every lane has a thread of its own and the caller's thread
+  // conducts (queues the work that follows the transfers, as they are issued)
+  const int first_thread = conductor ? 0 : 1;
+  for (int l = first_thread; l < nl; ++l) th[l] = std::thread(lane, l);
+  int conducted = PLR_OK;
+  if (conductor) conducted = (*conductor)();
+  else lane(0);
+  for (int l = first_thread; l < nl; ++l) th[l].join();
+  if (conducted != PLR_OK) return conducted;
   for (int l = 0; l < kCopyLanes; ++l)
     if (errs[l] != hipSuccess) {
       (void)hipGetLastError();
@@ -1581,7 +1907,7 @@ static int copy_bytes_in(plr_ctx* c, const std::vector<CopyPiece>& pieces) {
         memcpy(blk, src[j], jobs[j].bytes);
         return true;
       },
-      SentFn(), "copying to the device failed");
+      SentFn(), "copying to the device failed", nullptr, nullptr);
 }
 
 // Rows [row0, row0 + nrows) of the caller's row-major X (leading dimension ldx) into the
@@ -1661,7 +1987,8 @@ static int copy_rows_in(plr_ctx* c, int64_t row0, int64_t nrows, const double* X
       return hipGetLastError();
     };
   }
-  const int rc = lanes_in(c, jobs, fill, sent, "upload: host-to-device copy failed");
+  const int rc = lanes_in(c, jobs, fill, sent, "upload: host-to-device copy failed", nullptr,
+                          nullptr);
   if (bad_row.load() != INT64_MAX) {
     // lanes run ahead of each other: an earlier row may break the statement too
     int64_t first = bad_row.load();
@@ -1794,6 +2121,10 @@ int plr_set_option(plr_ctx* c, const char* key, int64_t value) {
   }
   if (strcmp(key, "first_column_is_one") == 0) {
     c->opt_first_col_one = value != 0;  // takes effect at the next plr_set_data / plr_alloc_data
+    return PLR_OK;
+  }
+  if (strcmp(key, "csv_overlap") == 0) {
+    c->opt_csv_overlap = value != 0;
     return PLR_OK;
   }
   if (strcmp(key, "csv_lane_per_row") == 0) {

@@ -9,6 +9,10 @@
 //   csv_count_rows   line starts per 4 KiB block of text
 //   csv_scan_counts  their running sum (one workgroup): first row of a block
 //   csv_row_starts   byte offset of every row
+// (these three and the parser also run on one stretch of the text at a time,
+// in text order, so that a stretch can be parsed while the next one is still
+// on its way from the host: the running row count is carried in device
+// memory from stretch to stretch, and the parser reads its row range there)
 //   csv_parse_rows   a lane per row, 64 rows per wave: every lane walks its own
 //                    row through strtod's grammar (shards of many rows)
 //   csv_parse        a wave per row: separators by ballot, one lane per field
@@ -55,7 +59,9 @@ struct CsvArgs {
   const unsigned char* text;  // len bytes followed by kCsvPadBytes of '\n'
   int64_t len;
   const int64_t* row_start;   // n byte offsets
-  int64_t n;
+  int64_t n;                  // rows of the shard (row_start, X, y hold that many)
+  const int64_t* row_range;   // nullptr: parse rows 0 .. n-1; else the rows
+                              //   row_range[0] .. min(row_range[1], n) - 1 (device memory)
   int d;                      // fields per line: k features, then the label
   unsigned char sep;
   double* X;                  // the shard: the k features of every row (the constant
@@ -90,10 +96,12 @@ __device__ __forceinline__ int csv_starts16(const unsigned char* t, int64_t base
   return c;
 }
 
+// counts[b] for the blocks block0 .. block0 + gridDim.x - 1 of the text
 __global__ __launch_bounds__(kCsvThreads) void csv_count_rows(const unsigned char* t, int64_t len,
-                                                              int* counts) {
+                                                              int* counts, int64_t block0) {
   __shared__ int part[kCsvThreads / 64];
-  const int64_t base = ((int64_t)blockIdx.x * kCsvThreads + threadIdx.x) * kCsvBytesPerThread;
+  const int64_t blk = block0 + blockIdx.x;
+  const int64_t base = (blk * kCsvThreads + threadIdx.x) * kCsvBytesPerThread;
   int c = csv_starts16(t, base, len, nullptr);
 #pragma unroll
   for (int m = 1; m < 64; m <<= 1) c += __shfl_xor(c, m, 64);
@@ -102,17 +110,24 @@ __global__ __launch_bounds__(kCsvThreads) void csv_count_rows(const unsigned cha
   if (threadIdx.x == 0) {
     int s = 0;
     for (int w = 0; w < kCsvThreads / 64; ++w) s += part[w];
-    counts[blockIdx.x] = s;
+    counts[blk] = s;
   }
 }
 
-// exclusive running sum of counts[0..nblocks) into first_row[], the total into *total
+// Running sum of counts[0..nblocks) into first_row[] (rows before each block),
+// starting from *total (the rows of the text in front of these blocks) and
+// leaving the new total there; range_out (nullable) receives the row range of
+// these blocks, [old total, new total].
 __global__ __launch_bounds__(1024) void csv_scan_counts(const int* counts, int64_t nblocks,
-                                                        int64_t* first_row, int64_t* total) {
+                                                        int64_t* first_row, int64_t* total,
+                                                        int64_t* range_out) {
   __shared__ int64_t wsum[16];
   __shared__ int64_t carry_s;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (threadIdx.x == 0) carry_s = 0;
+  if (threadIdx.x == 0) {
+    carry_s = *total;
+    if (range_out) range_out[0] = carry_s;
+  }
   __syncthreads();
   for (int64_t i0 = 0; i0 < nblocks; i0 += 1024) {
     const int64_t i = i0 + threadIdx.x;
@@ -132,15 +147,22 @@ __global__ __launch_bounds__(1024) void csv_scan_counts(const int* counts, int64
     if (threadIdx.x == 1023) carry_s = before + s;
     __syncthreads();
   }
-  if (threadIdx.x == 0) *total = carry_s;
+  if (threadIdx.x == 0) {
+    *total = carry_s;
+    if (range_out) range_out[1] = carry_s;
+  }
 }
 
+// row_start[] for the rows that start in blocks block0 .. block0 + gridDim.x - 1;
+// rows at or past `cap` (the entries row_start holds) are not stored
 __global__ __launch_bounds__(kCsvThreads) void csv_row_starts(const unsigned char* t, int64_t len,
                                                               const int64_t* first_row,
-                                                              int64_t* row_start) {
+                                                              int64_t* row_start, int64_t block0,
+                                                              int64_t cap) {
   __shared__ int part[kCsvThreads / 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t base = ((int64_t)blockIdx.x * kCsvThreads + threadIdx.x) * kCsvBytesPerThread;
+  const int64_t blk = block0 + blockIdx.x;
+  const int64_t base = (blk * kCsvThreads + threadIdx.x) * kCsvBytesPerThread;
   int64_t pos[kCsvBytesPerThread];
   const int c = csv_starts16(t, base, len, pos);
   int s = c;
@@ -153,8 +175,9 @@ __global__ __launch_bounds__(kCsvThreads) void csv_row_starts(const unsigned cha
   __syncthreads();
   int before = 0;
   for (int w = 0; w < wave; ++w) before += part[w];
-  int64_t* out = row_start + first_row[blockIdx.x] + before + s - c;
-  for (int k = 0; k < c; ++k) out[k] = pos[k];
+  const int64_t at = first_row[blk] + before + s - c;
+  for (int k = 0; k < c; ++k)
+    if (at + k < cap) row_start[at + k] = pos[k];
 }
 
 // exact powers of ten
@@ -214,8 +237,10 @@ __global__ __launch_bounds__(256) void csv_parse(CsvArgs a) {
   const int64_t wave0 = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int64_t nwaves = (int64_t)gridDim.x * 4;
   const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));  // lanes before mine
+  const int64_t row_lo = a.row_range ? a.row_range[0] : 0;
+  const int64_t row_hi = a.row_range ? (a.row_range[1] < a.n ? a.row_range[1] : a.n) : a.n;
 
-  for (int64_t r = wave0; r < a.n; r += nwaves) {
+  for (int64_t r = row_lo + wave0; r < row_hi; r += nwaves) {
     int64_t pos = a.row_start[r];
     int nfields = 0;       // fields of this row seen so far (uniform)
     bool prev_sep = true;  // the byte in front of the window ends a field (or the row starts here)
@@ -347,9 +372,12 @@ __global__ __launch_bounds__(256) void csv_parse_rows(CsvArgs a) {
   const int64_t wave0 = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int64_t nwaves = (int64_t)gridDim.x * 4;
 
-  for (int64_t r0 = wave0 * 64; r0 < a.n; r0 += nwaves * 64) {
+  const int64_t row_lo = a.row_range ? a.row_range[0] : 0;
+  const int64_t row_hi = a.row_range ? (a.row_range[1] < a.n ? a.row_range[1] : a.n) : a.n;
+
+  for (int64_t r0 = row_lo + wave0 * 64; r0 < row_hi; r0 += nwaves * 64) {
     const int64_t r = r0 + lane;
-    bool done = r >= a.n;
+    bool done = r >= row_hi;
     const int64_t start = done ? 0 : a.row_start[r];
     // the field in progress
     unsigned long long m = 0;

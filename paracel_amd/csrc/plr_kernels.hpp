@@ -777,6 +777,17 @@ __global__ void gather_rows(const double* X, int64_t pitch, int np, int64_t row0
   dst[i] = v;
 }
 
+// Rows row_lo .. row_hi-1 of a row-tiled shard (np column pairs per row) set to
+// zero: the rows behind the last one in the last group of tiles, which the
+// pass reads and which nobody else has written.
+__global__ void zero_tiled_rows(double* X, int np, int64_t row_lo, int64_t row_hi) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t row = row_lo + i / np;
+  const int p = (int)(i % np);
+  if (row >= row_hi) return;
+  reinterpret_cast<v2d*>(X)[((row / kWave) * np + p) * kWave + (row % kWave)] = v2d{0., 0.};
+}
+
 // lane_pass for the wider tiles (34..64 columns), where rows and accumulators
 // of a whole tile fill the registers of a wave (one wave per SIMD): a PAIR of
 // waves shares every tile, each holding half of the column pairs of the same

@@ -189,6 +189,77 @@ def test_pieces_of_text_and_rows_across_windows(plr, oracle):
     check_equal(plr, oracle, "\n".join(lines) + "\n")
 
 
+@pytest.fixture()
+def overlap(plr):
+    plr.set_option("csv_overlap", 1)
+    yield plr
+    plr.set_option("csv_overlap", 0)
+
+
+def test_text_parsed_while_it_arrives(overlap, oracle):
+    # option "csv_overlap": from 256 MiB on the text is parsed stretch by stretch while the rest
+    # is still on its way from the host (the shard reserved for an estimated row count); same
+    # shard, bit for bit, as with the whole text transferred first
+    plr = overlap
+    rng = np.random.default_rng(11)
+    block = make_text(rng, 2000, 512, kinds=[0]).encode()
+    reps = (300 << 20) // len(block) + 1
+    pieces = [block] * (reps - 1) + [block[:-1]]        # the last line without its newline
+    print("text: %d x %.1f MB" % (reps, len(block) / 1e6), flush=True)
+    n, d = plr.set_data_csv(pieces)
+    assert (n, d) == (2000 * reps, 513)
+    info = plr.kernel_info()
+    print(info, flush=True)
+    assert "while it arrived" in info
+    X, y = plr.get_data()
+    Xo, yo = oracle.local_parser(block.decode())
+    assert X[:2000].tobytes() == Xo.tobytes() and y[:2000].tobytes() == yo.tobytes()
+    Xr = X.reshape(reps, 2000, 513)
+    assert all(Xr[i].tobytes() == Xo.tobytes() for i in range(reps))
+    assert y.reshape(reps, 2000).tobytes() == np.tile(yo, reps).tobytes()
+    th = rng.normal(size=513)
+    g, loss, cnt = plr.loss_grad(th)
+    # the other order: transfer, then parse
+    plr.set_option("csv_overlap", 0)
+    try:
+        assert plr.set_data_csv(pieces) == (n, d)
+        assert "while it arrived" not in plr.kernel_info()
+        X2, y2 = plr.get_data()
+        g2, loss2, _ = plr.loss_grad(th)
+    finally:
+        plr.set_option("csv_overlap", 1)
+    assert X2.tobytes() == X.tobytes() and y2.tobytes() == y.tobytes()
+    np.testing.assert_array_equal(g, g2)
+    assert cnt == n and loss == loss2
+    # a ragged line deep in the text is still named by its number
+    from paracel_amd import PlrError
+
+    bad = block.replace(b",", b";", 1)                   # one line with a field less
+    with pytest.raises(PlrError) as e:
+        plr.set_data_csv([block] * 40 + [bad] + [block] * (reps - 41))
+    assert e.value.code == -1 and "ragged sample line %d" % (40 * 2000) in str(e.value)
+    assert plr.shape == (0, 0)
+
+
+def test_more_rows_than_the_sampled_lines_suggest(overlap):
+    # (with "csv_overlap") the row count is estimated from the lengths of 256 sampled lines; text whose short lines
+    # hide between the samples has several times the rows reserved, and the call must notice
+    # and start over (transfer, count, parse) instead of writing past the shard
+    long_line, short_line = b"0.12345678901234,1\n", b".5,0\n"
+    plr = overlap
+    pattern = long_line * 40000 + short_line * 60000
+    pieces = [pattern] * 256
+    assert sum(len(p) for p in pieces) >= 256 << 20
+    n, d = plr.set_data_csv(pieces)
+    assert (n, d) == (256 * 100000, 2)
+    assert "while it arrived" not in plr.kernel_info()
+    X, y = plr.get_data()
+    want_x = np.tile(np.r_[np.full(40000, 0.12345678901234), np.full(60000, 0.5)], 256)
+    want_y = np.tile(np.r_[np.ones(40000), np.zeros(60000)], 256)
+    assert np.array_equal(X[:, 0], np.ones(n)) and np.array_equal(X[:, 1], want_x)
+    assert np.array_equal(y, want_y)
+
+
 def test_errors_are_the_reference_parsers(plr):
     from paracel_amd import PlrError
 
