@@ -152,6 +152,8 @@ def parse_args():
     ap.add_argument("--e2e", action="store_true",
                     help="end-to-end rounds through the host parameter server (C++ worker + "
                          "plr_ps_server over ZeroMQ) instead of the bare gradient step")
+    ap.add_argument("--workers", type=int, default=1,
+                    help="with --e2e: worker processes sharing the GPU, each with n / W rows")
     ap.add_argument("--no-dense-ps", action="store_true",
                     help="with --e2e: start the server with its dense-vector fast path off")
     ap.add_argument("--parse", action="store_true",
@@ -207,7 +209,7 @@ def reference_build_status():
     missing = [k for k, hs in need.items()
                if not any(os.path.exists(os.path.join(r, h)) for r in roots for h in hs)]
     if missing:
-        return "reference lr_serial not buildable on this box: missing " + ", ".join(missing)
+        return "reference not buildable here: no " + ", ".join(missing)
     return "reference dependencies present (reference binary not timed by this script)"
 
 
@@ -240,12 +242,10 @@ def cpu_baseline(cfg, Xs, ys, theta, reps1=4, repsp=20):
         "unit": "steps/s",
         "cores": cores,
         "host_cpu_count": os.cpu_count(),
-        "cores_note": "threads used = min(os.cpu_count(), %d): a one-GPU box gives a job a "
-                      "%d-CPU share of its host" % (CPU_SHARE, CPU_SHARE),
         "kind": "port",
         "sample": "%s (d=%d), gradient traversal lr.cpp:132-138 in the reference's "
-                  "vector<vector<double>> layout, g++ -O3, %d threads as local workers"
-                  % (whole, cfg.d, cores),
+                  "vector<vector<double>> layout, g++ -O3, %d threads as local workers (a "
+                  "one-GPU box gives a job %d CPUs)" % (whole, cfg.d, cores, CPU_SHARE),
         "value_1core": 1.0 / (t1 * scale),
         "loss_pass_seconds_1core_scaled": tl1 * scale,
         "loss_pass_seconds_pcore_scaled": tlp * scale,
@@ -295,9 +295,10 @@ def run_train(a, cfg):
     print(json.dumps(out), flush=True)
 
 
-def run_e2e(a, cfg, rounds=None):
+def run_e2e(a, cfg, rounds=None, workers=1, theta_cpu=None):
     """steps rounds of read theta -> GPU delta -> bupdate against a real server
-    process; final theta against the CPU oracle's multi-worker training."""
+    process, by `workers` worker processes that share the GPU (each with its n / workers
+    rows of the shard); final theta against the CPU oracle's multi-worker training."""
     import subprocess
     import tempfile
 
@@ -316,35 +317,48 @@ def run_e2e(a, cfg, rounds=None):
         info = srv.stdout.readline().strip()
         with tempfile.TemporaryDirectory() as td:
             tout = os.path.join(td, "theta.bin")
-            cmd = [os.path.join(pkg, "plr_lr_worker"), "--server_info", info,
-                   "--synthetic", "%x,%d,%d,%.17g" % (cfg.seed, cfg.n, cfg.d, cfg.spec.scale),
-                   "--rounds", str(rounds), "--alpha", "%.17g" % cfg.alpha,
-                   "--beta", "%.17g" % cfg.beta, "--theta0", "zero",
-                   "--update_file", os.path.join(pkg, "liblr_update.so"), "--theta_out", tout]
-            r = subprocess.run(cmd, capture_output=True, text=True)
-            if r.returncode != 0:
-                raise RuntimeError("worker failed: " + r.stderr)
-            rep = json.loads(r.stdout.strip().splitlines()[-1])
+            procs = []
+            for r in range(workers):
+                cmd = [os.path.join(pkg, "plr_lr_worker"), "--server_info", info,
+                       "--synthetic", "%x,%d,%d,%.17g" % (cfg.seed, cfg.n, cfg.d, cfg.spec.scale),
+                       "--rounds", str(rounds), "--alpha", "%.17g" % cfg.alpha,
+                       "--beta", "%.17g" % cfg.beta, "--theta0", "zero",
+                       "--update_file", os.path.join(pkg, "liblr_update.so"), "--theta_out", tout,
+                       "--worker_id", str(r), "--worker_sz", str(workers)]
+                procs.append(subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                                              text=True))
+            reps = []
+            for p in procs:
+                o, e = p.communicate()
+                if p.returncode != 0:
+                    for q in procs:
+                        q.kill()
+                    raise RuntimeError("worker failed: " + e)
+                reps.append(json.loads(o.strip().splitlines()[-1]))
             theta_gpu = np.fromfile(tout)
     finally:
         srv.kill()
         srv.wait()
+    # the workers leave every round through the same barrier: the slowest one's clock
+    sec = max(r["seconds"] for r in reps)
+    kern_ms = sum(r["gpu_kernel_ms_per_iter"] for r in reps)  # the GPU runs them one after another
     out = {
-        "metric": "lr_e2e_iters_per_sec", "value": rep["iters_per_sec"], "unit": "iters/s",
+        "metric": "lr_e2e_iters_per_sec", "value": rounds / sec, "unit": "iters/s",
         "n_gpus": 1, "steps": rounds, "warmup": 0,
-        "ms_per_step": 1e3 / rep["iters_per_sec"], "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": 1e3 * sec / rounds, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": {"workload": cfg.name + " via parameter server", "n": cfg.n, "d": cfg.d,
+                   "workers": workers,
                    "step": "paracel_read theta -> plr_dgd_delta -> paracel_bupdate delta "
                            "(ZeroMQ REQ/REP, msgpack, dlopen'ed lr_theta_update)",
                    "ps_dense_fast_path": not a.no_dense_ps,
                    "alpha": cfg.alpha, "beta": cfg.beta},
-        "gpu_only_iters_per_sec": rep["gpu_only_iters_per_sec"],
-        "gpu_kernel_ms_per_iter": rep["gpu_kernel_ms_per_iter"],
-        "final_loss": rep["final_loss"],
+        "gpu_only_iters_per_sec": 1e3 / kern_ms,
+        "gpu_kernel_ms_per_iter": kern_ms,
+        "final_loss": reps[0]["final_loss"],
         "theta_rel_err_vs_cpu": None,
     }
-    if not a.no_cpu_baseline:
+    if theta_cpu is None and not a.no_cpu_baseline:
         from oracle import oracle
 
         cores = cpu_threads()
@@ -358,12 +372,14 @@ def run_e2e(a, cfg, rounds=None):
         theta_cpu = oracle.train_dgd_workers(X, y, np.zeros(cfg.d), cfg.alpha, cfg.beta,
                                              rounds, cores)
         sec = time.time() - t0
-        out["theta_rel_err_vs_cpu"] = float(np.linalg.norm(theta_gpu - theta_cpu) /
-                                            np.linalg.norm(theta_cpu))
         out["cpu_baseline"] = {"value": rounds / sec, "unit": "iters/s", "cores": cores,
                                "host_cpu_count": os.cpu_count(), "kind": "port",
                                "sample": "all %d rounds on the full shard, %d local workers "
                                          "(threads), in-process server add" % (rounds, cores)}
+    if theta_cpu is not None:
+        out["theta_rel_err_vs_cpu"] = float(np.linalg.norm(theta_gpu - theta_cpu) /
+                                            np.linalg.norm(theta_cpu))
+        out["theta_cpu"] = theta_cpu
     return out
 
 
@@ -432,8 +448,8 @@ def run_step(a, cfg, with_cpu, full_cpu_sample=False, cpu_reps=(4, 20), settle_m
     assert launches == a.steps and n == cfg.n
     kern_ms = kern_ms_sum / launches
 
-    read_ceiling = ctx.probe_read_bandwidth(10)
-    copy_ceiling = ctx.probe_copy_bandwidth(2 << 30, 5)   # read + written, runtime D2D copy
+    read_probe = ctx.probe_read_bandwidth(10)
+    copy_probe = ctx.probe_copy_bandwidth(2 << 30, 5)   # read + written, runtime D2D copy
     bytes_step = cfg.algorithmic_bytes()
     achieved = bytes_step / (kern_ms * 1e-3) / 1e9
     whole = bytes_step / (elapsed / a.steps) / 1e9
@@ -455,18 +471,26 @@ def run_step(a, cfg, with_cpu, full_cpu_sample=False, cpu_reps=(4, 20), settle_m
                    "step": "plr_loss_grad: theta host->device, fused loss+gradient pass, "
                            "gsum+loss device->host",
                    "lambda": cfg.lam, "alpha": cfg.alpha, "beta": cfg.beta,
-                   "kernel": info},
+                   "kernel": kernel_code(info)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "traffic_source": traffic_src,
                      "kernel_ms": kern_ms, "algorithmic_bytes": bytes_step,
                      "whole_step_gbs": whole, "whole_step_frac": whole / HBM_PEAK_GBS,
-                     "read_ceiling_gbs": read_ceiling,
-                     "frac_of_read_ceiling": achieved / read_ceiling,
-                     "copy_ceiling_gbs": copy_ceiling},
+                     # what a kernel that only reads the shard sustains, and the runtime's
+                     # device-to-device copy (bytes read + written): probes, not bounds
+                     "read_probe_gbs": read_probe,
+                     "frac_of_read_probe": achieved / read_probe,
+                     "copy_probe_gbs": copy_probe},
         "cpu_baseline": None,
         "loss_mean": loss / n,
     }
+    if cfg.bias_first and not KEEP_BIAS_COLUMN:
+        # the constant first column stays on the host: the kernel streams one column less
+        # than the reference's row has; both byte counts, both fractions
+        stored = bytes_step - 8 * cfg.n
+        out["roofline"]["stored_bytes"] = stored
+        out["roofline"]["frac_of_stored_bytes"] = stored / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg, Xs, ys, theta, *cpu_reps)
     ctx.close()
@@ -576,22 +600,40 @@ def run_parse(a, cfg):
     return out
 
 
-def per_config_entry(rec):
-    """The per_config summary of one bare-step record."""
+def kernel_code(info):
+    """'shard_pass<NCH=8,R=4,WCOL=1,WROW=4,ALLCH=1,TL=0> ...' -> 'shard_pass<8,4,1,4,1,0>' (+ what
+    else distinguishes the variant: team shape, the constant column left on the host)."""
+    import re
+
+    m = re.match(r"(\w+)<([^>]*)>", info)
+    code = info[:24] if not m else "%s<%s>" % (
+        m.group(1), ",".join(v.split("=")[-1] for v in m.group(2).split(",")))
+    t = re.search(r"(\d+) column blocks of (\d+-?) chunks", info)
+    if t:
+        code += " %sx%s" % (t.group(1), t.group(2))
+    if "two sweeps" in info:
+        code += " two-sweeps"
+    if "not stored" in info:
+        code += " col0-on-host"
+    return code
+
+
+# columns of the per_config / other_shapes rows
+ROW_COLS = ["steps_per_s", "ms_per_step", "kernel_ms", "gb_per_s", "frac", "whole_step_frac",
+            "read_probe_gb_per_s", "traffic_over_algorithmic", "cpu_steps_per_s_1core",
+            "cpu_steps_per_s_16", "kernel"]
+
+
+def compact_row(rec):
+    """One bare-step record as a row of ROW_COLS."""
     r = rec["roofline"]
-    e = {"steps_per_sec": rec["value"], "ms_per_step": rec["ms_per_step"],
-         "kernel_ms": r["kernel_ms"], "achieved_gbs": r["achieved"], "frac": r["frac"],
-         "whole_step_frac": r["whole_step_frac"], "algorithmic_bytes": r["algorithmic_bytes"],
-         "traffic": r["traffic"], "read_ceiling_gbs": r["read_ceiling_gbs"],
-         "n": rec["config"]["n"], "d": rec["config"]["d"], "kernel_info": rec["config"]["kernel"],
-         "steps": rec["steps"], "warmup": rec["warmup"]}
-    if rec["cpu_baseline"]:
-        c = rec["cpu_baseline"]
-        e["cpu_steps_per_sec"] = c["value"]
-        e["cpu_steps_per_sec_1core"] = c["value_1core"]
-        e["cpu_cores"] = c["cores"]
-        e["cpu_sample"] = c["sample"]
-    return e
+    c = rec["cpu_baseline"] or {}
+    sig = lambda v, nd=4: None if v is None else float("%.*g" % (nd, v))  # noqa: E731
+    return [sig(rec["value"]), sig(rec["ms_per_step"], 5), sig(r["kernel_ms"], 5),
+            sig(r["achieved"]), sig(r["frac"]), sig(r["whole_step_frac"]),
+            sig(r["read_probe_gbs"]),
+            sig(r["traffic"] / r["algorithmic_bytes"], 5) if r["traffic"] else None,
+            sig(c.get("value_1core"), 3), sig(c.get("value"), 3), rec["config"]["kernel"]]
 
 
 def main():
@@ -619,7 +661,9 @@ def main():
     if a.rows:
         cfg = cfg.scaled(a.rows)
     if a.e2e:
-        print(json.dumps(run_e2e(a, cfg)), flush=True)
+        rec = run_e2e(a, cfg, workers=a.workers)
+        rec.pop("theta_cpu", None)
+        print(json.dumps(rec), flush=True)
         return
     if a.train:
         run_train(a, cfg)
@@ -632,48 +676,100 @@ def main():
     out = run_step(a, cfg, with_cpu, full_cpu_sample=(a.workload is None and not a.rows),
                    settle_ms=(a.settle_ms if a.workload is not None else 0.0))
     if a.workload is None and not a.headline_only and not a.rows:
+        # Everything below rides in the same line, kept short: the harness keeps the tail of
+        # what a run prints.  Rows of numbers under one list of column names.
+        sig = lambda v, nd=4: None if v is None else float("%.*g" % (nd, v))  # noqa: E731
+        out["row_cols"] = ROW_COLS
         # the other configurations, same steps / warmup, bounded CPU legs
         per = {}
         for other in PER_CONFIG:
             rec = run_step(a, cfgs[other], with_cpu, cpu_reps=(2, 6), settle_ms=a.settle_ms)
-            per[other] = per_config_entry(rec)
-        # config 5 as it is defined: 100 rounds through the parameter server
-        e2e = run_e2e(a, cfgs["c5_e2e_2m_x_512"], rounds=100)
-        per["c5_e2e_2m_x_512_via_ps"] = {
-            "iters_per_sec": e2e["value"], "ms_per_iter": e2e["ms_per_step"], "rounds": 100,
-            "gpu_only_iters_per_sec": e2e["gpu_only_iters_per_sec"],
-            "gpu_kernel_ms_per_iter": e2e["gpu_kernel_ms_per_iter"],
-            "theta_rel_err_vs_cpu": e2e["theta_rel_err_vs_cpu"],
-            "final_loss": e2e["final_loss"],
-            "cpu_iters_per_sec": (e2e.get("cpu_baseline") or {}).get("value"),
-            "cpu_cores": (e2e.get("cpu_baseline") or {}).get("cores"),
-            "step": e2e["config"]["step"]}
+            per[other] = compact_row(rec)
+        out["per_config"] = per
+        # config 1 is an 80 MB shard (cache-resident): what its rounds cost end to end
+        try:
+            out["c1_latency_us"] = c1_latency(cfgs["c1_dense_100k_x_100"])
+        except Exception as e:
+            out["c1_latency_us"] = {"error": "%s: %s" % (type(e).__name__, e)}
+        # config 5 as it is defined: 100 rounds through the parameter server -- by one worker,
+        # and by 2 and 4 worker processes that share the GPU (n / W rows each)
+        c5 = cfgs["c5_e2e_2m_x_512"]
+        e2e = {"cols": ["workers", "iters_per_s", "ms_per_iter", "gpu_kernel_ms_per_iter",
+                        "theta_rel_err_vs_cpu"], "rows": [], "rounds": 100}
+        theta_cpu = None
+        for W in (1, 2, 4):
+            try:
+                r = run_e2e(a, c5, rounds=100, workers=W, theta_cpu=theta_cpu)
+                theta_cpu = r.pop("theta_cpu", theta_cpu)
+                e2e["rows"].append([W, sig(r["value"]), sig(r["ms_per_step"]),
+                                    sig(r["gpu_kernel_ms_per_iter"]),
+                                    sig(r["theta_rel_err_vs_cpu"], 3)])
+                if W == 1:
+                    e2e["final_loss"] = r["final_loss"]
+                    e2e["cpu_iters_per_s"] = sig((r.get("cpu_baseline") or {}).get("value"))
+                    e2e["cpu_cores"] = (r.get("cpu_baseline") or {}).get("cores")
+            except Exception as e:
+                e2e["rows"].append([W, "%s: %s" % (type(e).__name__, e)])
+        out["c5_via_ps"] = e2e
         # the loader of the same configuration: its sample text parsed on the device
         try:
-            pr = run_parse(a, cfgs["c5_e2e_2m_x_512"])
-            per["c5_e2e_2m_x_512_text_to_shard"] = {
-                "text_gb_per_sec": pr["value"], "ms_per_call": pr["ms_per_step"],
+            pr = run_parse(a, c5)
+            out["c5_text_to_shard"] = {
+                "text_gb_per_s": sig(pr["value"]), "ms_per_call": sig(pr["ms_per_step"]),
                 "text_bytes": pr["config"]["text_bytes"], "rows": pr["config"]["rows"],
-                "fields_per_row": pr["config"]["fields_per_row"],
-                "parse_kernel_ms": pr["roofline"]["kernel_ms"],
-                "parse_kernel_text_gbs": pr["roofline"]["text_gbs_kernel_only"],
-                "parse_kernel_frac_of_hbm": pr["roofline"]["frac"],
-                "cpu_text_gb_per_sec": pr["cpu_baseline"]["value"],
-                "cpu_cores": pr["cpu_baseline"]["cores"],
-                "cpu_text_gb_per_sec_1core": pr["cpu_baseline"]["value_1core"],
-                "reference_stod_1core_gbs": pr["cpu_baseline"]["reference_stod_1core_gbs"],
-                "step": pr["config"]["step"]}
+                "parse_kernel_ms": sig(pr["roofline"]["kernel_ms"]),
+                "parse_kernel_text_gb_per_s": sig(pr["roofline"]["text_gbs_kernel_only"]),
+                "parse_kernel_frac_of_hbm": sig(pr["roofline"]["frac"]),
+                "ms_per_call_with_csv_overlap": pr["config"]["ms_per_call_with_csv_overlap"],
+                "cpu_text_gb_per_s_16": sig(pr["cpu_baseline"]["value"]),
+                "cpu_text_gb_per_s_1core": sig(pr["cpu_baseline"]["value_1core"]),
+                "reference_stod_1core_gb_per_s": sig(pr["cpu_baseline"]["reference_stod_1core_gbs"])}
         except Exception as e:
-            per["c5_e2e_2m_x_512_text_to_shard"] = {"error": "%s: %s" % (type(e).__name__, e)}
-        out["per_config"] = per
+            out["c5_text_to_shard"] = {"error": "%s: %s" % (type(e).__name__, e)}
         extra = {}
         for other in OTHER_SHAPES:
             try:
-                extra[other] = per_config_entry(run_step(a, cfgs[other], False, settle_ms=a.settle_ms))
+                extra[other] = compact_row(run_step(a, cfgs[other], False, settle_ms=a.settle_ms))
             except Exception as e:  # the headline line must survive a shape that does not fit
-                extra[other] = {"error": "%s: %s" % (type(e).__name__, e)}
+                extra[other] = ["%s: %s" % (type(e).__name__, e)]
         out["other_shapes"] = extra
-    print(json.dumps(out), flush=True)
+    print(json.dumps(out, separators=(",", ":")), flush=True)
+
+
+def c1_latency(cfg):
+    """Microseconds per call on the 100 000 x 100 shard, wall clock over 300 calls each:
+    the bare step, the same with the timing events off, one round of plr_dgd_delta, and
+    one device-resident round of plr_train_dgd (100 rounds per call)."""
+    import numpy as np
+
+    from paracel_amd import Plr
+
+    with Plr(0) as ctx:
+        X, y = cfg.rows(0, cfg.n)
+        ctx.set_data(X, y)
+        th = cfg.theta()
+
+        def per_call(fn, reps=300):
+            for _ in range(30):
+                fn()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                fn()
+            return round((time.perf_counter() - t0) / reps * 1e6, 2)
+
+        res = {"loss_grad": per_call(lambda: ctx.loss_grad(th))}
+        ctx.set_timing(False)
+        res["loss_grad_timing_off"] = per_call(lambda: ctx.loss_grad(th))
+        res["dgd_delta_no_loss_timing_off"] = per_call(
+            lambda: ctx.dgd_delta(th, cfg.alpha, cfg.beta, want_loss=False))
+        z = np.zeros(cfg.d)
+        ctx.train_dgd(z, cfg.alpha, cfg.beta, 100)
+        t0 = time.perf_counter()
+        for _ in range(10):
+            ctx.train_dgd(z, cfg.alpha, cfg.beta, 100)
+        res["train_dgd_per_round"] = round((time.perf_counter() - t0) / 1000 * 1e6, 2)
+        ctx.set_timing(True)
+    return res
 
 
 if __name__ == "__main__":

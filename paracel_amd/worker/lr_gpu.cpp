@@ -24,13 +24,9 @@ logistic_regression_gpu::logistic_regression_gpu(
       rounds(_rounds),
       alpha(_alpha),
       beta(_beta),
-      debug(_debug) {
+      debug(_debug),
+      turn(device_id, _worker_sz > 1) {
   check(plr_create(&gpu, device_id), "plr_create");
-  // Several workers on one GPU: the one-read pass over rows wider than 19456
-  // columns needs its whole grid resident at once, which processes that share
-  // the compute units cannot count on; such shards take the two-sweep pass.
-  if (get_worker_size() > 1)
-    check(plr_set_option(gpu, "column_blocks_two_sweeps", 1), "plr_set_option");
 }
 
 logistic_regression_gpu::~logistic_regression_gpu() { plr_destroy(gpu); }
@@ -127,9 +123,12 @@ void logistic_regression_gpu::dgd_learning() {
     // round's loss at the theta just read is recorded (the reference records
     // it after every sample, an O(n^2 d) loop)
     double loss_sum = 0.;
-    check(plr_dgd_delta(gpu, theta.data(), alpha, beta, delta.data(),
-                        debug ? &loss_sum : nullptr),
-          "plr_dgd_delta");
+    {
+      gpu_turn_guard mine(turn);  // several workers on the GPU: one pass at a time
+      check(plr_dgd_delta(gpu, theta.data(), alpha, beta, delta.data(),
+                          debug ? &loss_sum : nullptr),
+            "plr_dgd_delta");
+    }
     if (debug) loss_error.push_back(n_local ? loss_sum / (double)n_local : 0.);
     paracel_sync();
     paracel_bupdate("theta", delta);
@@ -160,7 +159,10 @@ void logistic_regression_gpu::solve() {
 double logistic_regression_gpu::calc_loss() {
   double loss = 0.;
   int64_t cnt = 0;
-  check(plr_calc_loss(gpu, theta.data(), &loss, &cnt, PLR_LOSS_REFERENCE), "plr_calc_loss");
+  {
+    gpu_turn_guard mine(turn);
+    check(plr_calc_loss(gpu, theta.data(), &loss, &cnt, PLR_LOSS_REFERENCE), "plr_calc_loss");
+  }
   allreduce(loss);  // lr.cpp:331-334
   int sz = (int)cnt;
   allreduce(sz);

@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "../../include/plr.h"
+#include "gpu_turn.hpp"
 #include "paralg_lite.hpp"
 
 namespace plr_ps {
@@ -68,6 +69,7 @@ class logistic_regression_gpu : public paralg {
   std::vector<double> pred_samples;   // flattened prediction rows (lr.hpp: pred_samples)
   int64_t pred_dim = 0;
   plr_ctx* gpu = nullptr;
+  gpu_turn turn;
   double round_sec = 0.;
 };
 

@@ -7,9 +7,10 @@
 //
 // A second mode serves the end-to-end benchmark: --synthetic SEED,N,D,SCALE
 // builds the shard in memory with the seeded generator instead of parsing a
-// file, runs the rounds against the parameter server and prints one JSON line
-// with the end-to-end and GPU-only rates; --theta_out writes the final theta
-// as raw doubles.
+// file (worker R of W takes rows [N R / W, N (R + 1) / W) of the N-row shard, as
+// the loader would hand it its share of a file), runs the rounds against the
+// parameter server and prints one JSON line with the end-to-end and GPU-only
+// rates; --theta_out writes the final theta as raw doubles (worker 0).
 //
 // Where the reference takes rank and size from MPI (lr_driver.cpp:36-37, one
 // process per worker under mpirun), --worker_id R --worker_sz W name this
@@ -73,22 +74,25 @@ int main(int argc, char** argv) {
         throw std::invalid_argument("--synthetic wants SEEDHEX,N,D,SCALE");
       logistic_regression_gpu lr(server_info, "", "", update_file, update_func, "dgd", rounds,
                                  alpha, beta, false, device, worker_id, worker_sz);
+      const long long lo = n * worker_id / worker_sz, hi = n * (worker_id + 1) / worker_sz;
       {
         plr_gen_spec sp = {seed, PLR_GEN_NORMAL, 0, scale, 0.0, 1.0};
-        std::vector<double> X((size_t)n * d), y(n), ts(d);
-        plr_gen_X(&sp, 0, n, d, d, X.data(), 16);
+        const long long m = hi - lo;
+        std::vector<double> X((size_t)m * d), y(m), ts(d);
+        plr_gen_X(&sp, lo, m, d, d, X.data(), 16);
         plr_gen_vec(seed, PLR_STREAM_THETA_STAR, PLR_GEN_NORMAL, 1.0, 1.0, d, ts.data());
-        plr_gen_labels(&sp, 0, n, d, d, X.data(), ts.data(), y.data(), 16);
-        lr.set_samples(X.data(), n, d, d, y.data());
+        plr_gen_labels(&sp, lo, m, d, d, X.data(), ts.data(), y.data(), 16);
+        lr.set_samples(X.data(), m, d, d, y.data());
       }
       if (theta0 == "zero") lr.set_theta0(std::vector<double>(d, 0.));
       lr.solve();
       const double loss = lr.calc_loss();
       const double sec = lr.round_seconds(), kms = lr.gpu_kernel_ms();
-      if (!theta_out.empty()) {
+      if (!theta_out.empty() && worker_id == 0) {
         std::ofstream o(theta_out, std::ios::binary);
         o.write((const char*)lr.get_theta().data(), lr.get_theta().size() * sizeof(double));
       }
+      n = hi - lo;  // this worker's rows
       printf("{\"rounds\": %d, \"n\": %lld, \"d\": %lld, \"seconds\": %.6f, "
              "\"iters_per_sec\": %.3f, \"gpu_kernel_ms_per_iter\": %.6f, "
              "\"gpu_only_iters_per_sec\": %.3f, \"final_loss\": %.17g}\n",

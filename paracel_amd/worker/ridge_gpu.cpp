@@ -22,13 +22,9 @@ ridge_regression_gpu::ridge_regression_gpu(const std::string& hosts_dct_str,
       worker_id((int)get_worker_id()),
       rounds(_rounds),
       alpha(_alpha),
-      beta(_beta) {
+      beta(_beta),
+      turn(device_id, _worker_sz > 1) {
   check(plr_create(&gpu, device_id), "plr_create");
-  // Several workers on one GPU: the one-read pass over rows wider than 19456
-  // columns needs its whole grid resident at once, which processes that share
-  // the compute units cannot count on; such shards take the two-sweep pass.
-  if (get_worker_size() > 1)
-    check(plr_set_option(gpu, "column_blocks_two_sweeps", 1), "plr_set_option");
   // every shard this worker uploads starts its rows with the bias 1.0
   // (ridge.hpp:149,168): that column need not be kept in HBM
   check(plr_set_option(gpu, "first_column_is_one", 1), "plr_set_option");
@@ -81,8 +77,11 @@ void ridge_regression_gpu::batch_learning() {
   std::vector<double> delta(data_dim);
   for (int rd = 0; rd < rounds; ++rd) {
     theta = paracel_read<std::vector<double> >("theta");
-    check(plr_dgd_delta_linear(gpu, theta.data(), alpha, beta, delta.data(), nullptr),
-          "plr_dgd_delta_linear");
+    {
+      gpu_turn_guard mine(turn);  // several workers on the GPU: one pass at a time
+      check(plr_dgd_delta_linear(gpu, theta.data(), alpha, beta, delta.data(), nullptr),
+            "plr_dgd_delta_linear");
+    }
     paracel_sync();
     paracel_bupdate("theta", delta);
     paracel_sync();
@@ -102,7 +101,10 @@ void ridge_regression_gpu::solve() {
 double ridge_regression_gpu::calc_loss() {
   double loss = 0.;
   int64_t cnt = 0;
-  check(plr_calc_loss(gpu, theta.data(), &loss, &cnt, PLR_LOSS_SQUARED), "plr_calc_loss");
+  {
+    gpu_turn_guard mine(turn);
+    check(plr_calc_loss(gpu, theta.data(), &loss, &cnt, PLR_LOSS_SQUARED), "plr_calc_loss");
+  }
   allreduce(loss);  // ridge.hpp:109-112
   int sz = (int)cnt;
   allreduce(sz);

@@ -22,6 +22,7 @@
 #include <vector>
 
 #include "../../include/plr.h"
+#include "gpu_turn.hpp"
 #include "paralg_lite.hpp"
 
 namespace plr_ps {
@@ -60,6 +61,7 @@ class ridge_regression_gpu : public paralg {
   std::vector<double> pred_z, pred_samples;
   int64_t pred_dim = 0;
   plr_ctx* gpu = nullptr;
+  gpu_turn turn;
 };
 
 }  // namespace plr_ps

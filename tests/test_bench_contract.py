@@ -79,6 +79,38 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert 0.3 < rf["frac"] < 1.0
     assert rf["traffic"] is None          # 200 000 rows: not the shard the counters were read on
     assert abs(rf["whole_step_frac"] - rf["whole_step_gbs"] / rf["peak"]) < 1e-12
+    assert rf["read_probe_gbs"] > 0 and rf["copy_probe_gbs"] > 0
+    assert out["config"]["kernel"].startswith("shard_pass<8,4,1,4")
     cb = out["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["sample"]
     assert cb["cores"] <= cb["host_cpu_count"] and cb["cores"] <= 16
+
+
+@pytest.mark.gpu
+def test_the_default_run_fits_what_the_harness_keeps():
+    # the default run: headline + the other configurations, config 5 through the parameter
+    # server with 1, 2 and 4 workers, the loader, the other shapes -- ONE line, short enough
+    # that nothing falls off the front of a log that keeps its last few KB
+    r = subprocess.run([sys.executable, BENCH, "--steps", "3", "--warmup", "1"],
+                       capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stderr[-3000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    assert len(lines[0]) < 6144, len(lines[0])
+    out = json.loads(lines[0])
+    assert out["config"]["workload"] == "c2_headline_1m_x_1000" and out["steps"] == 3
+    cols = out["row_cols"]
+    for name in ("c1_dense_100k_x_100", "c3_tall_10m_x_256", "c4_wide_200k_x_16384",
+                 "c4b_wide_200k_x_16385", "c5_e2e_2m_x_512"):
+        row = out["per_config"][name]
+        assert len(row) == len(cols) and row[cols.index("kernel_ms")] > 0, (name, row)
+        assert row[cols.index("cpu_steps_per_s_16")] > 0
+    for name, row in out["other_shapes"].items():
+        assert len(row) == len(cols) and 0.3 < row[cols.index("frac")] < 1.0, (name, row)
+    assert "x_wide_75k_x_20000" in out["other_shapes"]
+    ps = out["c5_via_ps"]
+    assert [r[0] for r in ps["rows"]] == [1, 2, 4]
+    for r_ in ps["rows"]:
+        assert r_[1] > 0 and r_[4] <= 1e-8, r_
+    assert out["c1_latency_us"]["train_dgd_per_round"] > 0
+    assert out["c5_text_to_shard"]["text_gb_per_s"] > 0
