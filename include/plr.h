@@ -160,11 +160,20 @@ int plr_predict_linear(plr_ctx* ctx, const double* theta, double* z_out);
  *   dy     n labels;   dtheta  d doubles
  *   dout   d + 1 doubles: gsum as plr_loss_grad defines it, then loss_sum
  *   flags  a PLR_LOSS_* value
+ * dX must be 16-byte aligned (the pass loads 16 bytes per lane), the other
+ * pointers 8-byte aligned.
  * The work is enqueued on `hip_stream` (a hipStream_t; NULL = the default
  * stream) and the call returns without waiting: dout is valid once the stream
  * has reached that point.  All calls on one GPU share that GPU's static array,
  * so calls that may overlap on a GPU (different streams, different threads)
- * race; order them on one stream.  Errors are described by
+ * race; order them on one stream.
+ * The first call on a device looks up the device's address of the static array
+ * and its compute units, and the first call with a given ldx on a device asks
+ * the runtime for that kernel's occupancy; both are remembered.  These
+ * look-ups are not stream work: a caller that captures a stream makes one
+ * call per ldx it will use BEFORE the capture begins; the captured calls then
+ * only enqueue kernels (no memset or copy commands).  The caller's current
+ * device is left as it was found.  Errors are described by
  * plr_last_error(NULL). */
 int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX,
                           const double* dy, int64_t n, int64_t d, int64_t ldx,
@@ -213,10 +222,24 @@ int plr_set_timing(plr_ctx* ctx, int enabled);
  *        of once by cooperating workgroups; applies from the next
  *        plr_set_data / plr_alloc_data.  Default 0.
  *   "team_spin_limit"  how many times a workgroup of the one-read wide-row
- *        pass polls for a partner's partial dot product before it gives up
- *        (the call then fails with PLR_ERR_HIP instead of hanging).  Default
- *        4194304; 0 makes every wait give up at once (used to test the
- *        failure path). */
+ *        pass polls for a partner's partial dot product before it gives up.
+ *        Default 4194304; 0 makes every wait give up at once (used to test the
+ *        paths below).
+ *   "team_fallback"  what happens when such a pass gives up -- its workgroups
+ *        must all be resident at once, which other processes or streams on the
+ *        device can prevent.  != 0 (default): the pass is run again in two
+ *        sweeps, which need no residency, and the caller gets its results; after
+ *        two such passes the resident shard stays on two sweeps
+ *        (plr_kernel_info says so).  0: the call fails with PLR_ERR_HIP.
+ *   "team_lag"  how many rows the rank-1 update of that pass trails the dot
+ *        product: 1, 2, or 0 (default) = chosen by the width.  Same results;
+ *        applies from the next plr_set_data / plr_alloc_data.
+ *   "csv_overlap"  value != 0: plr_set_data_csv parses texts of 256 MiB and
+ *        more stretch by stretch while the rest is still arriving from the
+ *        host, into a shard reserved for an estimated number of rows (a few
+ *        rows more than needed stay allocated).  Same shard.  Default 0: on
+ *        the devices measured the transfers slow down beside the kernels by
+ *        as much as the overlap gains. */
 int plr_set_option(plr_ctx* ctx, const char* key, int64_t value);
 
 /* Read ceiling of this device, measured on the resident shard: a kernel that

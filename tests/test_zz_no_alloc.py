@@ -111,3 +111,93 @@ def test_noalloc_empty_shard_and_refusals(plr, gen):
         assert e.value.code == -1 and what in str(e.value), str(e.value)
     with pytest.raises(PlrError):
         capi.loss_grad_noalloc(dX.ptr, dy.ptr, 4, 100, 128, None, dout.ptr)
+
+
+def _free_bytes(hip):
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def test_noalloc_leaves_device_memory_as_it_found_it(plr, gen):
+    # what the name promises: once the first call on the device has looked up the static
+    # array, calls neither take nor return device memory, whatever their size
+    from paracel_amd import PlrError, capi
+
+    hip = DevBuf.hip()
+    hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    rng = np.random.default_rng(3)
+    n, d, ldx = 5000, 300, 384
+    X = rng.normal(size=(n, d)) / np.sqrt(d)
+    y = (rng.random(n) < 0.5) * 1.0
+    dX, dy, dth, dout = _device_inputs(X, y, rng.normal(size=d), ldx)
+    capi.loss_grad_noalloc(dX.ptr, dy.ptr, n, d, ldx, dth.ptr, dout.ptr)   # first call: set-up
+    assert hip.hipDeviceSynchronize() == 0
+    before = _free_bytes(hip)
+    for rows, cols, pitch, flags in ((n, d, ldx, 0), (n // 3, 200, ldx, 1), (17, d, ldx, 3),
+                                     (0, d, ldx, 0), (n, d, ldx, 2)):
+        capi.loss_grad_noalloc(dX.ptr, dy.ptr, rows, cols, pitch, dth.ptr, dout.ptr, flags)
+    assert hip.hipDeviceSynchronize() == 0
+    assert _free_bytes(hip) == before
+    # the pass loads X 16 bytes per lane: a pointer that is not 16-byte aligned is refused
+    with pytest.raises(PlrError) as e:
+        capi.loss_grad_noalloc(dX.ptr + 8, dy.ptr, n - 1, d, ldx, dth.ptr, dout.ptr)
+    assert e.value.code == -1 and "16-byte aligned" in str(e.value)
+    for b in (dX, dy, dth, dout):
+        b.free()
+
+
+def test_noalloc_under_stream_capture(plr, gen):
+    # the caller it is for: a stream under capture.  The first call per device and pitch (the
+    # look-ups) is made before the capture begins; the captured call then only enqueues
+    # kernels.  The graph is replayed several times, with eager work and synchronisations in
+    # between, and every replay must give the eager call's bits.
+    from paracel_amd import capi
+
+    hip = DevBuf.hip()
+    for f, args in (("hipStreamCreate", [C.POINTER(C.c_void_p)]),
+                    ("hipStreamBeginCapture", [C.c_void_p, C.c_int]),
+                    ("hipStreamEndCapture", [C.c_void_p, C.POINTER(C.c_void_p)]),
+                    ("hipGraphInstantiate", [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p,
+                                             C.c_char_p, C.c_size_t]),
+                    ("hipGraphLaunch", [C.c_void_p, C.c_void_p]),
+                    ("hipStreamSynchronize", [C.c_void_p]),
+                    ("hipGraphExecDestroy", [C.c_void_p]), ("hipGraphDestroy", [C.c_void_p]),
+                    ("hipStreamDestroy", [C.c_void_p])):
+        getattr(hip, f).argtypes = args
+    rng = np.random.default_rng(8)
+    n, d, ldx = 9000, 500, 512
+    X = rng.normal(size=(n, d)) / np.sqrt(d)
+    y = (rng.random(n) < 0.5) * 1.0
+    theta = rng.normal(size=d)
+    dX, dy, dth, dout = _device_inputs(X, y, theta, ldx)
+    stream = C.c_void_p()
+    assert hip.hipStreamCreate(C.byref(stream)) == 0
+    # eager, on the same stream: the reference bits, and the set-up of this device and pitch
+    capi.loss_grad_noalloc(dX.ptr, dy.ptr, n, d, ldx, dth.ptr, dout.ptr, stream=stream.value)
+    assert hip.hipStreamSynchronize(stream) == 0
+    want = dout.numpy()
+    assert np.all(np.isfinite(want))
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 0) == 0          # hipStreamCaptureModeGlobal
+    try:
+        capi.loss_grad_noalloc(dX.ptr, dy.ptr, n, d, ldx, dth.ptr, dout.ptr, stream=stream.value)
+    finally:
+        rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+    assert rc == 0 and graph.value
+    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+    poison = np.full(d + 1, np.nan)
+    for replay in range(4):
+        assert hip.hipMemcpy(dout.ptr, poison.ctypes.data, poison.nbytes, 1) == 0
+        assert hip.hipGraphLaunch(gexec, stream) == 0
+        assert hip.hipStreamSynchronize(stream) == 0
+        got = dout.numpy()
+        assert np.array_equal(got, want), "replay %d differs from the eager call" % replay
+        # the program's own eager work between replays: another shape through the same array
+        capi.loss_grad_noalloc(dX.ptr, dy.ptr, 333, 100, ldx, dth.ptr, dout.ptr,
+                               stream=stream.value)
+        assert hip.hipStreamSynchronize(stream) == 0
+    assert hip.hipGraphExecDestroy(gexec) == 0 and hip.hipGraphDestroy(graph) == 0
+    assert hip.hipStreamDestroy(stream) == 0
+    for b in (dX, dy, dth, dout):
+        b.free()
