@@ -119,9 +119,12 @@ void logistic_regression_gpu::dgd_learning() {
   const auto t0 = std::chrono::steady_clock::now();
   for (int rd = 0; rd < rounds; ++rd) {
     theta = paracel_read<std::vector<double> >("theta");
-    // lr.cpp:125-142 in one fused pass over the resident shard; with debug the
-    // round's loss at the theta just read is recorded (the reference records
-    // it after every sample, an O(n^2 d) loop)
+    // lr.cpp:125-142 in one fused pass over the resident shard.  With debug the
+    // reference pushes calc_loss() after EVERY sample (lr.cpp:139-141) -- theta
+    // does not change inside the round, so these are n_local copies of the
+    // global mean loss at the theta just read, which is what is recorded here
+    // (one fused pass and the two all-reduces of lr.cpp:331-335 per round
+    // instead of n_local passes)
     double loss_sum = 0.;
     {
       gpu_turn_guard mine(turn);  // several workers on the GPU: one pass at a time
@@ -129,7 +132,13 @@ void logistic_regression_gpu::dgd_learning() {
                           debug ? &loss_sum : nullptr),
             "plr_dgd_delta");
     }
-    if (debug) loss_error.push_back(n_local ? loss_sum / (double)n_local : 0.);
+    if (debug) {
+      double total = loss_sum;
+      int cnt = (int)n_local;
+      allreduce(total);
+      allreduce(cnt);
+      loss_error.insert(loss_error.end(), (size_t)n_local, cnt ? total / (double)cnt : 0.);
+    }
     paracel_sync();
     paracel_bupdate("theta", delta);
     paracel_sync();

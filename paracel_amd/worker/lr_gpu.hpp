@@ -64,7 +64,7 @@ class logistic_regression_gpu : public paralg {
   int64_t n_local = 0, data_dim = 0;
   std::vector<double> flat, labels;   // staging only
   std::vector<double> theta, theta0;
-  std::vector<double> loss_error;     // one entry per round when debug
+  std::vector<double> loss_error;     // debug: n_local entries per round (lr.cpp:139-141)
   std::vector<double> pred_h;
   std::vector<double> pred_samples;   // flattened prediction rows (lr.hpp: pred_samples)
   int64_t pred_dim = 0;

@@ -93,9 +93,17 @@ def test_csv_driver_follows_the_reference_call_order(server_info, oracle, tmp_pa
     np.testing.assert_allclose(pred, oracle.predict(X, theta_ref), atol=5.1e-7, rtol=0)
     xs = np.array([[float(t) for t in l.split(":")[0].split(",")] for l in plines])
     np.testing.assert_allclose(xs, X, atol=5.1e-7, rtol=0)
-    # debug: one loss per round, at the theta read at the start of that round
+    # debug: the loss after every sample of every round (lr.cpp:139-141, 341-343) -- n equal
+    # entries per round, the mean loss at the theta read at the start of that round
     curve = np.array([float(t) for t in (outdir / "lr_loss_error_0").read_text().split()])
-    assert curve.shape == (20,) and abs(curve[0] - np.log(2)) < 1e-6 and curve[-1] < curve[0]
+    assert curve.shape == (20 * n,)
+    per_round = curve.reshape(20, n)
+    assert np.all(per_round == per_round[:, :1])
+    assert abs(per_round[0, 0] - np.log(2)) < 1e-6 and per_round[-1, 0] < per_round[0, 0]
+    th = np.zeros(k + 1)
+    for rd in range(20):
+        assert abs(per_round[rd, 0] - oracle.calc_loss(X, y, th)) <= 5.1e-7
+        th = th + oracle.dgd_delta(X, y, th, 0.001, 0.01)
 
     # the first run parsed the training text on the device and wrote the binary shard cache
     assert "parsed on the device: 400 x 7" in r.stdout and "lines got: 400" in r.stdout
