@@ -84,7 +84,9 @@ int plr_set_data_chunk(plr_ctx* ctx, int64_t row0, int64_t nrows,
  * std::stod rejects, a line with another number of fields) come back as
  * PLR_ERR_INVALID with the line number; lines of a single field are refused
  * with PLR_ERR_UNSUPPORTED.  The text is copied; the caller keeps it.
- * (plr_get_timing's last_ms afterwards: the duration of the parsing kernel.) */
+ * (plr_get_timing's last_ms afterwards: the duration of the parsing kernel;
+ * for a text parsed while it arrived, option "csv_overlap", the time from the
+ * first stretch's kernels to the last one's.) */
 int plr_set_data_csv(plr_ctx* ctx, const char* const* text, const int64_t* len,
                      int nspans, char sep, int64_t* n_out, int64_t* d_out);
 
@@ -214,9 +216,6 @@ int plr_set_timing(plr_ctx* ctx, int enabled);
  *        have given.  The upload checks the statement row by row and fails
  *        with PLR_ERR_INVALID at the first row that does not start with 1.0.
  *        Applies from the next plr_set_data / plr_alloc_data.  Default 0.
- *   "csv_lane_per_row"  which kernel plr_set_data_csv parses with: 1 a lane
- *        per row (64 rows per wave), 0 a wave per row, -1 (default) by the
- *        number of rows.  Same results either way.
  *   "column_blocks_two_sweeps"  value != 0: rows wider than 19456 columns are
  *        processed in two sweeps over X (dot products, then updates) instead
  *        of once by cooperating workgroups; applies from the next
@@ -234,12 +233,12 @@ int plr_set_timing(plr_ctx* ctx, int enabled);
  *   "team_lag"  how many rows the rank-1 update of that pass trails the dot
  *        product: 1, 2, or 0 (default) = chosen by the width.  Same results;
  *        applies from the next plr_set_data / plr_alloc_data.
- *   "csv_overlap"  value != 0: plr_set_data_csv parses texts of 256 MiB and
- *        more stretch by stretch while the rest is still arriving from the
- *        host, into a shard reserved for an estimated number of rows (a few
- *        rows more than needed stay allocated).  Same shard.  Default 0: on
- *        the devices measured the transfers slow down beside the kernels by
- *        as much as the overlap gains. */
+ *   "csv_overlap"  value != 0 (default): plr_set_data_csv parses texts of
+ *        256 MiB and more stretch by stretch while the rest is still arriving
+ *        from the host, into a shard reserved for an estimated number of rows
+ *        (a few rows more than needed stay allocated; when the estimate is too
+ *        low the call starts over with 0's way).  0: transfer, count the rows,
+ *        reserve exactly that shard, parse.  Same shard contents. */
 int plr_set_option(plr_ctx* ctx, const char* key, int64_t value);
 
 /* Read ceiling of this device, measured on the resident shard: a kernel that

@@ -260,9 +260,8 @@ struct plr_ctx {
   int64_t part_len = 0;           // entries of d_part_loss and d_part_res
   std::string base_info;          // kernel description without the give-up note
   bool opt_two_sweeps = false;  // plr_set_option("column_blocks_two_sweeps")
-  bool opt_csv_overlap = false;  // plr_set_option("csv_overlap")
+  bool opt_csv_overlap = true;  // plr_set_option("csv_overlap")
   bool synth_first_col = false; // the shard being reserved comes from plr_set_data_csv
-  int opt_csv_lane_rows = -1;   // plr_set_option("csv_lane_per_row"): -1 by row count, 0, 1
   int csv_slow_fields = 0;      // fields of the last plr_set_data_csv the host converted
   bool team_check = false;      // a team pass ran since the status word was last read
   double* d_z = nullptr;        // n: blocked rows only, x.theta accumulated over the blocks
@@ -1167,33 +1166,10 @@ static int resolve_slow_fields(plr_ctx* c, const CsvText& ct, int64_t d, char se
 constexpr int kCsvSlowCap = 1 << 20;
 constexpr int kCsvRetrySerial = 1;  // the pipelined parse leaves the input to the serial one
 
-static plr::CsvArgs csv_args(plr_ctx* c, const unsigned char* dt, int64_t total,
-                             const int64_t* rows, int64_t n, int64_t d, char sep,
-                             plr::CsvSlow* slow, int64_t* ctl) {
-  plr::CsvArgs ca;
-  ca.text = dt;
-  ca.len = total;
-  ca.row_start = rows;
-  ca.n = n;
-  ca.row_range = nullptr;
-  ca.d = (int)d;
-  ca.sep = (unsigned char)sep;
-  ca.X = c->dX;
-  ca.y = c->dy;
-  ca.pitch = c->pitch;
-  ca.np = c->lane ? c->lane->np : 0;
-  ca.slow = slow;
-  ca.slow_cap = kCsvSlowCap;
-  ca.slow_count = reinterpret_cast<unsigned long long*>(ctl + 2);
-  ca.bad_row = reinterpret_cast<long long*>(ctl + 1);
-  ca.flush_at = 52;  // of 64 lanes (sweep: 32..64 within 3 %, 1 is 40 % slower)
-  return ca;
-}
-
 // What both parses end with: the parser's verdict, the fields left to the
 // host, the description.
 static int finish_csv(plr_ctx* c, const CsvText& ct, int64_t d, char sep, const int64_t res[3],
-                      const void* d_slow, bool lane_rows, const char* how) {
+                      const void* d_slow, const char* parser, const char* how = "") {
   if (res[1] != INT64_MAX)  // parse_lines' message for the same input
     return fail(c, PLR_ERR_INVALID, "ragged sample line " + std::to_string(res[1]));
   if (res[2] > (int64_t)kCsvSlowCap)
@@ -1203,8 +1179,8 @@ static int finish_csv(plr_ctx* c, const CsvText& ct, int64_t d, char sep, const 
   const int rc = resolve_slow_fields(c, ct, d, sep, nslow, d_slow);
   if (rc != PLR_OK) return rc;
   c->csv_slow_fields = nslow;
-  c->info += std::string("; parsed from text") + how + " (a " + (lane_rows ? "lane" : "wave") +
-             " per row), " + std::to_string(nslow) + " fields converted on the host";
+  c->info += std::string("; parsed from text") + how + " (" + parser + "), " +
+             std::to_string(nslow) + " fields converted on the host";
   c->base_info = c->info;
   if (c->timing) {  // plr_get_timing's last_ms: the parsing kernel(s)
     float ms = 0.f;
@@ -1214,10 +1190,34 @@ static int finish_csv(plr_ctx* c, const CsvText& ct, int64_t d, char sep, const 
   return PLR_OK;
 }
 
+static plr::CsvFieldArgs csv_field_args(plr_ctx* c, const unsigned char* dt,
+                                        const int64_t* first_row, const int64_t* first_field,
+                                        int64_t rows_cap, int64_t d, char sep, plr::CsvSlow* slow,
+                                        int64_t* ctl) {
+  plr::CsvFieldArgs fa;
+  fa.text = dt;
+  fa.first_row = first_row;
+  fa.first_field = first_field;
+  fa.block0 = 0;
+  fa.rows_cap = rows_cap;
+  fa.d = (int)d;
+  fa.sep = (unsigned char)sep;
+  fa.inv_d = 1.0 / (double)d;
+  fa.X = c->dX;
+  fa.y = c->dy;
+  fa.pitch = c->pitch;
+  fa.np = c->lane ? c->lane->np : 0;
+  fa.slow = slow;
+  fa.slow_cap = kCsvSlowCap;
+  fa.slow_count = reinterpret_cast<unsigned long long*>(ctl + 2);
+  fa.bad_row = reinterpret_cast<long long*>(ctl + 1);
+  return fa;
+}
+
 // Transfer, then parse: the whole text goes to the device, the rows are counted
 // (the host learns n and reserves exactly that shard), then located and parsed.
 static int csv_serial(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int64_t* n_out) {
-  DevBuf d_text, d_counts, d_first, d_rows, d_slow, d_ctl;
+  DevBuf d_text, d_slow, d_ctl;
   const int64_t total = ct.total;
   if (hipMalloc(&d_text.p, (size_t)ct.padded) != hipSuccess) {
     (void)hipGetLastError();
@@ -1235,23 +1235,31 @@ static int csv_serial(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int64_
   }
   PLR_HIP(c, hipMemsetAsync(dt + total, '\n', (size_t)(ct.padded - total), c->stream));
 
-  // rows: count, running sum, offsets
   const int64_t nblocks = (total + plr::kCsvBlockBytes - 1) / plr::kCsvBlockBytes;
   if (nblocks > (int64_t)INT32_MAX) return fail(c, PLR_ERR_INVALID, "sample text too large");
-  PLR_HIP(c, hipMalloc(&d_counts.p, (size_t)nblocks * sizeof(int)));
-  PLR_HIP(c, hipMalloc(&d_first.p, (size_t)nblocks * sizeof(int64_t)));
-  PLR_HIP(c, hipMalloc(&d_ctl.p, 4 * sizeof(int64_t)));  // [0] rows, [1] bad row, [2] slow fields
+
+  // rows and fields per block, and what lies in front of every block
+  DevBuf d_rcount, d_fcount, d_frow, d_ffield;
+  PLR_HIP(c, hipMalloc(&d_rcount.p, (size_t)nblocks * sizeof(int)));
+  PLR_HIP(c, hipMalloc(&d_fcount.p, (size_t)nblocks * sizeof(int)));
+  PLR_HIP(c, hipMalloc(&d_frow.p, (size_t)nblocks * sizeof(int64_t)));
+  PLR_HIP(c, hipMalloc(&d_ffield.p, (size_t)nblocks * sizeof(int64_t)));
+  PLR_HIP(c, hipMalloc(&d_ctl.p, 4 * sizeof(int64_t)));  // rows, bad row, slow fields, fields
   int64_t* ctl = static_cast<int64_t*>(d_ctl.p);
-  PLR_HIP(c, hipMemsetAsync(ctl, 0, 4 * sizeof(int64_t), c->stream));
-  hipLaunchKernelGGL(plr::csv_count_rows, dim3((unsigned)nblocks), dim3(plr::kCsvThreads), 0,
-                     c->stream, dt, total, static_cast<int*>(d_counts.p), (int64_t)0);
-  hipLaunchKernelGGL(plr::csv_scan_counts, dim3(1), dim3(1024), 0, c->stream,
-                     static_cast<const int*>(d_counts.p), nblocks,
-                     static_cast<int64_t*>(d_first.p), ctl, static_cast<int64_t*>(nullptr));
+  const int64_t ctl_init[4] = {0, INT64_MAX, 0, 0};
+  PLR_HIP(c, hipMemcpyAsync(ctl, ctl_init, sizeof ctl_init, hipMemcpyHostToDevice, c->stream));
+  hipLaunchKernelGGL(plr::csv_count_blocks, dim3((unsigned)nblocks), dim3(plr::kCsvThreads), 0,
+                     c->stream, dt, (unsigned char)sep, static_cast<int*>(d_rcount.p),
+                     static_cast<int*>(d_fcount.p), (int64_t)0);
+  hipLaunchKernelGGL(plr::csv_scan_blocks, dim3(1), dim3(1024), 0, c->stream,
+                     static_cast<const int*>(d_rcount.p), static_cast<const int*>(d_fcount.p),
+                     nblocks, static_cast<int64_t*>(d_frow.p), static_cast<int64_t*>(d_ffield.p),
+                     ctl);
   PLR_HIP(c, hipGetLastError());
-  int64_t n = 0;
-  PLR_HIP(c, hipMemcpyAsync(&n, ctl, sizeof n, hipMemcpyDeviceToHost, c->stream));
+  int64_t tot[4] = {0, 0, 0, 0};
+  PLR_HIP(c, hipMemcpyAsync(tot, ctl, sizeof tot, hipMemcpyDeviceToHost, c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
+  const int64_t n = tot[0], nfields = tot[3];
   if (n_out) *n_out = n;
 
   // the shard: k = d - 1 feature columns; the sample's constant first column is
@@ -1261,32 +1269,21 @@ static int csv_serial(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int64_
   int rc = alloc_shape_buffers(c, n, d, /*zero_fill=*/false);
   c->synth_first_col = false;
   if (rc != PLR_OK) return rc;
-  PLR_HIP(c, hipMalloc(&d_rows.p, (size_t)std::max<int64_t>(n, 1) * sizeof(int64_t)));
-  hipLaunchKernelGGL(plr::csv_row_starts, dim3((unsigned)nblocks), dim3(plr::kCsvThreads), 0,
-                     c->stream, dt, total, static_cast<const int64_t*>(d_first.p),
-                     static_cast<int64_t*>(d_rows.p), (int64_t)0, n);
-  PLR_HIP(c, hipGetLastError());
-
   PLR_HIP(c, hipMalloc(&d_slow.p, (size_t)kCsvSlowCap * sizeof(plr::CsvSlow)));
-  const int64_t ctl_init[3] = {n, INT64_MAX, 0};
-  PLR_HIP(c, hipMemcpyAsync(ctl, ctl_init, sizeof ctl_init, hipMemcpyHostToDevice, c->stream));
-  const plr::CsvArgs ca = csv_args(c, dt, total, static_cast<const int64_t*>(d_rows.p), n, d, sep,
-                                   static_cast<plr::CsvSlow*>(d_slow.p), ctl);
-  // many rows: a lane per row (every lane in the character step); few rows: a wave per row
-  const bool lane_rows = c->opt_csv_lane_rows < 0 ? n >= (int64_t)c->num_cu * 4 * 64 * 2
-                                                  : c->opt_csv_lane_rows != 0;
-  const int64_t want = lane_rows ? (n + 255) / 256 : (n + 3) / 4;
-  const unsigned grid = (unsigned)std::min<int64_t>(
-      std::max<int64_t>(want, 1), (int64_t)c->num_cu * 8);
+  plr::CsvFieldArgs fa = csv_field_args(c, dt, static_cast<const int64_t*>(d_frow.p),
+                                        static_cast<const int64_t*>(d_ffield.p), n, d, sep,
+                                        static_cast<plr::CsvSlow*>(d_slow.p), ctl);
   if (c->timing) PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
-  hipLaunchKernelGGL(lane_rows ? plr::csv_parse_rows : plr::csv_parse, dim3(grid), dim3(256), 0,
-                     c->stream, ca);
+  hipLaunchKernelGGL(plr::csv_parse_fields, dim3((unsigned)nblocks), dim3(plr::kCsvThreads), 0,
+                     c->stream, fa);
   PLR_HIP(c, hipGetLastError());
   if (c->timing) PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
-  int64_t res[3] = {0, 0, 0};
+  int64_t res[4] = {0, 0, 0, 0};
   PLR_HIP(c, hipMemcpyAsync(res, ctl, sizeof res, hipMemcpyDeviceToHost, c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
-  return finish_csv(c, ct, d, sep, res, d_slow.p, lane_rows, "");
+  // the line-start checks cover every row but the last
+  if (res[1] == INT64_MAX && nfields != n * d) res[1] = n - 1;
+  return finish_csv(c, ct, d, sep, res, d_slow.p, "a lane per field");
 }
 
 // Lines per byte from a sample of the text: the lengths of up to 256 lines at
@@ -1317,51 +1314,31 @@ static double sampled_line_bytes(const CsvText& ct) {
   return cnt ? sum / (double)cnt : 0.;
 }
 
-// Device offset of the first newline at or behind device offset `off`.
-static int64_t newline_at_or_after(const CsvText& ct, int64_t off) {
-  int s = 0;
-  while (s + 1 < ct.nspans && off >= ct.span_at[s + 1]) ++s;
-  const int64_t p = off - ct.span_at[s];
-  if (p < ct.len[s]) {
-    const void* nl = memchr(ct.text[s] + p, '\n', (size_t)(ct.len[s] - p));
-    if (nl) return ct.span_at[s] + (static_cast<const char*>(nl) - ct.text[s]);
-  }
-  return ct.span_at[s] + ct.len[s];  // the newline behind the span
-}
-
 struct LaneProgress;
 static int lanes_in(plr_ctx* c, const std::vector<InJob>& jobs, const FillFn& fill,
                     const SentFn& sent, const char* what, LaneProgress* prog,
                     const std::function<int()>* conductor);
 
 // Parse while the text arrives.  The text crosses the host link in 4 MiB blocks
-// on the copy lanes; cut into stretches, every stretch is counted, located and
-// parsed on the context's stream as soon as it and the end of its last row
-// are on the device -- so the parser works in the shadow of the transfer and
-// only the last stretch's kernels are left when the last byte has arrived.
-// A wave of the lane-per-row parser walks 64 whole rows in lockstep, which on
-// rows of kilobytes takes it milliseconds however few rows there are; it pays
-// when some thousands of waves are in flight -- 262144 rows or more.  A stretch
-// (64 MiB, the last one 16 MiB) with fewer rows goes to the wave-per-row
-// parser, whose waves are done with a row in tens of microseconds and which
-// still parses faster than the host link delivers (measured on rows of 512
-// six-decimal fields: 62 GB/s of text against 50).
+// on the copy lanes; cut into stretches (64 MiB, the last one 16 MiB), every
+// stretch is counted, scanned and parsed on the context's stream as soon as it
+// and the 64 bytes behind it are on the device -- so the parser works in the
+// shadow of the transfer and only the last stretch's kernels are left when the
+// last byte has arrived.  The per-block parser does not care how few rows a
+// stretch holds: a stretch of 16 MiB is 4096 workgroups.
 // The shard has to exist before the number of rows is known: it is reserved
 // for an estimate from the lengths of sampled lines plus 1/64 and 4096 rows;
 // the few rows reserved in excess stay allocated.  Whenever that does not work
 // out -- more rows than reserved, no memory for the generous shard -- the call
 // falls back to csv_serial (kCsvRetrySerial; nothing is left behind).
-// Off unless plr_set_option("csv_overlap", 1).  Measured on 1.96 GB of text
-// (rows of 512 six-decimal fields): the kernels do keep pace -- the stream has
-// drained 0.03 ms after the last block has landed -- but the transfer itself
-// takes 41-63 ms beside them instead of the 36-41 ms it takes alone (the copy
-// lanes' streams and the kernels' stream share the device's few hardware
-// queues, and a block queued behind a kernel waits for it; with the kernels
-// dealt over the lanes' own streams, or the lanes sharing two or three
-// streams, 41-61 ms), so that the whole call is 44-62 ms against 48-53 ms for
-// transfer-then-parse: no gain that could be relied on.
+// plr_set_option("csv_overlap", 0) switches it off.  Measured on 1.96 GB of
+// text (rows of 512 six-decimal fields), the two alternating in one process,
+// 12 calls each: median 39.0 ms against 45.3 ms for transfer-then-parse (the
+// count and the parse, 5.7 ms, gone from the critical path).  The transfer
+// itself is a little slower beside the kernels than alone: the copy lanes'
+// streams and the kernels' stream share the device's few hardware queues, and
+// a block queued behind a kernel waits for it.
 constexpr int64_t kCsvStretch = 64ll << 20, kCsvLastStretch = 16ll << 20;
-constexpr int64_t kCsvLaneRowsMin = 4 * 1024 * 64;  // rows that fill the device's SIMDs 4 deep
 static_assert(kCsvLastStretch % (int64_t)kCopyBlock == 0 &&
                   (int64_t)kCopyBlock % plr::kCsvBlockBytes == 0,
               "a stretch is whole copy blocks and whole counting blocks");
@@ -1387,19 +1364,17 @@ static int csv_pipelined(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int
   // stretch boundaries (multiples of the copy block, so of the counting block)
   std::vector<int64_t> bound(1, 0);
   {
-    const int64_t S = kCsvStretch;
     const int64_t last = (total - kCsvLastStretch) / (int64_t)kCopyBlock * (int64_t)kCopyBlock;
-    for (int64_t b = S; b + S / 2 < last; b += S) bound.push_back(b);
+    for (int64_t b = kCsvStretch; b + kCsvStretch / 2 < last; b += kCsvStretch) bound.push_back(b);
     if (last > bound.back()) bound.push_back(last);
     bound.push_back(total);
   }
   const int64_t nslabs = (int64_t)bound.size() - 1;
-  DevBuf d_text, d_counts, d_first, d_rows, d_slow, d_ctl;
-  auto no_room = [&]() {
+  DevBuf d_text, d_rcount, d_fcount, d_frow, d_ffield, d_slow, d_ctl;
+  if (hipMalloc(&d_text.p, (size_t)ct.padded) != hipSuccess) {
     (void)hipGetLastError();
     return kCsvRetrySerial;
-  };
-  if (hipMalloc(&d_text.p, (size_t)ct.padded) != hipSuccess) return no_room();
+  }
   unsigned char* dt = static_cast<unsigned char*>(d_text.p);
   for (int s = 0; s < ct.nspans; ++s)
     PLR_HIP(c, hipMemsetAsync(dt + ct.span_at[s] + ct.len[s], '\n', 1, c->stream));
@@ -1422,8 +1397,7 @@ static int csv_pipelined(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int
     PLR_HIP(c, hipEventCreateWithFlags(&prog.done[j], hipEventDisableTiming));
   for (int l = 0; l < kCopyLanes; ++l) prog.issued[l].store(0);
 
-  int64_t res[3] = {0, INT64_MAX, 0};
-  bool lane_rows = false, any_by_lane = false;
+  int64_t res[4] = {0, INT64_MAX, 0, 0};
   int fallback = 0;  // set by the conductor: leave the input to csv_serial
   const std::function<int()> conductor = [&]() -> int {
     // (runs on the calling thread while the lanes move the text)
@@ -1435,29 +1409,27 @@ static int csv_pipelined(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int
       return PLR_OK;
     }
     if (rc != PLR_OK) return rc;
-    if (hipMalloc(&d_counts.p, (size_t)nblocks * sizeof(int)) != hipSuccess ||
-        hipMalloc(&d_first.p, (size_t)nblocks * sizeof(int64_t)) != hipSuccess ||
-        hipMalloc(&d_rows.p, (size_t)cap * sizeof(int64_t)) != hipSuccess ||
+    if (hipMalloc(&d_rcount.p, (size_t)nblocks * sizeof(int)) != hipSuccess ||
+        hipMalloc(&d_fcount.p, (size_t)nblocks * sizeof(int)) != hipSuccess ||
+        hipMalloc(&d_frow.p, (size_t)nblocks * sizeof(int64_t)) != hipSuccess ||
+        hipMalloc(&d_ffield.p, (size_t)nblocks * sizeof(int64_t)) != hipSuccess ||
         hipMalloc(&d_slow.p, (size_t)kCsvSlowCap * sizeof(plr::CsvSlow)) != hipSuccess ||
-        hipMalloc(&d_ctl.p, (size_t)(4 + 2 * nslabs) * sizeof(int64_t)) != hipSuccess) {
+        hipMalloc(&d_ctl.p, 4 * sizeof(int64_t)) != hipSuccess) {
       (void)hipGetLastError();
       fallback = 1;
       return PLR_OK;
     }
-    int64_t* ctl = static_cast<int64_t*>(d_ctl.p);  // [0] rows so far, [1] bad row, [2] slow fields
-    int64_t* ranges = ctl + 4;                       // [stretch][2]: its rows
+    int64_t* ctl = static_cast<int64_t*>(d_ctl.p);  // rows so far, bad row, slow fields, fields so far
     const int64_t ctl_init[4] = {0, INT64_MAX, 0, 0};
     PLR_HIP(c, hipMemcpyAsync(ctl, ctl_init, sizeof ctl_init, hipMemcpyHostToDevice, c->stream));
-    plr::CsvArgs ca = csv_args(c, dt, total, static_cast<const int64_t*>(d_rows.p), cap, d, sep,
-                               static_cast<plr::CsvSlow*>(d_slow.p), ctl);
-    lane_rows = c->opt_csv_lane_rows > 0;  // forced; otherwise by the rows of a stretch
+    plr::CsvFieldArgs fa = csv_field_args(c, dt, static_cast<const int64_t*>(d_frow.p),
+                                          static_cast<const int64_t*>(d_ffield.p), cap, d, sep,
+                                          static_cast<plr::CsvSlow*>(d_slow.p), ctl);
     size_t ready = 0;  // jobs [0, ready) are behind the context's stream already
     for (int64_t s = 0; s < nslabs; ++s) {
-      hipStream_t cs = c->stream;
-      // what this stretch needs on the device: itself, and the row that starts
-      // last in it to its end, plus what the parser reads ahead
-      const int64_t need = std::min<int64_t>(
-          total, newline_at_or_after(ct, bound[s + 1] - 1) + 1 + plr::kCsvPadBytes);
+      // what this stretch needs on the device: itself and what a field that starts at its
+      // end may still read
+      const int64_t need = std::min<int64_t>(total, bound[s + 1] + plr::kCsvPadBytes);
       size_t upto = ready;
       while (upto < jobs.size() && job_end[upto] - (int64_t)jobs[upto].bytes < need) ++upto;
       for (int l = 0; l < kCopyLanes; ++l) {
@@ -1468,31 +1440,23 @@ static int csv_pipelined(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int
           std::this_thread::sleep_for(std::chrono::microseconds(20));
         }
         if (mine > 0 && (size_t)l + (mine - 1) * kCopyLanes >= ready)
-          PLR_HIP(c, hipStreamWaitEvent(cs, prog.done[l + (mine - 1) * kCopyLanes], 0));
+          PLR_HIP(c, hipStreamWaitEvent(c->stream, prog.done[l + (mine - 1) * kCopyLanes], 0));
       }
       ready = upto;
       const int64_t b0 = bound[s] / plr::kCsvBlockBytes;
       const int64_t nb = ceil_div(bound[s + 1], (int64_t)plr::kCsvBlockBytes) - b0;
-      if (s == 0 && c->timing) PLR_HIP(c, hipEventRecord(c->ev0, cs));
-      hipLaunchKernelGGL(plr::csv_count_rows, dim3((unsigned)nb), dim3(plr::kCsvThreads), 0,
-                         cs, dt, total, static_cast<int*>(d_counts.p), b0);
-      hipLaunchKernelGGL(plr::csv_scan_counts, dim3(1), dim3(1024), 0, cs,
-                         static_cast<const int*>(d_counts.p) + b0, nb,
-                         static_cast<int64_t*>(d_first.p) + b0, ctl, ranges + 2 * s);
-      hipLaunchKernelGGL(plr::csv_row_starts, dim3((unsigned)nb), dim3(plr::kCsvThreads), 0,
-                         cs, dt, total, static_cast<const int64_t*>(d_first.p),
-                         static_cast<int64_t*>(d_rows.p), b0, cap);
-      ca.row_range = ranges + 2 * s;
-      // rows of this stretch, roughly
-      const int64_t rows = std::max<int64_t>(
-          1, (int64_t)((double)(bound[s + 1] - bound[s]) / line_bytes));
-      const bool by_lane = c->opt_csv_lane_rows < 0 ? rows >= kCsvLaneRowsMin : lane_rows;
-      any_by_lane = any_by_lane || by_lane;
-      const int64_t want = by_lane ? (rows + 255) / 256 : (rows + 3) / 4;
-      const unsigned pgrid = (unsigned)std::min<int64_t>(std::max<int64_t>(want, 1),
-                                                         (int64_t)c->num_cu * 8);
-      hipLaunchKernelGGL(by_lane ? plr::csv_parse_rows : plr::csv_parse, dim3(pgrid), dim3(256), 0,
-                         cs, ca);
+      if (s == 0 && c->timing) PLR_HIP(c, hipEventRecord(c->ev0, c->stream));
+      hipLaunchKernelGGL(plr::csv_count_blocks, dim3((unsigned)nb), dim3(plr::kCsvThreads), 0,
+                         c->stream, dt, (unsigned char)sep, static_cast<int*>(d_rcount.p),
+                         static_cast<int*>(d_fcount.p), b0);
+      hipLaunchKernelGGL(plr::csv_scan_blocks, dim3(1), dim3(1024), 0, c->stream,
+                         static_cast<const int*>(d_rcount.p) + b0,
+                         static_cast<const int*>(d_fcount.p) + b0, nb,
+                         static_cast<int64_t*>(d_frow.p) + b0,
+                         static_cast<int64_t*>(d_ffield.p) + b0, ctl);
+      fa.block0 = b0;
+      hipLaunchKernelGGL(plr::csv_parse_fields, dim3((unsigned)nb), dim3(plr::kCsvThreads), 0,
+                         c->stream, fa);
       PLR_HIP(c, hipGetLastError());
     }
     if (c->timing) PLR_HIP(c, hipEventRecord(c->ev1, c->stream));
@@ -1513,6 +1477,7 @@ static int csv_pipelined(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int
   // the exact shape: n rows of the cap reserved; variant, grid and workspace for n
   const int64_t n = res[0];
   if (n_out) *n_out = n;
+  if (res[1] == INT64_MAX && res[3] != n * d) res[1] = n - 1;  // the last row's field count
   if (c->lane && n < c->n_alloc) {
     // the row-tiled layout's last group: its rows past n must read as zeros
     const int64_t group = (int64_t)plr::kWave * c->lane->U;
@@ -1530,7 +1495,7 @@ static int csv_pipelined(plr_ctx* c, const CsvText& ct, int64_t d, char sep, int
   c->bias_slot = c->theta_len;
   rc = alloc_workspace(c);
   if (rc != PLR_OK) return rc;
-  return finish_csv(c, ct, d, sep, res, d_slow.p, any_by_lane, " while it arrived");
+  return finish_csv(c, ct, d, sep, res, d_slow.p, "a lane per field", " while it arrived");
 }
 
 int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, int nspans,
@@ -1550,7 +1515,9 @@ int plr_set_data_csv(plr_ctx* c, const char* const* text, const int64_t* len, in
     ct.span_at[s + 1] = ct.span_at[s] + len[s] + 1;  // a newline behind every span
   }
   ct.total = ct.span_at[nspans];
-  ct.padded = (ct.total + 15) / 16 * 16 + plr::kCsvPadBytes;
+  // (whole counting blocks, then the pad the parsers may read ahead into)
+  ct.padded = ceil_div(ct.total, (int64_t)plr::kCsvBlockBytes) * plr::kCsvBlockBytes +
+              plr::kCsvPadBytes;
   const int64_t d = first_line_fields(text, len, nspans, sep);
   if (n_out) *n_out = 0;
   if (d_out) *d_out = d;
@@ -2125,10 +2092,6 @@ int plr_set_option(plr_ctx* c, const char* key, int64_t value) {
   }
   if (strcmp(key, "csv_overlap") == 0) {
     c->opt_csv_overlap = value != 0;
-    return PLR_OK;
-  }
-  if (strcmp(key, "csv_lane_per_row") == 0) {
-    c->opt_csv_lane_rows = value < 0 ? -1 : (value != 0);
     return PLR_OK;
   }
   if (strcmp(key, "column_blocks_two_sweeps") == 0) {

@@ -6,18 +6,14 @@
 // parse, not the training pass, is what a worker waits for.  Here the worker's
 // byte range of the input is copied to HBM as it is and parsed there:
 //
-//   csv_count_rows   line starts per 4 KiB block of text
-//   csv_scan_counts  their running sum (one workgroup): first row of a block
-//   csv_row_starts   byte offset of every row
-// (these three and the parser also run on one stretch of the text at a time,
-// in text order, so that a stretch can be parsed while the next one is still
-// on its way from the host: the running row count is carried in device
-// memory from stretch to stretch, and the parser reads its row range there)
-//   csv_parse_rows   a lane per row, 64 rows per wave: every lane walks its own
-//                    row through strtod's grammar (shards of many rows)
-//   csv_parse        a wave per row: separators by ballot, one lane per field
-//                    that starts in the wave's 64-byte window, the field's
-//                    characters fetched from the neighbouring lanes (few rows)
+//   csv_count_blocks  rows and fields that start in each 4 KiB block of text
+//   csv_scan_blocks   their running sums (one workgroup): rows and fields in
+//                     front of every block
+//   csv_parse_fields  a workgroup per block, a lane per field
+// (the three also run on one stretch of the text at a time, in text order, so
+// that a stretch can be parsed while the next one is still on its way from the
+// host: the running totals are carried in device memory from stretch to
+// stretch)
 //
 // A field is converted on the device only when the result is provably strtod's,
 // the correctly rounded value of the decimal.  The spelling must be
@@ -54,131 +50,6 @@ struct CsvSlow {
   int32_t col;   // field index in the line (0 .. d-1; d-1 is the label)
   int32_t len;   // characters, or -1: longer than one window shows (the host finds its end)
 };
-
-struct CsvArgs {
-  const unsigned char* text;  // len bytes followed by kCsvPadBytes of '\n'
-  int64_t len;
-  const int64_t* row_start;   // n byte offsets
-  int64_t n;                  // rows of the shard (row_start, X, y hold that many)
-  const int64_t* row_range;   // nullptr: parse rows 0 .. n-1; else the rows
-                              //   row_range[0] .. min(row_range[1], n) - 1 (device memory)
-  int d;                      // fields per line: k features, then the label
-  unsigned char sep;
-  double* X;                  // the shard: the k features of every row (the constant
-  double* y;                  //   first column of the reference's sample is not stored)
-  int64_t pitch;
-  int np;                     // > 0: row-tiled layout with np column pairs per row
-  CsvSlow* slow;
-  int slow_cap;
-  unsigned long long* slow_count;
-  long long* bad_row;         // smallest row whose field count is not d
-  int flush_at;               // csv_parse_rows: waiting fields that trigger their conversion
-};
-
-// line starts among the 16 bytes at `base` (a line starts after a newline, or
-// at offset 0, and is not empty); their offsets go to out[] when given
-__device__ __forceinline__ int csv_starts16(const unsigned char* t, int64_t base, int64_t len,
-                                            int64_t* out) {
-  if (base >= len) return 0;
-  const uint4 v = *reinterpret_cast<const uint4*>(t + base);
-  const unsigned w[4] = {v.x, v.y, v.z, v.w};
-  unsigned char prev = base == 0 ? (unsigned char)'\n' : t[base - 1];
-  int c = 0;
-#pragma unroll
-  for (int k = 0; k < 16; ++k) {
-    const unsigned char ch = (unsigned char)(w[k >> 2] >> (8 * (k & 3)));
-    if (base + k < len && ch != '\n' && prev == '\n') {
-      if (out) out[c] = base + k;
-      ++c;
-    }
-    prev = ch;
-  }
-  return c;
-}
-
-// counts[b] for the blocks block0 .. block0 + gridDim.x - 1 of the text
-__global__ __launch_bounds__(kCsvThreads) void csv_count_rows(const unsigned char* t, int64_t len,
-                                                              int* counts, int64_t block0) {
-  __shared__ int part[kCsvThreads / 64];
-  const int64_t blk = block0 + blockIdx.x;
-  const int64_t base = (blk * kCsvThreads + threadIdx.x) * kCsvBytesPerThread;
-  int c = csv_starts16(t, base, len, nullptr);
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) c += __shfl_xor(c, m, 64);
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int s = 0;
-    for (int w = 0; w < kCsvThreads / 64; ++w) s += part[w];
-    counts[blk] = s;
-  }
-}
-
-// Running sum of counts[0..nblocks) into first_row[] (rows before each block),
-// starting from *total (the rows of the text in front of these blocks) and
-// leaving the new total there; range_out (nullable) receives the row range of
-// these blocks, [old total, new total].
-__global__ __launch_bounds__(1024) void csv_scan_counts(const int* counts, int64_t nblocks,
-                                                        int64_t* first_row, int64_t* total,
-                                                        int64_t* range_out) {
-  __shared__ int64_t wsum[16];
-  __shared__ int64_t carry_s;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (threadIdx.x == 0) {
-    carry_s = *total;
-    if (range_out) range_out[0] = carry_s;
-  }
-  __syncthreads();
-  for (int64_t i0 = 0; i0 < nblocks; i0 += 1024) {
-    const int64_t i = i0 + threadIdx.x;
-    const int64_t v = i < nblocks ? counts[i] : 0;
-    int64_t s = v;  // inclusive scan inside the wave
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) {
-      const int64_t o = __shfl_up(s, m, 64);
-      if (lane >= m) s += o;
-    }
-    if (lane == 63) wsum[wave] = s;
-    __syncthreads();
-    int64_t before = carry_s;
-    for (int w = 0; w < wave; ++w) before += wsum[w];
-    if (i < nblocks) first_row[i] = before + s - v;
-    __syncthreads();
-    if (threadIdx.x == 1023) carry_s = before + s;
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) {
-    *total = carry_s;
-    if (range_out) range_out[1] = carry_s;
-  }
-}
-
-// row_start[] for the rows that start in blocks block0 .. block0 + gridDim.x - 1;
-// rows at or past `cap` (the entries row_start holds) are not stored
-__global__ __launch_bounds__(kCsvThreads) void csv_row_starts(const unsigned char* t, int64_t len,
-                                                              const int64_t* first_row,
-                                                              int64_t* row_start, int64_t block0,
-                                                              int64_t cap) {
-  __shared__ int part[kCsvThreads / 64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t blk = block0 + blockIdx.x;
-  const int64_t base = (blk * kCsvThreads + threadIdx.x) * kCsvBytesPerThread;
-  int64_t pos[kCsvBytesPerThread];
-  const int c = csv_starts16(t, base, len, pos);
-  int s = c;
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) {
-    const int o = __shfl_up(s, m, 64);
-    if (lane >= m) s += o;
-  }
-  if (lane == 63) part[wave] = s;
-  __syncthreads();
-  int before = 0;
-  for (int w = 0; w < wave; ++w) before += part[w];
-  const int64_t at = first_row[blk] + before + s - c;
-  for (int k = 0; k < c; ++k)
-    if (at + k < cap) row_start[at + k] = pos[k];
-}
 
 // exact powers of ten
 __device__ const double kCsvPow10[23] = {1e0,  1e1,  1e2,  1e3,  1e4,  1e5,  1e6,  1e7,
@@ -223,257 +94,243 @@ __device__ __forceinline__ bool csv_scale_dd(unsigned long long m, int e, double
   return true;
 }
 
-__device__ __forceinline__ int csv_wave_max(int v) {
+// ---------------------------------------------------------------------------
+// A lane per field.  A field belongs to the block its first character lies in,
+// a row to the block its line starts in.  csv_count_blocks counts both per
+// block, csv_scan_blocks turns the counts into "rows / fields in front of this
+// block", and then every block is parsed on its own by one workgroup:
+//   * the block (and the 64 bytes behind it) go to LDS with dense 16-byte loads
+//     -- the text is read from memory once here, once by the count;
+//   * every thread classifies its 16 bytes (terminators, field starts, line
+//     starts), a prefix sum over the workgroup numbers the block's fields, and
+//     the threads write the offsets of their field starts into a list in LDS;
+//   * the fields of the list are dealt to the threads in turn: field k of the
+//     block is field F + k of the text, i.e. (all lines holding d fields)
+//     column (F + k) mod d of row (F + k) div d -- consecutive lanes convert
+//     consecutive fields and store consecutive doubles of the shard;
+//   * at every line start the number of fields in front of it must be d times
+//     the number of rows in front of it; the first row for which it is not
+//     names the ragged line (the host checks the last row against the total).
+// Neither the length of a line nor the number of lines matters to the balance:
+// 20001 fields a line or 3 parse at the same rate per byte.
+struct CsvFieldArgs {
+  const unsigned char* text;   // whole 4 KiB blocks, padded with '\n', + kCsvPadBytes
+  const int64_t* first_row;    // per block: rows of the text in front of it
+  const int64_t* first_field;  // per block: fields of the text in front of it
+  int64_t block0;              // first block of this launch
+  int64_t rows_cap;            // rows the shard holds: fields of later rows are dropped
+  int d;                       // fields per line: k features, then the label
+  unsigned char sep;
+  double inv_d;                // 1.0 / d
+  double* X;
+  double* y;
+  int64_t pitch;
+  int np;                      // > 0: row-tiled layout with np column pairs per row
+  CsvSlow* slow;
+  int slow_cap;
+  unsigned long long* slow_count;
+  long long* bad_row;
+};
+
+// Field starts and line starts among 16 bytes of text (bit k = byte k); prev is
+// the byte in front of them.  A field starts at a byte that is no terminator
+// and follows one; a line starts at a byte that is no newline and follows one.
+__device__ __forceinline__ void csv_classify16(const uint4 v, unsigned char prev, unsigned char sep,
+                                               unsigned& fmask, unsigned& lmask) {
+  const unsigned w[4] = {v.x, v.y, v.z, v.w};
+  fmask = lmask = 0u;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const unsigned char ch = (unsigned char)(w[k >> 2] >> (8 * (k & 3)));
+    const bool term = ch == sep || ch == '\n';
+    const bool pterm = prev == sep || prev == '\n';
+    if (!term && pterm) fmask |= 1u << k;
+    if (ch != '\n' && prev == '\n') lmask |= 1u << k;
+    prev = ch;
+  }
+}
+
+// rows[b], fields[b] for the blocks block0 .. block0 + gridDim.x - 1
+__global__ __launch_bounds__(kCsvThreads) void csv_count_blocks(const unsigned char* t,
+                                                                unsigned char sep, int* rows,
+                                                                int* fields, int64_t block0) {
+  __shared__ int pr[kCsvThreads / 64], pf[kCsvThreads / 64];
+  const int64_t blk = block0 + blockIdx.x;
+  const int64_t base = (blk * kCsvThreads + threadIdx.x) * kCsvBytesPerThread;
+  const uint4 v = *reinterpret_cast<const uint4*>(t + base);
+  const unsigned char prev = base == 0 ? (unsigned char)'\n' : t[base - 1];
+  unsigned fm, lm;
+  csv_classify16(v, prev, sep, fm, lm);
+  int cf = __builtin_popcount(fm), cr = __builtin_popcount(lm);
 #pragma unroll
   for (int m = 1; m < 64; m <<= 1) {
-    const int o = __shfl_xor(v, m, 64);
-    v = o > v ? o : v;
+    cf += __shfl_xor(cf, m, 64);
+    cr += __shfl_xor(cr, m, 64);
   }
-  return v;
-}
-
-__global__ __launch_bounds__(256) void csv_parse(CsvArgs a) {
-  const int lane = threadIdx.x & 63;
-  const int64_t wave0 = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int64_t nwaves = (int64_t)gridDim.x * 4;
-  const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));  // lanes before mine
-  const int64_t row_lo = a.row_range ? a.row_range[0] : 0;
-  const int64_t row_hi = a.row_range ? (a.row_range[1] < a.n ? a.row_range[1] : a.n) : a.n;
-
-  for (int64_t r = row_lo + wave0; r < row_hi; r += nwaves) {
-    int64_t pos = a.row_start[r];
-    int nfields = 0;       // fields of this row seen so far (uniform)
-    bool prev_sep = true;  // the byte in front of the window ends a field (or the row starts here)
-    bool done = false;
-    while (!done) {
-      // 128 bytes of the row: `cur` is this window, `nxt` the one behind it (the
-      // text is padded with newlines, so both loads stay inside the buffer)
-      const int cur = a.text[pos + lane];
-      const int nxt = a.text[pos + 64 + lane];
-      const unsigned long long nl_cur = __ballot(cur == '\n');
-      const unsigned long long sep_cur = __ballot(cur == a.sep);
-      const unsigned long long term_cur = nl_cur | sep_cur;
-      const unsigned long long term_nxt = __ballot(nxt == '\n' || nxt == a.sep);
-      const int endp = nl_cur ? __builtin_ctzll(nl_cur) : 64;  // the row's bytes are lanes < endp
-      done = nl_cur != 0;
-      // a field starts at a byte that is no terminator and follows one
-      const bool after_term = lane == 0 ? prev_sep : ((term_cur >> (lane - 1)) & 1ull) != 0;
-      const bool start = lane < endp && ((term_cur >> lane) & 1ull) == 0 && after_term;
-      const unsigned long long start_mask = __ballot(start);
-      int flen = 0;
-      bool bad = false;
-      if (start) {
-        const unsigned long long t1 = lane == 63 ? 0ull : term_cur >> (lane + 1);
-        if (t1)
-          flen = 1 + __builtin_ctzll(t1);
-        else if (term_nxt)
-          flen = 64 - lane + __builtin_ctzll(term_nxt);
-        else
-          flen = -1;  // no end in sight
-        if (flen < 0 || flen > kCsvMaxFieldChars) bad = true;
-      }
-      const int L = csv_wave_max((start && !bad) ? flen : 0);
-
-      // strtod's grammar for the exact spellings, one character per step
-      unsigned long long m = 0;
-      int sig = 0, ndig = 0, frac = 0, e10 = 0, ed = 0, st = 0;  // st: 0 int, 1 frac, 2 exp sign, 3 exp
-      bool neg = false, eneg = false;
-      for (int j = 0; j < L; ++j) {
-        const int src = lane + j;
-        const int c0 = __shfl(cur, src & 63, 64);
-        const int c1 = __shfl(nxt, src & 63, 64);
-        const int ch = src < 64 ? c0 : c1;
-        if (!start || bad || j >= flen) continue;
-        const bool digit = ch >= '0' && ch <= '9';
-        if (st <= 1) {
-          if (digit) {
-            m = m * 10ull + (unsigned long long)(ch - '0');
-            if (m) ++sig;
-            if (sig > 19) bad = true;  // 19 digits fit 64 bits
-            ++ndig;
-            if (st == 1) ++frac;
-          } else if (ch == '-' && j == 0) {
-            neg = true;
-          } else if (ch == '.' && st == 0) {
-            st = 1;
-          } else if ((ch == 'e' || ch == 'E') && ndig > 0) {
-            st = 2;
-          } else {
-            bad = true;
-          }
-        } else if (st == 2 && (ch == '+' || ch == '-')) {
-          eneg = ch == '-';
-          st = 3;
-        } else if (digit) {
-          st = 3;
-          e10 = e10 * 10 + (ch - '0');
-          if (e10 > 9999) bad = true;
-          ++ed;
-        } else {
-          bad = true;
-        }
-      }
-
-      if (start) {
-        const int col = nfields + __builtin_popcountll(start_mask & below);
-        int e = (eneg ? -e10 : e10) - frac;
-        if (ndig == 0 || st == 2 || (st == 3 && ed == 0) || e < -44 || e > 44) bad = true;
-        double v = 0.;
-        if (!bad) {
-          if (sig <= 15 && e >= -22 && e <= 22) {
-            v = (double)m;
-            v = e < 0 ? v / kCsvPow10[-e] : v * kCsvPow10[e];
-          } else if (m == 0) {
-            v = 0.;
-          } else if (!csv_scale_dd(m, e, v)) {
-            bad = true;
-          }
-        }
-        if (col < a.d) {
-          if (!bad) {
-            if (neg) v = -v;
-            if (col == a.d - 1) {
-              a.y[r] = v;
-            } else if (a.np > 0) {
-              a.X[((((r >> 6) * a.np + (col >> 1)) << 6) + (r & 63)) * 2 + (col & 1)] = v;
-            } else {
-              a.X[r * a.pitch + col] = v;
-            }
-          } else {
-            const unsigned long long k = atomicAdd(a.slow_count, 1ull);
-            if (k < (unsigned long long)a.slow_cap) {
-              CsvSlow s;
-              s.row = r;
-              s.pos = pos + lane;
-              s.col = col;
-              s.len = flen > kCsvMaxFieldChars ? -1 : flen;
-              a.slow[k] = s;
-            }
-          }
-        }
-      }
-      nfields += __builtin_popcountll(start_mask);
-      prev_sep = ((term_cur >> 63) & 1ull) != 0;
-      pos += 64;
+  if ((threadIdx.x & 63) == 0) {
+    pf[threadIdx.x >> 6] = cf;
+    pr[threadIdx.x >> 6] = cr;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int sf = 0, sr = 0;
+    for (int w = 0; w < kCsvThreads / 64; ++w) {
+      sf += pf[w];
+      sr += pr[w];
     }
-    if (nfields != a.d && lane == 0) atomicMin(a.bad_row, (long long)r);
+    fields[blk] = sf;
+    rows[blk] = sr;
   }
 }
 
-// The same parser with a lane per ROW: 64 consecutive rows per wave, every lane
-// walking its own row 16 bytes at a time through strtod's grammar -- all 64
-// lanes busy in the character step instead of the few that hold a field start.
-// The conversion of a finished field (a division, the stores) is deferred: the
-// field waits in a slot of its lane until most lanes have one waiting (or its
-// lane finishes the next field), so that code runs once per several steps and
-// with nearly every lane in it.
-__global__ __launch_bounds__(256) void csv_parse_rows(CsvArgs a) {
-  const int lane = threadIdx.x & 63;
-  const int64_t wave0 = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int64_t nwaves = (int64_t)gridDim.x * 4;
+// Running sums of rows[0..nblocks) and fields[0..nblocks) into first_row[] and
+// first_field[] (what lies in front of each block), starting from totals[0]
+// (rows) and totals[3] (fields) -- the text in front of these blocks -- and
+// leaving the new totals there.  One workgroup.
+__global__ __launch_bounds__(1024) void csv_scan_blocks(const int* rows, const int* fields,
+                                                        int64_t nblocks, int64_t* first_row,
+                                                        int64_t* first_field, int64_t* totals) {
+  __shared__ int64_t wr[16], wf[16];
+  __shared__ int64_t carry_r, carry_f;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) {
+    carry_r = totals[0];
+    carry_f = totals[3];
+  }
+  __syncthreads();
+  for (int64_t i0 = 0; i0 < nblocks; i0 += 1024) {
+    const int64_t i = i0 + threadIdx.x;
+    const int64_t vr = i < nblocks ? rows[i] : 0, vf = i < nblocks ? fields[i] : 0;
+    int64_t sr = vr, sf = vf;  // inclusive scans inside the wave
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+      const int64_t orr = __shfl_up(sr, m, 64), of = __shfl_up(sf, m, 64);
+      if (lane >= m) {
+        sr += orr;
+        sf += of;
+      }
+    }
+    if (lane == 63) {
+      wr[wave] = sr;
+      wf[wave] = sf;
+    }
+    __syncthreads();
+    int64_t br = carry_r, bf = carry_f;
+    for (int w = 0; w < wave; ++w) {
+      br += wr[w];
+      bf += wf[w];
+    }
+    if (i < nblocks) {
+      first_row[i] = br + sr - vr;
+      first_field[i] = bf + sf - vf;
+    }
+    __syncthreads();
+    if (threadIdx.x == 1023) {
+      carry_r = br + sr;
+      carry_f = bf + sf;
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    totals[0] = carry_r;
+    totals[3] = carry_f;
+  }
+}
 
-  const int64_t row_lo = a.row_range ? a.row_range[0] : 0;
-  const int64_t row_hi = a.row_range ? (a.row_range[1] < a.n ? a.row_range[1] : a.n) : a.n;
+__global__ __launch_bounds__(kCsvThreads) void csv_parse_fields(CsvFieldArgs a) {
+  constexpr int kAhead = 64;  // staged behind the block: a field of 32 characters and its end
+  static_assert(kAhead > kCsvMaxFieldChars + 1 && kAhead <= kCsvPadBytes, "look-ahead");
+  __shared__ __align__(16) unsigned char txt[kCsvBlockBytes + kAhead];
+  __shared__ unsigned short fpos[kCsvBlockBytes / 2 + 1];  // a field start at every other byte at most
+  __shared__ int wf[kCsvThreads / 64], wr[kCsvThreads / 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t blk = a.block0 + blockIdx.x;
+  const int64_t base = blk * kCsvBlockBytes;
 
-  for (int64_t r0 = row_lo + wave0 * 64; r0 < row_hi; r0 += nwaves * 64) {
-    const int64_t r = r0 + lane;
-    bool done = r >= row_hi;
-    const int64_t start = done ? 0 : a.row_start[r];
-    // the field in progress
+  const uint4 mine = *reinterpret_cast<const uint4*>(a.text + base + tid * kCsvBytesPerThread);
+  *reinterpret_cast<uint4*>(txt + tid * kCsvBytesPerThread) = mine;
+  if (tid < kAhead / 16)
+    *reinterpret_cast<uint4*>(txt + kCsvBlockBytes + tid * 16) =
+        *reinterpret_cast<const uint4*>(a.text + base + kCsvBlockBytes + tid * 16);
+  const unsigned char prev =
+      (base == 0 && tid == 0) ? (unsigned char)'\n' : a.text[base + tid * kCsvBytesPerThread - 1];
+  unsigned fm, lm;
+  csv_classify16(mine, prev, a.sep, fm, lm);
+
+  // fields and line starts in front of this thread's bytes, within the block
+  const int nf = __builtin_popcount(fm), nl = __builtin_popcount(lm);
+  int sf = nf, sl = nl;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) {
+    const int of = __shfl_up(sf, m, 64), ol = __shfl_up(sl, m, 64);
+    if (lane >= m) {
+      sf += of;
+      sl += ol;
+    }
+  }
+  if (lane == 63) {
+    wf[wave] = sf;
+    wr[wave] = sl;
+  }
+  __syncthreads();
+  int f0 = sf - nf, r0 = sl - nl, nfields = 0;
+#pragma unroll
+  for (int w = 0; w < kCsvThreads / 64; ++w) {
+    if (w < wave) {
+      f0 += wf[w];
+      r0 += wr[w];
+    }
+    nfields += wf[w];
+  }
+  const int64_t blk_f0 = a.first_field[blk], blk_r0 = a.first_row[blk];
+
+  // every line must hold d fields: in front of row r there are r * d of them
+  {
+    unsigned m = lm;
+    int j = 0;
+    while (m) {
+      const int k = __builtin_ctz(m);
+      m &= m - 1;
+      const int64_t r = blk_r0 + r0 + j;
+      const int64_t f = blk_f0 + f0 + __builtin_popcount(fm & ((1u << k) - 1u));
+      if (f != r * (int64_t)a.d) atomicMin(a.bad_row, (long long)(r - 1));
+      ++j;
+    }
+  }
+  // this thread's field starts into the block's list
+  {
+    unsigned m = fm;
+    int j = 0;
+    while (m) {
+      const int k = __builtin_ctz(m);
+      m &= m - 1;
+      fpos[f0 + j] = (unsigned short)(tid * kCsvBytesPerThread + k);
+      ++j;
+    }
+  }
+  __syncthreads();
+
+  const int64_t fcap = a.rows_cap * (int64_t)a.d;
+  for (int k = tid; k < nfields; k += kCsvThreads) {
+    const int64_t f = blk_f0 + k;
+    if (f >= fcap) continue;
+    const int pos = fpos[k];
+    // strtod's grammar for the exact spellings, a character per step.  The step
+    // is straight-line code (selects, no branches): the lanes of a wave are at
+    // different places of different fields, and every branch of an if-chain
+    // would be walked by the whole wave.  A lane whose field has ended idles
+    // until the longest field of the wave is through.
     unsigned long long m = 0;
-    int sig = 0, ndig = 0, frac = 0, e10 = 0, ed = 0, st = 0, flen = 0;
-    bool neg = false, eneg = false, bad = false, infield = false;
-    int col = 0;
-    // the finished field waiting for its conversion
-    bool pend = false, pneg = false, pbad = false;
-    unsigned long long pm = 0;
-    int pe = 0, psig = 0, pcol = 0, plen = 0;
-    int64_t ppos = 0;
-
-    auto flush = [&]() {
-      if (pend) {
-        double v = 0.;
-        bool fb = pbad;
-        if (!fb) {
-          if (psig <= 15 && pe >= -22 && pe <= 22) {
-            v = (double)pm;
-            v = pe < 0 ? v / kCsvPow10[-pe] : v * kCsvPow10[pe];
-          } else if (pm != 0 && !csv_scale_dd(pm, pe, v)) {
-            fb = true;
-          }
-        }
-        if (pcol < a.d) {
-          if (!fb) {
-            if (pneg) v = -v;
-            if (pcol == a.d - 1) {
-              a.y[r] = v;
-            } else if (a.np > 0) {
-              a.X[((((r >> 6) * a.np + (pcol >> 1)) << 6) + (r & 63)) * 2 + (pcol & 1)] = v;
-            } else {
-              a.X[r * a.pitch + pcol] = v;
-            }
-          } else {
-            const unsigned long long k = atomicAdd(a.slow_count, 1ull);
-            if (k < (unsigned long long)a.slow_cap) {
-              CsvSlow s;
-              s.row = r;
-              s.pos = ppos;
-              s.col = pcol;
-              s.len = plen;
-              a.slow[k] = s;
-            }
-          }
-        }
-        pend = false;
-      }
-    };
-
-    // one character of this lane's row: `ch` at byte offset `at`
-    auto step = [&](const int ch, const int64_t at) {
-      const bool live = !done && at >= start;
+    int sig = 0, ndig = 0, frac = 0, e10 = 0, ed = 0, st = 0, flen = 0;  // st: 0 int, 1 frac, 2 exp sign, 3 exp
+    bool neg = false, eneg = false, bad = false, act = true;
+    for (int j = 0; __any(act); ++j) {
+      const int ch = txt[pos + (act ? j : 0)];
       const bool term = ch == a.sep || ch == '\n';
-      const bool closes = live && term && infield;
-      // a lane about to finish a field while its slot is taken forces the conversions;
-      // otherwise they wait until most lanes have one
-      const unsigned long long waiting = __ballot(pend);
-      if (__any(closes && pend) || __builtin_popcountll(waiting) >= a.flush_at) flush();
-      // (everything below is straight-line code: selects, no branches)
-      {
-        const int e = (eneg ? -e10 : e10) - frac;
-        const bool fbad = bad || ndig == 0 || st == 2 || (st == 3 && ed == 0) || e10 > 9999 ||
-                          e < -44 || e > 44;
-        pbad = closes ? fbad : pbad;
-        pm = closes ? m : pm;
-        pe = closes ? e : pe;
-        psig = closes ? sig : psig;
-        pneg = closes ? neg : pneg;
-        pcol = closes ? col : pcol;
-        plen = closes ? flen : plen;
-        ppos = closes ? at - flen : ppos;
-        pend = pend || closes;
-        col += closes ? 1 : 0;
-        infield = infield && !closes;
-      }
-      const bool ends = live && ch == '\n';
-      if (__any(ends)) {
-        if (ends && col != a.d) atomicMin(a.bad_row, (long long)r);
-      }
-      done = done || ends;
-      // one character of the field
-      const bool act = live && !term;
-      const bool begin = act && !infield;
-      m = begin ? 0ull : m;
-      sig = begin ? 0 : sig;
-      ndig = begin ? 0 : ndig;
-      frac = begin ? 0 : frac;
-      e10 = begin ? 0 : e10;
-      ed = begin ? 0 : ed;
-      st = begin ? 0 : st;
-      flen = begin ? 0 : flen;
-      neg = neg && !begin;
-      eneg = eneg && !begin;
-      bad = bad && !begin;
-      infield = infield || act;
+      // longer than the device converts: the host finds its end
+      const bool over = act && !term && j == kCsvMaxFieldChars;
+      bad = bad || over;
+      flen = over ? -1 : flen;
+      act = act && !term && !over;
       const int dv = ch - '0';
       const bool digit = (unsigned)dv <= 9u;
       const bool mant = act && st <= 1;
@@ -482,7 +339,7 @@ __global__ __launch_bounds__(256) void csv_parse_rows(CsvArgs a) {
       sig += (mdig && m != 0ull) ? 1 : 0;
       ndig += mdig ? 1 : 0;
       frac += (mdig && st == 1) ? 1 : 0;
-      const bool minus0 = mant && ch == '-' && flen == 0;
+      const bool minus0 = mant && ch == '-' && j == 0;
       neg = neg || minus0;
       const bool dot = mant && ch == '.' && st == 0;
       const bool ee = mant && (ch | 0x20) == 'e' && ndig > 0;
@@ -495,30 +352,49 @@ __global__ __launch_bounds__(256) void csv_parse_rows(CsvArgs a) {
       bad = bad || (act && !(mdig || minus0 || dot || ee || esign || edig)) || sig > 19;
       st = dot ? 1 : ee ? 2 : (esign || edig) ? 3 : st;
       flen += act ? 1 : 0;
-    };
-
-    // A lane walks its row 16 bytes at a time; the chunk after the one being walked is
-    // already on its way.  (Holding a whole 128-byte line per lane in registers, so that
-    // no line is asked for twice, was measured: 15 % slower on 4.7 KB rows, 2.7 x slower
-    // on 150-byte rows, whose neighbours share their lines.)
-    int64_t chunk_at = start & ~(int64_t)15;
-    uint4 nx = make_uint4(0x0a0a0a0au, 0x0a0a0a0au, 0x0a0a0a0au, 0x0a0a0a0au);
-    if (!done) nx = *reinterpret_cast<const uint4*>(a.text + chunk_at);
-    while (__any(!done)) {
-      const uint4 v4 = nx;
-      if (!done) nx = *reinterpret_cast<const uint4*>(a.text + chunk_at + 16);
-      unsigned long long lo = ((unsigned long long)v4.y << 32) | v4.x;
-      unsigned long long hi = ((unsigned long long)v4.w << 32) | v4.z;
-#pragma clang loop unroll(disable)
-      for (int k = 0; k < 16; ++k) {
-        const int ch = (int)(lo & 0xffull);
-        lo = (lo >> 8) | (hi << 56);
-        hi >>= 8;
-        step(ch, chunk_at + k);
-      }
-      chunk_at += 16;
     }
-    flush();
+    if (e10 > 9999) bad = true;
+    const int e = (eneg ? -e10 : e10) - frac;
+    if (ndig == 0 || st == 2 || (st == 3 && ed == 0) || e < -44 || e > 44) bad = true;
+    double v = 0.;
+    if (!bad) {
+      if (sig <= 15 && e >= -22 && e <= 22) {
+        v = (double)m;
+        v = e < 0 ? v / kCsvPow10[-e] : v * kCsvPow10[e];
+      } else if (m != 0 && !csv_scale_dd(m, e, v)) {
+        bad = true;
+      }
+    }
+    // (row, column) of field f: f = row * d + col; the quotient by a reciprocal, corrected
+    int64_t row = (int64_t)((double)f * a.inv_d);
+    int64_t col = f - row * (int64_t)a.d;
+    if (col < 0) {
+      --row;
+      col += a.d;
+    } else if (col >= a.d) {
+      ++row;
+      col -= a.d;
+    }
+    if (!bad) {
+      if (neg) v = -v;
+      if (col == a.d - 1) {
+        a.y[row] = v;
+      } else if (a.np > 0) {
+        a.X[((((row >> 6) * a.np + (col >> 1)) << 6) + (row & 63)) * 2 + (col & 1)] = v;
+      } else {
+        a.X[row * a.pitch + col] = v;
+      }
+    } else {
+      const unsigned long long q = atomicAdd(a.slow_count, 1ull);
+      if (q < (unsigned long long)a.slow_cap) {
+        CsvSlow s;
+        s.row = row;
+        s.pos = base + pos;
+        s.col = (int)col;
+        s.len = flen;
+        a.slow[q] = s;
+      }
+    }
   }
 }
 

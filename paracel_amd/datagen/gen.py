@@ -172,9 +172,15 @@ def configs():
         # narrow rows: the row-tiled layout, a lane per row
         "x_narrow_30m_x_16": Config("x_narrow_30m_x_16", 30_000_000, 16, 0x5EED0007, NORMAL, 0.25,
                                     lam=0.01),
+        # ... at the narrowest width: one exp (and, with the loss, one log) per 16 bytes
+        "x_narrow_100m_x_2": Config("x_narrow_100m_x_2", 100_000_000, 2, 0x5EED0010, NORMAL,
+                                    1.0 / np.sqrt(2), lam=0.01),
         # ... at a width that is neither a power of two nor even
         "x_narrow_10m_x_41": Config("x_narrow_10m_x_41", 10_000_000, 41, 0x5EED000D, NORMAL,
                                     1.0 / np.sqrt(41), lam=0.01),
+        # eight waves side by side, theta in LDS, the last wave one chunk short (71 chunks = 7 x 9 + 8)
+        "x_wide_250k_x_9000": Config("x_wide_250k_x_9000", 250_000, 9000, 0x5EED0011, NORMAL,
+                                     1.0 / np.sqrt(9000), lam=0.01),
         # wider than the widest one-workgroup kernel: column blocks, a team of workgroups per row
         "x_verywide_100k_x_32768": Config("x_verywide_100k_x_32768", 100_000, 32768, 0x5EED0006,
                                           NORMAL, 1.0, lam=0.1, zero_prob=0.9, theta_nonzero=0.05),

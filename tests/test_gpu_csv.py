@@ -11,13 +11,11 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module", params=["wave per row", "lane per row"])
-def plr(request):
-    # both parsing kernels on every input (the library picks by row count otherwise)
+@pytest.fixture(scope="module")
+def plr():
     from paracel_amd import Plr
 
     with Plr(0) as c:
-        c.set_option("csv_lane_per_row", int(request.param == "lane per row"))
         yield c
 
 
@@ -67,7 +65,8 @@ def check_equal(plr, oracle, text, pieces=None, sep=","):
     n, d = plr.set_data_csv(pieces if pieces is not None else data, sep=sep)
     assert (n, d) == Xo.shape
     assert "not stored" in plr.kernel_info()
-    assert ("a lane per row" in plr.kernel_info()) or ("a wave per row" in plr.kernel_info())
+    assert any(("a %s per %s" % k) in plr.kernel_info()
+               for k in (("lane", "field"), ("lane", "row"), ("wave", "row")))
     X, y = plr.get_data()
     assert X.tobytes() == Xo.tobytes()
     assert y.tobytes() == yo.tobytes()
@@ -122,7 +121,7 @@ def test_fields_the_host_converts_and_odd_lines(plr, oracle):
 
 
 def host_converted(plr):
-    return int(plr.kernel_info().split("per row), ")[1].split(" ")[0])
+    return int(plr.kernel_info().split("), ")[-1].split(" ")[0])
 
 
 def test_long_mantissas_are_converted_on_the_device_and_still_exact(plr, oracle):
@@ -191,13 +190,13 @@ def test_pieces_of_text_and_rows_across_windows(plr, oracle):
 
 @pytest.fixture()
 def overlap(plr):
-    plr.set_option("csv_overlap", 1)
+    plr.set_option("csv_overlap", 1)     # the default, whatever a test before left
     yield plr
-    plr.set_option("csv_overlap", 0)
+    plr.set_option("csv_overlap", 1)
 
 
 def test_text_parsed_while_it_arrives(overlap, oracle):
-    # option "csv_overlap": from 256 MiB on the text is parsed stretch by stretch while the rest
+    # option "csv_overlap" (on by default): from 256 MiB on the text is parsed stretch by stretch while the rest
     # is still on its way from the host (the shard reserved for an estimated row count); same
     # shard, bit for bit, as with the whole text transferred first
     plr = overlap

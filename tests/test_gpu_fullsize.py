@@ -47,7 +47,8 @@ FULL = ["c2_headline_1m_x_1000", "c3_tall_10m_x_256", "c4_wide_200k_x_16384",
         # the shapes of the other kernel families, at the sizes bench.py times them:
         # lane_pass, lane2_pass, pair_pass, the one-chunk shard_pass, team_pass
         "x_narrow_30m_x_16", "x_narrow_10m_x_41", "x_short_30m_x_66", "x_c1shape_20m_x_100",
-        "x_verywide_100k_x_32768", "x_wide_75k_x_20000", "x_wide_30k_x_50000"]
+        "x_verywide_100k_x_32768", "x_wide_75k_x_20000", "x_wide_30k_x_50000",
+        "x_narrow_100m_x_2", "x_wide_250k_x_9000"]
 
 
 @pytest.mark.parametrize("name", FULL)
