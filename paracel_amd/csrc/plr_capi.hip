@@ -111,6 +111,11 @@ static_assert(plr_plan::kTeamMinNch == 7 && plr_plan::kTeamNch == 8 &&
                   plr_plan::kTeamWaves == plr::kTeamWaves,
               "one team kernel set per chunk count");
 constexpr int64_t kHostPredictCols = 192;  // from this pitch on predictions go straight to host
+// Results watched for by the host thread (results_arrived): shards of up to
+// 1 GiB (a pass of some 150 us at most), finishing kernels of up to 64 blocks.
+constexpr int kDoneWords = 64;
+constexpr int64_t kPollShardDoubles = 1ll << 27;
+constexpr int kPollLimitUs = 2000;
 constexpr unsigned kTeamSpinLimit = 1u << 22;  // polls before a wait for a partner gives up
 
 // Narrow rows (d <= 64): row-tiled layout, a lane per row.
@@ -285,6 +290,13 @@ struct plr_ctx {
   double* h_theta_dev = nullptr;  // the device's address of h_theta
   double* h_out = nullptr;      // pinned + device-mapped, d + 1: finish_pass writes it
   double* h_out_dev = nullptr;  // the device's address of h_out
+  // behind h_out's d + 1 doubles, on a cache line of their own: the words the
+  // finishing kernel's blocks store the pass number to (FinishArgs::done)
+  volatile unsigned long long* h_done = nullptr;
+  unsigned long long* h_done_dev = nullptr;
+  unsigned long long pass_seq = 0;
+  int done_blocks = 0;          // > 0: the pass just enqueued reports through h_done
+  bool opt_poll_results = true; // plr_set_option("poll_results")
 
   double last_ms = 0., sum_ms = 0.;
   int64_t launches = 0;
@@ -616,9 +628,13 @@ int alloc_workspace(plr_ctx* c) {
   PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_theta_dev), c->h_theta, 0));
   // results land in host memory straight from the finishing kernel (no
   // device-to-host copy in the step): pinned, mapped, coherent
-  PLR_HIP(c, hipHostMalloc(&c->h_out, (size_t)(d + 1) * sizeof(double),
+  const size_t done_at = ((size_t)(d + 1) + 7) / 8 * 8;  // in doubles: the next cache line
+  PLR_HIP(c, hipHostMalloc(&c->h_out, (done_at + kDoneWords) * sizeof(double),
                            hipHostMallocMapped | hipHostMallocCoherent));
   PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_out_dev), c->h_out, 0));
+  memset(c->h_out, 0, (done_at + kDoneWords) * sizeof(double));
+  c->h_done = reinterpret_cast<volatile unsigned long long*>(c->h_out + done_at);
+  c->h_done_dev = reinterpret_cast<unsigned long long*>(c->h_out_dev + done_at);
   memset(c->h_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double));
   PLR_HIP(c, hipMemsetAsync(c->d_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double), c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
@@ -669,6 +685,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
   const Shape* v = c->var;
   const bool grad = (kind == kPassGrad || kind == kPassDelta);
   const bool predict = (kind == kPassPredict || kind == kPassPredictLinear);
+  c->done_blocks = 0;
   // rows shared by a team of workgroups: with a gradient the one-read pass with
   // its exchange (unless switched off), without one the exchange-free team_dot
   const bool team = c->team_blocks > 0 && !c->team_off && grad;
@@ -822,6 +839,17 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     fa.nparts_loss = (team || team_dot) ? c->res_grid : grid;
     fa.delta_mode = (kind == kPassDelta) ? (train_round >= 0 ? 2 : 1) : 0;
     fa.have_grad = grad ? 1 : 0;
+    const int fblocks = grad ? (int)ceil_div(c->dcols, plr::kFinCols) : 1;
+    // a pass short enough for the stream's own completion signal to matter
+    // reports to the polling host thread as well (run_pass)
+    fa.done = nullptr;
+    fa.seq = 0;
+    if (c->opt_poll_results && out == c->h_out_dev && fblocks <= kDoneWords &&
+        c->n * c->pitch <= kPollShardDoubles) {
+      c->done_blocks = fblocks;
+      fa.done = c->h_done_dev;
+      fa.seq = ++c->pass_seq;
+    }
     fa.alpha = alpha;
     fa.coff2 = 2. * beta * alpha;
     fa.theta_rw = c->d_theta;
@@ -848,7 +876,13 @@ int stage_theta_from_host(plr_ctx* c, const double* theta) {
 int account_timing(plr_ctx* c) {
   if (!c->timing) return PLR_OK;
   float ms = 0.f;
-  PLR_HIP(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
+  hipError_t e = hipEventElapsedTime(&ms, c->ev0, c->ev1);
+  if (e == hipErrorNotReady) {  // (the results were polled for: the stream may trail them)
+    (void)hipGetLastError();
+    PLR_HIP(c, hipEventSynchronize(c->ev1));
+    e = hipEventElapsedTime(&ms, c->ev0, c->ev1);
+  }
+  PLR_HIP(c, e);
   c->last_ms = ms;
   c->sum_ms += ms;
   c->launches += 1;
@@ -913,6 +947,32 @@ int fall_back_to_two_sweeps(plr_ctx* c) {
   return PLR_OK;
 }
 
+// A short pass's results are in host memory microseconds before the runtime
+// reports the stream drained: the finishing kernel's blocks store the pass
+// number behind the results, and this thread watches those words.  False when
+// the pass does not report that way or the words have not all arrived within
+// the time limit (the caller then waits for the stream, which also brings a
+// kernel's failure to light).  The stream may still be finishing the kernel's
+// last instructions when this returns true; later work is ordered behind it.
+bool results_arrived(plr_ctx* c) {
+  const int nb = c->done_blocks;
+  if (nb <= 0) return false;
+  const unsigned long long seq = c->pass_seq;
+  const auto t0 = std::chrono::steady_clock::now();
+  for (unsigned spin = 1;; ++spin) {
+    int b = 0;
+    while (b < nb && c->h_done[b] == seq) ++b;
+    if (b == nb) {
+      std::atomic_thread_fence(std::memory_order_acquire);
+      return true;
+    }
+    if ((spin & 255u) == 0 &&
+        std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(kPollLimitUs))
+      return false;
+    __builtin_ia32_pause();
+  }
+}
+
 // One synchronous pass: theta in, kernels, results in the mapped host buffer.
 int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
              double alpha, double beta) {
@@ -941,7 +1001,7 @@ int run_pass(plr_ctx* c, PassKind kind, const double* theta, unsigned loss_mode,
   rc = enqueue_pass(c, kind, loss_mode, alpha, beta, c->h_out_dev, -1);
   if (rc != PLR_OK) return rc;
   // (measured: hipStreamSynchronize returns ~7 us sooner than a hipStreamQuery poll loop)
-  PLR_HIP(c, hipStreamSynchronize(c->stream));
+  if (!results_arrived(c)) PLR_HIP(c, hipStreamSynchronize(c->stream));
   rc = team_gave_up(c);
   if (rc < 0) return rc;
   if (rc == 1) {
@@ -2090,6 +2150,10 @@ int plr_set_option(plr_ctx* c, const char* key, int64_t value) {
     c->opt_first_col_one = value != 0;  // takes effect at the next plr_set_data / plr_alloc_data
     return PLR_OK;
   }
+  if (strcmp(key, "poll_results") == 0) {
+    c->opt_poll_results = value != 0;
+    return PLR_OK;
+  }
   if (strcmp(key, "csv_overlap") == 0) {
     c->opt_csv_overlap = value != 0;
     return PLR_OK;
@@ -2281,6 +2345,8 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
   fa.loss_slot = nullptr;
   fa.part_res = nullptr;
   fa.theta_bias = nullptr;
+  fa.done = nullptr;
+  fa.seq = 0;
   hipLaunchKernelGGL(plr::finish_pass, dim3((int)ceil_div(d, plr::kFinCols)),
                      dim3(plr::kFinCols * plr::kFinSlices), 0, stream, fa);
   PLR_NA_HIP(hipGetLastError());

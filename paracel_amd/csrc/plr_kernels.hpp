@@ -1580,6 +1580,11 @@ struct FinishArgs {
   double* loss_slot;      // nullable: also store the loss sum here
   double alpha;
   double coff2;
+  // nullable, host memory the device can write: block b stores `seq` to done[b]
+  // when everything it writes to `out` has been written (a host thread that
+  // polls these words has the results without waiting for the stream to drain)
+  unsigned long long* done;
+  unsigned long long seq;
 };
 
 constexpr int kFinCols = 16;
@@ -1656,6 +1661,11 @@ __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a
         }
       }
     }
+  }
+  if (a.done) {
+    __syncthreads();  // every store of this block to `out` has been issued ...
+    if (threadIdx.x == 0)  // ... and is visible to the host before the word is
+      __hip_atomic_store(a.done + blockIdx.x, a.seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 

@@ -673,6 +673,27 @@ def test_timing_switch(plr, gen):
     assert plr.timing()[2] == 2
 
 
+def test_results_watched_for_in_host_memory(plr, gen):
+    # option "poll_results" (default on): the caller's thread takes the results as soon as the
+    # finishing kernel has written them and their pass number to host memory.  Many calls in a
+    # row with theta changing every time -- a stale result of the call before, or one taken
+    # before all of it had arrived, would differ from the same call with the option off.
+    X, y, th = make(gen, 3000, 300)          # 19 finishing blocks, each with a word of its own
+    plr.set_data(X, y)
+    thetas = [th * (1.0 + 0.01 * k) for k in range(200)]
+    got = [plr.loss_grad(t) for t in thetas]
+    got_delta = [plr.dgd_delta(t, 1e-3, 1e-2) for t in thetas]
+    plr.set_option("poll_results", 0)
+    try:
+        for k, t in enumerate(thetas):
+            g, loss, cnt = plr.loss_grad(t)
+            assert np.array_equal(g, got[k][0]) and loss == got[k][1] and cnt == got[k][2], k
+            dl, loss = plr.dgd_delta(t, 1e-3, 1e-2)
+            assert np.array_equal(dl, got_delta[k][0]) and loss == got_delta[k][1], k
+    finally:
+        plr.set_option("poll_results", 1)
+
+
 def test_bandwidth_probes(plr, gen):
     X, y, _ = make(gen, 4096, 512)
     plr.set_data(X, y)
