@@ -335,6 +335,12 @@ def run_e2e(a, cfg, rounds=None, workers=1, theta_cpu=None):
                         q.kill()
                     raise RuntimeError("worker failed: " + e)
                 reps.append(json.loads(o.strip().splitlines()[-1]))
+                # "workerR ms per round: read theta a, wait for the GPU b, pass c, barrier d,
+                # bupdate e, barrier f"
+                for ln in o.splitlines():
+                    if " ms per round: " in ln:
+                        reps[-1]["phases_ms"] = [float(t.rsplit(" ", 1)[1])
+                                                 for t in ln.split(": ", 1)[1].split(", ")]
             theta_gpu = np.fromfile(tout)
     finally:
         srv.kill()
@@ -357,6 +363,8 @@ def run_e2e(a, cfg, rounds=None, workers=1, theta_cpu=None):
         "gpu_kernel_ms_per_iter": kern_ms,
         "final_loss": reps[0]["final_loss"],
         "theta_rel_err_vs_cpu": None,
+        # worker 0's round: read theta, wait for the GPU, pass, barrier, bupdate, barrier
+        "worker0_phases_ms": reps[0].get("phases_ms"),
     }
     if theta_cpu is None and not a.no_cpu_baseline:
         from oracle import oracle
@@ -700,7 +708,9 @@ def main():
         # and by 2 and 4 worker processes that share the GPU (n / W rows each)
         c5 = cfgs["c5_e2e_2m_x_512"]
         e2e = {"cols": ["workers", "iters_per_s", "ms_per_iter", "gpu_kernel_ms_per_iter",
-                        "theta_rel_err_vs_cpu"], "rows": [], "rounds": 100}
+                        "theta_rel_err_vs_cpu",
+                        "worker0_ms:read,wait_for_gpu,pass,barrier,bupdate,barrier"],
+               "rows": [], "rounds": 100}
         theta_cpu = None
         for W in (1, 2, 4):
             try:
@@ -708,7 +718,8 @@ def main():
                 theta_cpu = r.pop("theta_cpu", theta_cpu)
                 e2e["rows"].append([W, sig(r["value"]), sig(r["ms_per_step"]),
                                     sig(r["gpu_kernel_ms_per_iter"]),
-                                    sig(r["theta_rel_err_vs_cpu"], 3)])
+                                    sig(r["theta_rel_err_vs_cpu"], 3),
+                                    [round(v, 2) for v in r["worker0_phases_ms"] or []]])
                 if W == 1:
                     e2e["final_loss"] = r["final_loss"]
                     e2e["cpu_iters_per_s"] = sig((r.get("cpu_baseline") or {}).get("value"))

@@ -2,6 +2,7 @@
 
 #include "device_load.hpp"
 
+#include <stdio.h>
 #include <stdlib.h>
 
 #include <chrono>
@@ -116,9 +117,20 @@ void logistic_regression_gpu::dgd_learning() {
   paracel_write("theta", theta);  // first push
   paracel_register_bupdate(update_file, update_func);
   std::vector<double> delta(data_dim);
-  const auto t0 = std::chrono::steady_clock::now();
+  using clk = std::chrono::steady_clock;
+  // where a round's time goes: read theta, wait for the GPU (other workers' passes),
+  // the pass, barrier, bupdate, barrier
+  double phase[6] = {0., 0., 0., 0., 0., 0.};
+  auto lap = [](clk::time_point& t, double& into) {
+    const clk::time_point now = clk::now();
+    into += std::chrono::duration<double>(now - t).count();
+    t = now;
+  };
+  const auto t0 = clk::now();
   for (int rd = 0; rd < rounds; ++rd) {
+    clk::time_point t = clk::now();
     theta = paracel_read<std::vector<double> >("theta");
+    lap(t, phase[0]);
     // lr.cpp:125-142 in one fused pass over the resident shard.  With debug the
     // reference pushes calc_loss() after EVERY sample (lr.cpp:139-141) -- theta
     // does not change inside the round, so these are n_local copies of the
@@ -128,9 +140,11 @@ void logistic_regression_gpu::dgd_learning() {
     double loss_sum = 0.;
     {
       gpu_turn_guard mine(turn);  // several workers on the GPU: one pass at a time
+      lap(t, phase[1]);
       check(plr_dgd_delta(gpu, theta.data(), alpha, beta, delta.data(),
                           debug ? &loss_sum : nullptr),
             "plr_dgd_delta");
+      lap(t, phase[2]);
     }
     if (debug) {
       double total = loss_sum;
@@ -140,11 +154,24 @@ void logistic_regression_gpu::dgd_learning() {
       loss_error.insert(loss_error.end(), (size_t)n_local, cnt ? total / (double)cnt : 0.);
     }
     paracel_sync();
+    lap(t, phase[3]);
     paracel_bupdate("theta", delta);
+    lap(t, phase[4]);
     paracel_sync();
+    lap(t, phase[5]);
     std::cout << "worker" << get_worker_id() << " finished round: " << rd << std::endl;
   }
-  round_sec += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  round_sec += std::chrono::duration<double>(clk::now() - t0).count();
+  if (rounds > 0) {
+    char line[256];
+    const double ms = 1e3 / rounds;
+    snprintf(line, sizeof line,
+             "worker%d ms per round: read theta %.3f, wait for the GPU %.3f, pass %.3f, "
+             "barrier %.3f, bupdate %.3f, barrier %.3f",
+             (int)get_worker_id(), phase[0] * ms, phase[1] * ms, phase[2] * ms, phase[3] * ms,
+             phase[4] * ms, phase[5] * ms);
+    std::cout << line << std::endl;
+  }
   theta = paracel_read<std::vector<double> >("theta");  // last pull
 }
 

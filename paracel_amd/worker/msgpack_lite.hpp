@@ -226,6 +226,52 @@ inline void dec(Reader& r, std::vector<double>& v) {
   for (size_t i = 0; i < n; ++i) dec(r, v[i]);
 }
 
+// a list of strings (packer<list_type<str_type>>: an array of str)
+inline void enc(std::string& o, const std::vector<std::string>& v) {
+  enc_array_header(o, v.size());
+  for (const std::string& s : v) enc(o, s);
+}
+inline void dec(Reader& r, std::vector<std::string>& v) {
+  const uint8_t t = r.byte();
+  size_t n;
+  if ((t & 0xf0) == 0x90) n = t & 0x0f;
+  else if (t == 0xdc) n = r.be(2);
+  else if (t == 0xdd) n = r.be(4);
+  else throw std::runtime_error("msgpack: not an array");
+  if ((size_t)(r.end - r.p) < n) throw std::runtime_error("msgpack: array longer than its field");
+  v.resize(n);
+  for (size_t i = 0; i < n; ++i) dec(r, v[i]);
+}
+
+// a dict of key -> stored bytes (packer<dict_type<str_type, str_type>>: a map
+// of str to str), kept in the order it was packed in
+using StrMap = std::vector<std::pair<std::string, std::string> >;
+inline void enc_map_header(std::string& o, size_t n) {
+  if (n < 16) {
+    o.push_back((char)(0x80 | n));
+  } else if (n < 65536) {
+    o.push_back((char)0xde);
+    put_be(o, n, 2);
+  } else {
+    o.push_back((char)0xdf);
+    put_be(o, n, 4);
+  }
+}
+inline void dec(Reader& r, StrMap& m) {
+  const uint8_t t = r.byte();
+  size_t n;
+  if ((t & 0xf0) == 0x80) n = t & 0x0f;
+  else if (t == 0xde) n = r.be(2);
+  else if (t == 0xdf) n = r.be(4);
+  else throw std::runtime_error("msgpack: not a map");
+  if ((size_t)(r.end - r.p) < 2 * n) throw std::runtime_error("msgpack: map longer than its field");
+  m.resize(n);
+  for (size_t i = 0; i < n; ++i) {
+    dec(r, m[i].first);
+    dec(r, m[i].second);
+  }
+}
+
 }  // namespace detail
 
 // bare msgpack bytes of one value

@@ -10,8 +10,9 @@
 // utils/comm.hpp:629-636).  Here the workers are plain processes (one shard
 // each, sharing the GPU of the box), so the same two collectives run over what
 // every worker already has a connection to -- server 0's key-value table, with
-// push and pull only (the two ops whose behaviour on a missing key is the
-// same on the reference's server: push creates it, pull answers "nokey"):
+// push and pull_multi_check only (two ops whose behaviour on a missing key is
+// the same on the reference's server: push creates it, pull_multi_check leaves
+// it out of its answer; server.hpp:254-260, kv.hpp:94-103):
 //   barrier    worker r pushes the number k of the barrier it has reached
 //              under "plr_sync_<r>" (k = 1, 2, ...: all workers call their
 //              barriers in the same order, as MPI requires too) and waits
@@ -19,7 +20,7 @@
 //              grow, so nothing has to be removed and the table holds
 //              worker_sz such keys however long the job runs.
 //   allreduce  worker r pushes its value under "plr_ar_<k mod 2>_<r>", barrier,
-//              then pulls all worker_sz values and adds them in rank order --
+//              then pulls all worker_sz values (one request) and adds them in rank order --
 //              the same bits on every worker.  Two slots suffice: slot k mod 2
 //              is written again in call k + 2, behind the barrier of call
 //              k + 1, which nobody passes before every worker has read call k.
@@ -72,6 +73,13 @@ class kvclt {
     bool stat = false;
     const bool r = req(1, paste({pack<std::string>("push"), pack(key), pack(val)}), stat);
     return r && stat;
+  }
+  // client.hpp:93-101: the keys of the list that the table holds, with their
+  // stored (packed) values -- one round trip for any number of keys
+  detail::StrMap pull_multi_check(const std::vector<std::string>& keys) {
+    detail::StrMap got;
+    req(0, paste({pack<std::string>("pull_multi_check"), pack(keys)}), got);
+    return got;
   }
   bool register_bupdate(const std::string& file, const std::string& func) {
     bool stat = false;
@@ -263,27 +271,32 @@ class paralg {
     if (nworker_ <= 1) return;
     const int k = ++sync_count_;
     if (!kvm_[0]->push(sync_key(rank_), k)) throw std::runtime_error("paracel_sync: push failed");
-    const auto deadline =
-        std::chrono::steady_clock::now() + std::chrono::duration<double>(sync_timeout_s_);
-    int next = 0;  // workers [0, next) have been seen at barrier k
-    for (unsigned spins = 0; next < nworker_;) {
-      int at = 0;
-      if (next == rank_ || (kvm_[0]->pull(sync_key(next), at) && at >= k)) {
-        ++next;
-        continue;
-      }
-      if (std::chrono::steady_clock::now() > deadline) {
+    std::vector<std::string> others;
+    for (int r = 0; r < nworker_; ++r)
+      if (r != rank_) others.push_back(sync_key(r));
+    const auto start = std::chrono::steady_clock::now();
+    const auto deadline = start + std::chrono::duration<double>(sync_timeout_s_);
+    for (;;) {
+      // every other worker's counter in one round trip; a key not pushed yet is left out
+      const detail::StrMap got = kvm_[0]->pull_multi_check(others);
+      size_t arrived = 0;
+      for (const auto& kv : got) arrived += unpack<int>(kv.second) >= k ? 1 : 0;
+      if (arrived == others.size()) return;
+      const auto now = std::chrono::steady_clock::now();
+      if (now > deadline) {
         std::string missing;
-        for (int r = next; r < nworker_; ++r) {
-          at = 0;
-          if (r != rank_ && !(kvm_[0]->pull(sync_key(r), at) && at >= k))
-            missing += (missing.empty() ? "" : ", ") + std::to_string(r);
+        for (int r = 0; r < nworker_; ++r) {
+          if (r == rank_) continue;
+          bool here = false;
+          for (const auto& kv : got) here = here || (kv.first == sync_key(r) && unpack<int>(kv.second) >= k);
+          if (!here) missing += (missing.empty() ? "" : ", ") + std::to_string(r);
         }
         throw std::runtime_error("paracel_sync: barrier " + std::to_string(k) + ": worker(s) " +
                                  missing + " did not arrive within " +
                                  std::to_string(sync_timeout_s_) + " s");
       }
-      usleep(spins++ < 64 ? 20 : 200);
+      // the first 2 ms poll after poll (a round trip is tens of microseconds), then at ease
+      if (now - start > std::chrono::milliseconds(2)) usleep(100);
     }
   }
   void set_sync_timeout(double seconds) { sync_timeout_s_ = seconds; }
@@ -296,13 +309,15 @@ class paralg {
     if (!kvm_[0]->push(base + std::to_string(rank_), v))
       throw std::runtime_error("allreduce: push failed");
     paracel_sync();
+    // all values in one round trip, added in rank order whatever order they come in
+    std::vector<std::string> keys;
+    for (int r = 0; r < nworker_; ++r) keys.push_back(base + std::to_string(r));
+    const detail::StrMap got = kvm_[0]->pull_multi_check(keys);
+    if (got.size() != keys.size()) throw std::runtime_error("allreduce: a worker's value is missing");
     double sum = 0.;
-    for (int r = 0; r < nworker_; ++r) {
-      double part = 0.;
-      if (!kvm_[0]->pull(base + std::to_string(r), part))
-        throw std::runtime_error("allreduce: a worker's value is missing");
-      sum += part;
-    }
+    for (int r = 0; r < nworker_; ++r)
+      for (const auto& kv : got)
+        if (kv.first == keys[r]) sum += unpack<double>(kv.second);
     v = sum;
   }
   void allreduce(int& v) {

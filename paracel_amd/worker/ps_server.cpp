@@ -138,23 +138,31 @@ static void op_thread(void* sock) {
           }
           reply(sock, it->second);  // the new value
         }
-      } else if (op == "pullall") {
-        // server.hpp:261-264: the whole table as one packed map of key -> stored bytes
+      } else if (op == "pullall" || op == "pull_multi_check") {
+        // server.hpp:261-264: the whole table as one packed map of key -> stored bytes;
+        // server.hpp:254-260 with kv.hpp:94-103: the same for the keys of a list that
+        // are in the table (a missing key is left out, not an error)
         std::lock_guard<std::mutex> g(store_mutex);
         std::string body;
-        const size_t n = tbl_store.size();
-        if (n < 16) {
-          body.push_back((char)(0x80 | n));
-        } else if (n < 65536) {
-          body.push_back((char)0xde);
-          detail::put_be(body, n, 2);
+        if (op == "pullall") {
+          detail::enc_map_header(body, tbl_store.size());
+          for (const auto& kv : tbl_store) {
+            detail::enc(body, kv.first);
+            detail::enc(body, kv.second);
+          }
         } else {
-          body.push_back((char)0xdf);
-          detail::put_be(body, n, 4);
-        }
-        for (const auto& kv : tbl_store) {
-          detail::enc(body, kv.first);
-          detail::enc(body, kv.second);
+          const auto keys = unpack<std::vector<std::string> >(msg.at(1).str());
+          std::string entries;
+          size_t found = 0;
+          for (const std::string& k : keys) {
+            const auto it = tbl_store.find(k);
+            if (it == tbl_store.end()) continue;
+            detail::enc(entries, it->first);
+            detail::enc(entries, it->second);
+            ++found;
+          }
+          detail::enc_map_header(body, found);
+          body.append(entries);
         }
         const size_t len = body.size();
         std::string out((const char*)&len, sizeof len);

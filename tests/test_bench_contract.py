@@ -112,5 +112,7 @@ def test_the_default_run_fits_what_the_harness_keeps():
     assert [r[0] for r in ps["rows"]] == [1, 2, 4]
     for r_ in ps["rows"]:
         assert r_[1] > 0 and r_[4] <= 1e-8, r_
+        # worker 0's round in its six phases: they add up to the round
+        assert len(r_[5]) == 6 and abs(sum(r_[5]) - r_[2]) < 0.1 * r_[2], r_
     assert out["c1_latency_us"]["train_dgd_per_round"] > 0
     assert out["c5_text_to_shard"]["text_gb_per_s"] > 0

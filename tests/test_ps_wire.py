@@ -312,3 +312,18 @@ def test_incr_int_does_not_create_a_key(server):
     z.req(host, ports[4], SEP.join([field("push_int"), field("clock"), field(5)]))
     z.req(host, ports[4], SEP.join([field("incr_int"), field("clock"), field(2)]))
     assert unfield(z.req(host, ports[4], SEP.join([field("pull_int"), field("clock")]))) == 7
+
+
+def test_pull_multi_check_leaves_missing_keys_out(server):
+    # server.hpp:254-260 with kv.hpp:94-103: the keys of the list that the table holds, as a
+    # packed map of key -> stored bytes; a missing key is left out (the workers' barrier asks
+    # for every other worker's counter this way, before some of them have pushed theirs)
+    z, host, ports, _ = server
+    z.req(host, ports[1], SEP.join([field("push"), field("pm_a"), field(7)]))
+    z.req(host, ports[1], SEP.join([field("push"), field("pm_b"), field([1.5, 2.5])]))
+    got = unfield_raw(z.req(host, ports[0], SEP.join(
+        [field("pull_multi_check"), field(["pm_a", "pm_ghost", "pm_b"])])))
+    assert sorted(got) == [b"pm_a", b"pm_b"]
+    assert unfield(got[b"pm_a"]) == 7 and unfield(got[b"pm_b"]) == [1.5, 2.5]
+    none = unfield_raw(z.req(host, ports[0], SEP.join([field("pull_multi_check"), field(["pm_x"])])))
+    assert none == {}
