@@ -2,6 +2,7 @@
 #pragma once
 
 #include <fcntl.h>
+#include <stdlib.h>
 #include <sys/file.h>
 #include <unistd.h>
 
@@ -47,6 +48,25 @@ class gpu_turn {
  private:
   int fd_ = -1;
 };
+
+// To be called before the process's first GPU call when worker_sz > 1 workers
+// share the GPU.  The runtime spreads a process's streams (the pass's and the
+// eight upload lanes') over up to 4 hardware queues; the device serves 16 such
+// queues side by side, and with more in existence -- measured: four workers
+// and one idle process that had used the GPU before, 20 queues -- it
+// multiplexes them, and every pass, although it runs alone, takes 2.7 times as
+// long (0.79 ms instead of 0.29 on 500 000 x 512 rows; 220 rounds a second
+// instead of 600).  Two queues per worker (one from 8 workers on) keep the
+// total below that; the upload loses nothing measurable.  A smaller value
+// already in the environment is left alone, a larger one (4 is the runtime's
+// default) is lowered.
+inline void limit_hw_queues_of_gpu_sharers(int worker_sz) {
+  if (worker_sz <= 1) return;
+  const int want = worker_sz > 7 ? 1 : 2;
+  const char* cur = getenv("GPU_MAX_HW_QUEUES");
+  if (cur && atoi(cur) >= 1 && atoi(cur) <= want) return;
+  setenv("GPU_MAX_HW_QUEUES", want == 1 ? "1" : "2", /*overwrite=*/1);
+}
 
 struct gpu_turn_guard {
   explicit gpu_turn_guard(gpu_turn& t) : t_(t) { t_.lock(); }

@@ -65,6 +65,7 @@ int main(int argc, char** argv) {
       return 1;
     }
   }
+  plr_ps::limit_hw_queues_of_gpu_sharers(worker_sz);  // before the first GPU call
   try {
     if (!synthetic.empty()) {
       unsigned long long seed;

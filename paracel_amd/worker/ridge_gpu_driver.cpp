@@ -40,6 +40,7 @@ int main(int argc, char** argv) {
       return 1;
     }
   }
+  plr_ps::limit_hw_queues_of_gpu_sharers(worker_sz);  // before the first GPU call
   try {
     auto kv = plr_ps::parse_flat_json(cfg_file);
     plr_ps::ridge_regression_gpu solver(
