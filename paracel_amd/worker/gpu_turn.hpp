@@ -15,8 +15,7 @@ namespace plr_ps {
 // processes that run side by side do not add up: each is a persistent grid
 // sized to the whole device, and the device shares itself out between
 // processes in coarse slices (measured on 2 M x 512 rows: two workers' halves
-// 0.89 ms each instead of 0.58, four workers' quarters 1.43 ms each instead of
-// 0.29, 4.6 ms per round instead of 1.35).  An advisory lock on a per-device
+// 0.89 ms each instead of 0.58).  An advisory lock on a per-device
 // file (flock: released by the kernel when its holder dies) makes a pass
 // exclusive among the workers of this box; it also gives the one-read pass over
 // rows wider than 19456 columns the residency it needs (should another
