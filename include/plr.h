@@ -233,11 +233,11 @@ int plr_set_timing(plr_ctx* ctx, int enabled);
  *   "team_lag"  how many rows the rank-1 update of that pass trails the dot
  *        product: 1, 2, or 0 (default) = chosen by the width.  Same results;
  *        applies from the next plr_set_data / plr_alloc_data.
- *   "poll_results"  value != 0 (default): after a pass over a shard of up to
- *        1 GiB the calling thread watches host memory for the results, which
- *        the last kernel writes there with a pass number behind them, instead
- *        of waiting for the runtime to report the stream drained (3-4 us
- *        sooner on a pass of 20 us).  0: always wait for the stream.  Same
+ *   "poll_results"  value != 0 (default): after a pass over rows of up to 1024
+ *        stored columns the calling thread watches host memory for the
+ *        results, which the last kernel writes there with a pass number behind
+ *        them, instead of waiting for the runtime to report the stream
+ *        drained (3-4 us sooner).  0: always wait for the stream.  Same
  *        results.
  *   "csv_overlap"  value != 0 (default): plr_set_data_csv parses texts of
  *        256 MiB and more stretch by stretch while the rest is still arriving

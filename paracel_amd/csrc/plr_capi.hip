@@ -111,11 +111,11 @@ static_assert(plr_plan::kTeamMinNch == 7 && plr_plan::kTeamNch == 8 &&
                   plr_plan::kTeamWaves == plr::kTeamWaves,
               "one team kernel set per chunk count");
 constexpr int64_t kHostPredictCols = 192;  // from this pitch on predictions go straight to host
-// Results watched for by the host thread (results_arrived): shards of up to
-// 1 GiB (a pass of some 150 us at most), finishing kernels of up to 64 blocks.
+// Results watched for by the host thread (results_arrived): finishing kernels of
+// up to 64 blocks (1024 columns), for at most 20 ms -- longer than any pass over
+// a shard that fits the device -- before the thread waits for the stream instead.
 constexpr int kDoneWords = 64;
-constexpr int64_t kPollShardDoubles = 1ll << 27;
-constexpr int kPollLimitUs = 2000;
+constexpr int kPollLimitUs = 20000;
 constexpr unsigned kTeamSpinLimit = 1u << 22;  // polls before a wait for a partner gives up
 
 // Narrow rows (d <= 64): row-tiled layout, a lane per row.
@@ -844,8 +844,7 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     // reports to the polling host thread as well (run_pass)
     fa.done = nullptr;
     fa.seq = 0;
-    if (c->opt_poll_results && out == c->h_out_dev && fblocks <= kDoneWords &&
-        c->n * c->pitch <= kPollShardDoubles) {
+    if (c->opt_poll_results && out == c->h_out_dev && fblocks <= kDoneWords) {
       c->done_blocks = fblocks;
       fa.done = c->h_done_dev;
       fa.seq = ++c->pass_seq;
