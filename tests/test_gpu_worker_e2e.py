@@ -136,7 +136,7 @@ def test_csv_driver_follows_the_reference_call_order(server_info, oracle, tmp_pa
 
 
 def test_config_5_at_full_size_through_the_server(server_info, oracle, gen, tmp_path):
-    # BASELINE config 5 as it is defined: 2 000 000 x 512, 100 rounds of paracel_read ->
+    # benchmark configuration 5 as it is defined: 2 000 000 x 512, 100 rounds of paracel_read ->
     # GPU delta -> paracel_bupdate; theta against the CPU oracle's 16-worker training
     cfg = gen.configs()["c5_e2e_2m_x_512"]
     n, d, rounds = cfg.n, cfg.d, 100
