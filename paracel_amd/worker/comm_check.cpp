@@ -5,10 +5,14 @@
 // an int; between two barriers each worker bumps a shared counter and checks
 // after the second one that all W bumps are there (what a barrier is for).
 // Prints "ok <rank>" and exits 0, or a message and exits 1.
+//   plr_comm_check --hw_queues W
+// prints what GPU_MAX_HW_QUEUES reads after limit_hw_queues_of_gpu_sharers(W)
+// (or "unset"), for the value found in the environment.
 #include <stdlib.h>
 
 #include <iostream>
 
+#include "gpu_turn.hpp"
 #include "paralg_lite.hpp"
 
 int main(int argc, char** argv) {
@@ -20,6 +24,12 @@ int main(int argc, char** argv) {
     else if (a == "--worker_id") rank = atoi(v.c_str());
     else if (a == "--worker_sz") W = atoi(v.c_str());
     else if (a == "--rounds") rounds = atoi(v.c_str());
+    else if (a == "--hw_queues") {
+      plr_ps::limit_hw_queues_of_gpu_sharers(atoi(v.c_str()));
+      const char* q = getenv("GPU_MAX_HW_QUEUES");
+      std::cout << (q ? q : "unset") << std::endl;
+      return 0;
+    }
   }
   try {
     plr_ps::paralg pa(info, "", 1, rank, W);

@@ -327,3 +327,29 @@ def test_pull_multi_check_leaves_missing_keys_out(server):
     assert unfield(got[b"pm_a"]) == 7 and unfield(got[b"pm_b"]) == [1.5, 2.5]
     none = unfield_raw(z.req(host, ports[0], SEP.join([field("pull_multi_check"), field(["pm_x"])])))
     assert none == {}
+
+
+def test_workers_that_share_a_gpu_limit_their_hardware_queues():
+    # more than 16 hardware queues on a device slow every kernel down: W > 1 workers take two
+    # each (one from 8 workers on); a smaller value in the environment stays, a larger one --
+    # 4 is the runtime's default -- is lowered; a single worker changes nothing
+    _need_host_binaries()
+    tool = os.path.join(PKG, "plr_comm_check")
+    if not os.path.exists(tool):
+        subprocess.run(["make", "-C", os.path.join(PKG, "worker"), os.path.join("..", "plr_comm_check")],
+                       check=True)
+
+    def after(W, start):
+        env = dict(os.environ)
+        env.pop("GPU_MAX_HW_QUEUES", None)
+        if start is not None:
+            env["GPU_MAX_HW_QUEUES"] = start
+        r = subprocess.run([tool, "--hw_queues", str(W)], env=env, capture_output=True, text=True,
+                           timeout=30)
+        assert r.returncode == 0, r.stderr
+        return r.stdout.strip()
+
+    assert after(1, None) == "unset" and after(1, "4") == "4"
+    assert after(2, None) == "2" and after(4, "4") == "2" and after(7, "16") == "2"
+    assert after(8, "4") == "1" and after(16, None) == "1"
+    assert after(4, "1") == "1" and after(2, "2") == "2"
