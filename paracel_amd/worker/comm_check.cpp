@@ -50,6 +50,7 @@ int main(int argc, char** argv) {
       }
       // nobody passes the second barrier before everybody has written
       pa.paracel_write("bump_" + std::to_string(k) + "_" + std::to_string(rank), (double)rank);
+      if (k & 1) pa.paracel_sync_arrive();  // every other round: the barrier in two halves
       pa.paracel_sync();
       for (int r = 0; r < W; ++r) {
         const double got =

@@ -130,6 +130,9 @@ void logistic_regression_gpu::dgd_learning() {
   for (int rd = 0; rd < rounds; ++rd) {
     clk::time_point t = clk::now();
     theta = paracel_read<std::vector<double> >("theta");
+    // theta is read: as far as the barrier in front of the bupdate is concerned
+    // (nobody updates theta before everybody has read it) this worker has arrived
+    if (!debug) paracel_sync_arrive();
     lap(t, phase[0]);
     // lr.cpp:125-142 in one fused pass over the resident shard.  With debug the
     // reference pushes calc_loss() after EVERY sample (lr.cpp:139-141) -- theta

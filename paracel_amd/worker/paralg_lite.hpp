@@ -18,7 +18,8 @@
 //              barriers in the same order, as MPI requires too) and waits
 //              until every worker's key reads k or more.  The counters only
 //              grow, so nothing has to be removed and the table holds
-//              worker_sz such keys however long the job runs.
+//              worker_sz such keys however long the job runs.  The push may
+//              go out ahead of time (paracel_sync_arrive).
 //   allreduce  worker r pushes its value under "plr_ar_<k mod 2>_<r>", barrier,
 //              then pulls all worker_sz values (one request) and adds them in rank order --
 //              the same bits on every worker.  Two slots suffice: slot k mod 2
@@ -70,9 +71,28 @@ class kvclt {
   }
   template <class V>
   bool push(const std::string& key, const V& val) {
+    if (push_in_flight_ && !push_end()) return false;
     bool stat = false;
     const bool r = req(1, paste({pack<std::string>("push"), pack(key), pack(val)}), stat);
     return r && stat;
+  }
+  // A push in two halves: the request goes out now, the reply is collected by
+  // push_end() (or by the next push) -- the caller does something else while
+  // the server stores the value.
+  template <class V>
+  void push_begin(const std::string& key, const V& val) {
+    if (push_in_flight_) (void)push_end();
+    send_only(1, paste({pack<std::string>("push"), pack(key), pack(val)}));
+    push_in_flight_ = true;
+  }
+  bool push_end() {
+    if (!push_in_flight_) return true;
+    push_in_flight_ = false;
+    zmq_msg_t m;
+    recv_only(1, &m);
+    const std::string data((const char*)zmq_msg_data(&m), zmq_msg_size(&m));
+    zmq_msg_close(&m);
+    return unpack<bool>(data);
   }
   // client.hpp:93-101: the keys of the list that the table holds, with their
   // stored (packed) values -- one round trip for any number of keys
@@ -156,6 +176,10 @@ class kvclt {
   // caller closes *m.  An empty reply is the reference's internal error
   // (client.hpp:551).
   void roundtrip(int port_idx, const std::string& scrip, zmq_msg_t* m) {
+    send_only(port_idx, scrip);
+    recv_only(port_idx, m);
+  }
+  void send_only(int port_idx, const std::string& scrip) {
     void*& s = socks_[port_idx];
     if (!s) {
       s = zmq_socket(zctx_, ZMQ_REQ);
@@ -165,6 +189,9 @@ class kvclt {
     }
     if (zmq_send(s, scrip.data(), scrip.size(), 0) < 0)
       throw std::runtime_error(std::string("zmq_send: ") + zmq_strerror(zmq_errno()));
+  }
+  void recv_only(int port_idx, zmq_msg_t* m) {
+    void* s = socks_[port_idx];
     zmq_msg_init(m);
     if (zmq_msg_recv(m, s, 0) < 0) {
       zmq_msg_close(m);
@@ -191,6 +218,7 @@ class kvclt {
   void* zctx_;
   void* socks_[5];
   std::string buf_;  // request buffer of the dense forms, reused across rounds
+  bool push_in_flight_ = false;
 };
 
 class paralg {
@@ -270,7 +298,12 @@ class paralg {
   void paracel_sync() {
     if (nworker_ <= 1) return;
     const int k = ++sync_count_;
-    if (!kvm_[0]->push(sync_key(rank_), k)) throw std::runtime_error("paracel_sync: push failed");
+    if (announced_) {
+      announced_ = false;
+      if (!kvm_[0]->push_end()) throw std::runtime_error("paracel_sync: push failed");
+    } else if (!kvm_[0]->push(sync_key(rank_), k)) {
+      throw std::runtime_error("paracel_sync: push failed");
+    }
     std::vector<std::string> others;
     for (int r = 0; r < nworker_; ++r)
       if (r != rank_) others.push_back(sync_key(r));
@@ -299,12 +332,27 @@ class paralg {
       if (now - start > std::chrono::milliseconds(2)) usleep(100);
     }
   }
+  // The arrival half of the next paracel_sync(), ahead of time (no counterpart
+  // in the reference, whose barrier is MPI's): "whatever the next barrier
+  // protects, this worker has done it" -- its counter goes to the server now,
+  // without waiting for the reply, and the paracel_sync() that follows only
+  // waits for the others.  For a barrier whose purpose is met early: the one
+  // between a round's pass and its bupdate (lr.cpp:143) is there so that nobody
+  // updates theta before everybody has read it, which is true of a worker as
+  // soon as its read has returned.  The next collective after this call must
+  // be that paracel_sync() (an allreduce in between throws).
+  void paracel_sync_arrive() {
+    if (nworker_ <= 1 || announced_) return;
+    kvm_[0]->push_begin(sync_key(rank_), sync_count_ + 1);
+    announced_ = true;
+  }
   void set_sync_timeout(double seconds) { sync_timeout_s_ = seconds; }
   size_t get_worker_id() const { return rank_; }
   size_t get_worker_size() const { return nworker_; }
   // comm.hpp:629-636 (MPI_Allreduce, MPI_SUM): v becomes the sum over all workers
   void allreduce(double& v) {
     if (nworker_ <= 1) return;
+    if (announced_) throw std::logic_error("allreduce between paracel_sync_arrive and paracel_sync");
     const std::string base = "plr_ar_" + std::to_string(reduce_count_++ & 1) + "_";
     if (!kvm_[0]->push(base + std::to_string(rank_), v))
       throw std::runtime_error("allreduce: push failed");
@@ -367,6 +415,7 @@ class paralg {
   }
   int rank_, nworker_;
   int sync_count_ = 0;
+  bool announced_ = false;  // paracel_sync_arrive() has sent the next barrier's counter
   long reduce_count_ = 0;
   double sync_timeout_s_ = default_sync_timeout();
   void* zctx_ = nullptr;

@@ -77,6 +77,7 @@ void ridge_regression_gpu::batch_learning() {
   std::vector<double> delta(data_dim);
   for (int rd = 0; rd < rounds; ++rd) {
     theta = paracel_read<std::vector<double> >("theta");
+    paracel_sync_arrive();  // theta is read (see lr_gpu.cpp)
     {
       gpu_turn_guard mine(turn);  // several workers on the GPU: one pass at a time
       check(plr_dgd_delta_linear(gpu, theta.data(), alpha, beta, delta.data(), nullptr),
