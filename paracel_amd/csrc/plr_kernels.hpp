@@ -710,8 +710,11 @@ __global__ __launch_bounds__(kWave* WROW, MINW) void lane_pass(PassArgs a) {
           acc[p].y = fma(res, x[u][p].y, acc[p].y);
         }
       } else {
-        // predictions go with the passes that carry no gradient
-        if (a.h_out && valid) store_h(a.h_out + row0 + u * kWave, h);
+        // predictions go with the passes that carry no gradient.  A plain store: the
+        // destination is device memory here, and letting the L2 write the lines
+        // back in its own time is 3.5 % faster than the non-temporal form
+        // (30 M x 16: 0.720 against 0.746 ms)
+        if (a.h_out && valid) a.h_out[row0 + u * kWave] = h;
       }
     }
   };
