@@ -426,7 +426,11 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
     const int64_t ngroups = ceil_div(n, (int64_t)plr::kWave * lv->U);
     const int64_t want = std::max<int64_t>(1, ceil_div(ngroups, lv->wrow));
     c->grid = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ);
-    c->grid_nograd = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ2);
+    // (the instances without a gradient need fewer registers and would fit more
+    // workgroups per compute unit; measured, they stream fastest on the grid of
+    // the instance with one: more resident waves than the tile shape was tuned
+    // for cost 1-6 %)
+    c->grid_nograd = (int)std::min<int64_t>(want, (int64_t)c->num_cu * std::min(occ, occ2));
     char b[256];
     snprintf(b, sizeof b,
              "%s<NP=%d,U=%d,WROW=%d> row-tiled layout, pitch=%lld, %d rows per group, "
@@ -452,7 +456,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
     const int64_t ntiles = ceil_div(n, (int64_t)2 * pv->G);
     const int64_t want = std::max<int64_t>(1, ceil_div(ntiles, pv->wrow));
     c->grid = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ);
-    c->grid_nograd = (int)std::min<int64_t>(want, (int64_t)c->num_cu * occ2);
+    c->grid_nograd = (int)std::min<int64_t>(want, (int64_t)c->num_cu * std::min(occ, occ2));
     char b[256];
     snprintf(b, sizeof b,
              "pair_pass<G=%d,WROW=%d> pitch=%lld, %d rows per tile, grid=%d x %d threads "
@@ -529,7 +533,7 @@ int plan_shape(plr_ctx* c, int64_t n, int64_t d) {
                  &occ_ng, reinterpret_cast<const void*>(f->fn[0][c->allch]), threads, 0));
   if (occ < 1 || occ_ng < 1)
     return fail(c, PLR_ERR_HIP, "kernel variant does not fit on a compute unit");
-  int64_t g = (int64_t)c->num_cu * occ, g2 = (int64_t)c->num_cu * occ_ng;
+  int64_t g = (int64_t)c->num_cu * occ, g2 = (int64_t)c->num_cu * std::min(occ, occ_ng);
   if (g > want) g = want;
   if (g2 > want) g2 = want;
   if (g < 1) g = 1;
