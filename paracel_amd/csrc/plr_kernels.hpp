@@ -1371,8 +1371,7 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_pass(TeamArgs a) {
 // waves, but every wave just streams its chunks of its team's rows and stores
 // its partial dot products -- kept in the lanes for 64 rows, then written as one
 // dense 512-byte store to z_out[((blk * 8 + wave) * nteams + team) * zstride + i],
-// i counting the team's rows.  No exchange, no barrier, no residency
-// requirement.  residual_pass adds a row's partials --
+// i counting the team's rows.  No exchange and no residency requirement.  residual_pass adds a row's partials --
 // first over the waves of a block, then over the blocks, the order team_pass
 // adds them in, so both give the same bits -- and turns z into loss terms and
 // predictions.  Three row buffers rotate: rows t + 1 and t + 2 are in flight
@@ -1423,6 +1422,11 @@ __global__ __launch_bounds__(kWave* kTeamWaves, 2) void team_dot(TeamArgs a) {
   };
   auto step = [&](int64_t t, auto phase_tag) {
     constexpr int PH = decltype(phase_tag)::value;  // t mod 3
+    // Nothing is exchanged here: the barrier only keeps the block's eight waves
+    // at the same row, so that together they ask for one contiguous piece of it
+    // (measured: 6.64 -> 6.73 TB/s at 20000 to 131072 columns).  Every wave of
+    // the block takes the same number of steps.
+    __builtin_amdgcn_s_barrier();
     request(t + 2, X[(PH + 2) % D]);
     asm volatile("" ::: "memory");
     // the ragged chunk's lanes past the row end hold the next row's bytes: their
