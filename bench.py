@@ -48,94 +48,94 @@ MEASURED_TRAFFIC = {
         100000,
         "shard_pass<NCH=1,R=16,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=1 tail=0 pitch=100 "
         "grid=512 x 256 threads (occupancy 2 blocks/CU, 256 CUs)",
-        82200159, "profiles/shard_pass_c1_dense_100k_x_100.md"),
+        82217759, "profiles/shard_pass_c1_dense_100k_x_100.md"),
     "c2_headline_1m_x_1000": (
         1000000,
         "shard_pass<NCH=8,R=4,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=8 tail=0 pitch=1000 "
         "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)",
-        8054328548, "profiles/shard_pass_c2_headline_1m_x_1000.md"),
+        8055154154, "profiles/shard_pass_c2_headline_1m_x_1000.md"),
     "c3_tall_10m_x_256": (
         10000000,
         "shard_pass<NCH=2,R=32,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=2 tail=0 pitch=256 "
         "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)",
-        20560483632, "profiles/shard_pass_c3_tall_10m_x_256.md"),
+        20560483722, "profiles/shard_pass_c3_tall_10m_x_256.md"),
     "c4_wide_200k_x_16384": (
         200000,
         "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=0> nch_rt=16 tail=0 pitch=16384 "
         "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        26261496561, "profiles/shard_pass_c4_wide_200k_x_16384.md"),
+        26261494892, "profiles/shard_pass_c4_wide_200k_x_16384.md"),
     "c4b_wide_200k_x_16385": (
         200000,
         "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=1> nch_rt=16 tail=16 pitch=16400 "
         "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        26287136019, "profiles/shard_pass_c4b_wide_200k_x_16385.md"),
+        26287135758, "profiles/shard_pass_c4b_wide_200k_x_16385.md"),
     "c5_e2e_2m_x_512": (
         2000000,
         "shard_pass<NCH=4,R=16,WCOL=1,WROW=2,ALLCH=1,TL=0> nch_rt=4 tail=0 pitch=512 "
         "grid=512 x 128 threads (occupancy 2 blocks/CU, 256 CUs)",
-        8210239930, "profiles/shard_pass_c5_e2e_2m_x_512.md"),
+        8210240021, "profiles/shard_pass_c5_e2e_2m_x_512.md"),
     "x_narrow_100m_x_2": (
         100000000,
         "lane_pass<NP=1,U=4,WROW=4> row-tiled layout, pitch=2, 256 rows per group, "
         "grid=768 x 256 threads (occupancy 3 blocks/CU, 256 CUs)",
-        2400581146, "profiles/lane_pass_x_narrow_100m_x_2.md"),
+        2400596292, "profiles/lane_pass_x_narrow_100m_x_2.md"),
     "x_narrow_30m_x_16": (
         30000000,
         "lane_pass<NP=8,U=1,WROW=4> row-tiled layout, pitch=16, 64 rows per group, "
         "grid=512 x 256 threads (occupancy 2 blocks/CU, 256 CUs)",
-        4080833731, "profiles/lane_pass_x_narrow_30m_x_16.md"),
+        4080835977, "profiles/lane_pass_x_narrow_30m_x_16.md"),
     "x_narrow_10m_x_41": (
         10000000,
         "lane2_pass<NP=21,U=2,WROW=1> row-tiled layout, pitch=42, 128 rows per group, "
         "grid=1024 x 128 threads (occupancy 4 blocks/CU, 256 CUs)",
-        3440528997, "profiles/lane2_pass_x_narrow_10m_x_41.md"),
+        3440526459, "profiles/lane2_pass_x_narrow_10m_x_41.md"),
     "x_short_30m_x_66": (
         30000000,
         "pair_pass<G=8,WROW=4> pitch=66, 16 rows per tile, grid=512 x 256 threads "
         "(occupancy 2 blocks/CU, 256 CUs)",
-        16137251227, "profiles/pair_pass_x_short_30m_x_66.md"),
+        16138109813, "profiles/pair_pass_x_short_30m_x_66.md"),
     "x_short_30m_x_72": (
         30000000,
         "pair_pass<G=8,WROW=4> pitch=72, 16 rows per tile, grid=512 x 256 threads "
         "(occupancy 2 blocks/CU, 256 CUs)",
-        17583255112, "profiles/pair_pass_x_short_30m_x_72.md"),
+        17578887363, "profiles/pair_pass_x_short_30m_x_72.md"),
     "x_c1shape_20m_x_100": (
         20000000,
         "shard_pass<NCH=1,R=32,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=1 tail=0 pitch=100 "
         "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs)",
-        16356181337, "profiles/shard_pass_x_c1shape_20m_x_100.md"),
+        16356598780, "profiles/shard_pass_x_c1shape_20m_x_100.md"),
     "x_bias_10m_x_257": (
         10000000,
         "shard_pass<NCH=2,R=32,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=2 tail=0 pitch=256 "
         "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs); first column constant "
         "1, not stored",
-        20560492288, "profiles/shard_pass_x_bias_10m_x_257.md"),
+        20560493013, "profiles/shard_pass_x_bias_10m_x_257.md"),
     "x_bias_1m_x_2049": (
         1000000,
         "shard_pass<NCH=16,R=2,WCOL=1,WROW=4,ALLCH=1,TL=0> nch_rt=16 tail=0 pitch=2048 "
         "grid=256 x 256 threads (occupancy 1 blocks/CU, 256 CUs); first column constant "
         "1, not stored",
-        16404232201, "profiles/shard_pass_x_bias_1m_x_2049.md"),
+        16404232399, "profiles/shard_pass_x_bias_1m_x_2049.md"),
     "x_wide_250k_x_9000": (
         250000,
         "shard_pass<NCH=9,R=2,WCOL=8,WROW=1,ALLCH=0,TL=0> nch_rt=9 tail=0 pitch=9008 "
         "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        18190744339, "profiles/shard_pass_x_wide_250k_x_9000.md"),
+        18190815749, "profiles/shard_pass_x_wide_250k_x_9000.md"),
     "x_wide_75k_x_20000": (
         75000,
         "team_pass<NCH=7,LAG=2> 3 column blocks of 52- chunks, 85 teams, pitch=20000 "
         "grid=255 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        12153875169, "profiles/team_pass_x_wide_75k_x_20000.md"),
+        12154026131, "profiles/team_pass_x_wide_75k_x_20000.md"),
     "x_verywide_100k_x_32768": (
         100000,
         "team_pass<NCH=8,LAG=1> 4 column blocks of 64 chunks, 64 teams, pitch=32768 "
         "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        26346237104, "profiles/team_pass_x_verywide_100k_x_32768.md"),
+        26346230791, "profiles/team_pass_x_verywide_100k_x_32768.md"),
     "x_wide_30k_x_50000": (
         30000,
         "team_pass<NCH=7,LAG=2> 7 column blocks of 55- chunks, 36 teams, pitch=50000 "
         "grid=252 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        12111987148, "profiles/team_pass_x_wide_30k_x_50000.md"),
+        12112114281, "profiles/team_pass_x_wide_30k_x_50000.md"),
 }
 
 # The other configurations a default run times after the headline.
