@@ -295,3 +295,76 @@ def test_get_data_returns_what_set_data_took(plr):
         X3, y3 = plr.get_data(n // 3, n // 2)
         assert X3.tobytes() == X[n // 3:n // 3 + n // 2].tobytes()
         assert y3.tobytes() == y[n // 3:n // 3 + n // 2].tobytes()
+
+
+def _random_field(rng):
+    k = rng.integers(0, 12)
+    v = rng.normal() * 10.0 ** rng.integers(-6, 7)
+    if k == 0:
+        return "%.6f" % v
+    if k == 1:
+        return "%.14e" % v
+    if k == 2:
+        return repr(float(v))
+    if k == 3:
+        return "%d" % int(v)
+    if k == 4:
+        return "%.17g" % v
+    if k == 5:
+        return "%.*f" % (int(rng.integers(0, 12)), v)
+    if k == 6:
+        return "%.2fE%+d" % (v % 10, int(rng.integers(-30, 31)))
+    if k == 7:
+        return "%d." % int(v)
+    if k == 8:
+        return "0" * int(rng.integers(1, 25)) + "%.3f" % abs(v)
+    if k == 9:
+        return "%.9g" % v
+    if k == 10:
+        return "-0" if rng.random() < 0.5 else ".5"
+    return "%.1f" % v + "0" * int(rng.integers(0, 30))   # tails that pass 32 characters
+
+
+def _random_text(rng):
+    k = int(rng.choice([1, 2, 3, 5, 8, 15, 16, 17, 31, 40, 63, 64, 65, 100, 257, 600, 3000]))
+    target = int(rng.choice([300, 4000, 4096, 8192, 20000, 70000, 300000]))   # bytes
+    eol = "\r\n" if rng.random() < 0.15 else "\n"
+    lines, size = [], 0
+    while size < target:
+        f = [_random_field(rng) for _ in range(k)] + [str(int(rng.integers(0, 2)))]
+        if rng.random() < 0.05:
+            f.insert(int(rng.integers(0, len(f))), "")      # an empty field: dropped
+        lines.append(",".join(f))
+        size += len(lines[-1]) + 1
+        if rng.random() < 0.03:
+            lines.append("")                                # a blank line ("\r" with CR LF)
+    text = eol.join(lines)
+    if rng.random() < 0.7:
+        text += eol
+    if rng.random() < 0.2:
+        text = eol * int(rng.integers(1, 4)) + text
+    return text
+
+
+def test_random_texts_against_the_oracle(plr, oracle):
+    # widths from 2 to 3001 fields, texts from a fraction of a 4 KiB block to 70 blocks, every
+    # spelling class mixed within a line, empty fields, blank lines, CR LF -- where the oracle's
+    # parser refuses a text (a line that is only "\r"), the device must refuse it too
+    from paracel_amd import PlrError
+
+    refused = 0
+    for seed in range(250):
+        rng = np.random.default_rng(seed)
+        text = _random_text(rng)
+        try:
+            Xo, yo = oracle.local_parser(text)
+        except ValueError:
+            with pytest.raises(PlrError):
+                plr.set_data_csv(text.encode())
+            refused += 1
+            continue
+        n, d = plr.set_data_csv(text.encode())
+        X, y = plr.get_data()
+        assert (n, d) == Xo.shape, seed
+        assert X.tobytes() == Xo.tobytes() and y.tobytes() == yo.tobytes(), seed
+    assert refused < 60
