@@ -324,8 +324,11 @@ __global__ __launch_bounds__(kCsvThreads) void csv_parse_fields(CsvFieldArgs a) 
     int sig = 0, ndig = 0, frac = 0, e10 = 0, ed = 0, st = 0, flen = 0;  // st: 0 int, 1 frac, 2 exp sign, 3 exp
     bool neg = false, eneg = false, bad = false, act = true;
     for (int j = 0; __any(act); ++j) {
-      const int ch = txt[pos + (act ? j : 0)];
-      const bool term = ch == a.sep || ch == '\n';
+      const int at = pos + (act ? j : 0);
+      const int ch = txt[at];
+      // a carriage return in front of the newline ends the number like the
+      // newline does: std::stod stops there and ignores it (CR LF line ends)
+      const bool term = ch == a.sep || ch == '\n' || (ch == '\r' && txt[at + 1] == '\n');
       // longer than the device converts: the host finds its end
       const bool over = act && !term && j == kCsvMaxFieldChars;
       bad = bad || over;
