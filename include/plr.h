@@ -76,9 +76,11 @@ int plr_set_data_chunk(plr_ctx* ctx, int64_t row0, int64_t nrows,
  * *d_out) and the label -- with every field's value exactly std::stod's: the
  * device converts decimal spellings of up to 19 significant digits whose
  * correctly rounded value it can establish (all but those within 2^-30 of a
- * unit in the last place of a rounding tie), the rest (longer digit strings,
- * exponents beyond +-44, inf, nan, hex, blanks, trailing characters) are
- * converted by std::stod on the host.  Empty fields are
+ * unit in the last place of a rounding tie; blanks and tabs in front are
+ * skipped, a blank, a tab or the carriage return of a CR LF line end behind
+ * the number ends it, as for std::stod), the rest (longer digit strings,
+ * exponents beyond +-44, inf, nan, hex, a plus sign, other trailing
+ * characters) are converted by std::stod on the host.  Empty fields are
  * skipped like the reference's str_split does.  *n_out receives the number
  * of samples.  Errors as the reference's parser would raise them (a field
  * std::stod rejects, a line with another number of fields) come back as

@@ -17,7 +17,9 @@
 //
 // A field is converted on the device only when the result is provably strtod's,
 // the correctly rounded value of the decimal.  The spelling must be
-// [-]digits[.digits][e[+-]digits]; then
+// [-]digits[.digits][e[+-]digits], with blanks or tabs in front if any and,
+// behind a blank or tab (or the carriage return of a CR LF line end), anything
+// at all -- what std::stod skips and what it ignores; then
 //   * at most 15 significant digits and a decimal exponent within +-22: the
 //     digits are an exact double, 10^|e| is an exact double, and the one
 //     multiplication or division rounds once (Clinger's fast path; the host
@@ -323,6 +325,7 @@ __global__ __launch_bounds__(kCsvThreads) void csv_parse_fields(CsvFieldArgs a) 
     unsigned long long m = 0;
     int sig = 0, ndig = 0, frac = 0, e10 = 0, ed = 0, st = 0, flen = 0;  // st: 0 int, 1 frac, 2 exp sign, 3 exp
     bool neg = false, eneg = false, bad = false, act = true;
+    bool started = false, done = false;  // past the leading blanks; past a blank behind the number
     for (int j = 0; __any(act); ++j) {
       const int at = pos + (act ? j : 0);
       const int ch = txt[at];
@@ -334,25 +337,36 @@ __global__ __launch_bounds__(kCsvThreads) void csv_parse_fields(CsvFieldArgs a) 
       bad = bad || over;
       flen = over ? -1 : flen;
       act = act && !term && !over;
+      // std::stod skips blanks in front of the number and ignores whatever
+      // follows it: blanks and tabs in front are passed over here, and a blank
+      // or tab behind a complete number ends it (the rest of the field is not
+      // looked at); a number cut short by one ("1e 5") is the host's
+      const bool blank = ch == ' ' || ch == '\t';
+      const bool first = act && !started && !blank;
+      const bool ends = act && started && !done && blank;
+      bad = bad || (ends && !(ndig > 0 && (st <= 1 || (st == 3 && ed > 0))));
+      const bool live = act && !done && !ends && (started || first);
+      done = done || ends;
+      started = started || first;
       const int dv = ch - '0';
       const bool digit = (unsigned)dv <= 9u;
-      const bool mant = act && st <= 1;
+      const bool mant = live && st <= 1;
       const bool mdig = mant && digit;
       m = mdig ? m * 10ull + (unsigned long long)dv : m;
       sig += (mdig && m != 0ull) ? 1 : 0;
       ndig += mdig ? 1 : 0;
       frac += (mdig && st == 1) ? 1 : 0;
-      const bool minus0 = mant && ch == '-' && j == 0;
+      const bool minus0 = mant && ch == '-' && first;
       neg = neg || minus0;
       const bool dot = mant && ch == '.' && st == 0;
       const bool ee = mant && (ch | 0x20) == 'e' && ndig > 0;
-      const bool esign = act && st == 2 && (ch == '+' || ch == '-');
+      const bool esign = live && st == 2 && (ch == '+' || ch == '-');
       eneg = eneg || (esign && ch == '-');
-      const bool edig = act && st >= 2 && digit;
+      const bool edig = live && st >= 2 && digit;
       const int e_next = e10 * 10 + dv;
       e10 = edig ? (e_next > 99999 ? 99999 : e_next) : e10;
       ed += edig ? 1 : 0;
-      bad = bad || (act && !(mdig || minus0 || dot || ee || esign || edig)) || sig > 19;
+      bad = bad || (live && !(mdig || minus0 || dot || ee || esign || edig)) || sig > 19;
       st = dot ? 1 : ee ? 2 : (esign || edig) ? 3 : st;
       flen += act ? 1 : 0;
     }

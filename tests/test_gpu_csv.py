@@ -115,6 +115,14 @@ def test_fields_the_host_converts_and_odd_lines(plr, oracle):
            % ("0" * 40))
     Xo, _ = check_equal(plr, oracle, odd)
     assert np.isinf(Xo[0, 1]) and Xo[0, 3] == 8.0 and np.signbit(Xo[1, 5])
+    # blanks and tabs in front of a number, and a blank behind it with whatever follows, are
+    # what std::stod skips and ignores: converted on the device like the bare number
+    spaced = "".join("%.3f, %.2f,\t%d ,%.1f  x, -%.4f,1\n" % (v[0], v[1], int(v[2]), v[3], abs(v[4]))
+                     for v in rng.normal(size=(300, 5)) * 7)
+    check_equal(plr, oracle, spaced)
+    assert host_converted(plr) == 0
+    check_equal(plr, oracle, "1e 5,2,1\n3 e2, 4 5,0\n")      # "1e 5" is 1, and the host's
+    assert host_converted(plr) == 1
     check_equal(plr, oracle, "1,,2,,,3,1\n4,5,,6,0\n")
     check_equal(plr, oracle, "1;2;1\n3;4;0\n", sep=";")
     nan_line = "nan,1,1\n"
@@ -326,6 +334,14 @@ def _random_field(rng):
         return "%.9g" % v
     if k == 10:
         return "-0" if rng.random() < 0.5 else ".5"
+    if rng.random() < 0.3:
+        # blanks and tabs as std::stod treats them: skipped in front, the end of the number
+        # behind it (whatever follows), an error when nothing else is there
+        if rng.random() < 0.002:
+            return str(rng.choice(["- 5", " . 5", "  "]))       # no number: the text is refused
+        return str(rng.choice([" %.3f" % v, "\t%.4f " % v, "%.2f  " % v, "  %d\t" % int(v),
+                               "%.3f abc" % v, "%.1f 7" % v, "1e 5", "%.2e\tx" % v, " -.5",
+                               "5. ", " 1"]))
     return "%.1f" % v + "0" * int(rng.integers(0, 30))   # tails that pass 32 characters
 
 
@@ -371,4 +387,4 @@ def test_random_texts_against_the_oracle(plr, oracle):
         X, y = plr.get_data()
         assert (n, d) == Xo.shape, seed
         assert X.tobytes() == Xo.tobytes() and y.tobytes() == yo.tobytes(), seed
-    assert refused < 60
+    assert refused < 90
