@@ -240,8 +240,8 @@ __global__ __launch_bounds__(1024) void csv_scan_blocks(const int* rows, const i
 }
 
 __global__ __launch_bounds__(kCsvThreads) void csv_parse_fields(CsvFieldArgs a) {
-  constexpr int kAhead = 64;  // staged behind the block: a field of 32 characters and its end
-  static_assert(kAhead > kCsvMaxFieldChars + 1 && kAhead <= kCsvPadBytes, "look-ahead");
+  constexpr int kAhead = 64;  // staged behind the block: 8 blanks, a number of 32 characters, its end
+  static_assert(kAhead > 8 + kCsvMaxFieldChars + 2 && kAhead <= kCsvPadBytes, "look-ahead");
   __shared__ __align__(16) unsigned char txt[kCsvBlockBytes + kAhead];
   __shared__ unsigned short fpos[kCsvBlockBytes / 2 + 1];  // a field start at every other byte at most
   __shared__ int wf[kCsvThreads / 64], wr[kCsvThreads / 64];
@@ -325,51 +325,54 @@ __global__ __launch_bounds__(kCsvThreads) void csv_parse_fields(CsvFieldArgs a) 
     unsigned long long m = 0;
     int sig = 0, ndig = 0, frac = 0, e10 = 0, ed = 0, st = 0, flen = 0;  // st: 0 int, 1 frac, 2 exp sign, 3 exp
     bool neg = false, eneg = false, bad = false, act = true;
-    bool started = false, done = false;  // past the leading blanks; past a blank behind the number
+    // std::stod skips white space in front of the number and ignores whatever
+    // follows it.  White space in front (up to 8 characters) is passed over
+    // before the walk; white space met during the walk -- a blank, a tab, the
+    // carriage return of a CR LF line end -- ends the number like a terminator:
+    // if it is complete by then (the checks behind the loop), the rest of the
+    // field does not matter, and if not ("1e 5") the field is the host's, which
+    // finds its end itself.
+    auto blank = [](int ch) { return ch == ' ' || (unsigned)(ch - '\t') <= 4u; };  // isspace
+    int lead = 0;
+    while (lead < 8 && blank(txt[pos + lead]) && txt[pos + lead] != '\n' &&
+           txt[pos + lead] != a.sep)  // (a separator may itself be a blank or a tab)
+      ++lead;
+    const int num = pos + lead;  // the number's first character
+    bool blank_end = false;
     for (int j = 0; __any(act); ++j) {
-      const int at = pos + (act ? j : 0);
+      const int at = num + (act ? j : 0);
       const int ch = txt[at];
-      // a carriage return in front of the newline ends the number like the
-      // newline does: std::stod stops there and ignores it (CR LF line ends)
-      const bool term = ch == a.sep || ch == '\n' || (ch == '\r' && txt[at + 1] == '\n');
+      const bool term = ch == a.sep || ch == '\n';
       // longer than the device converts: the host finds its end
       const bool over = act && !term && j == kCsvMaxFieldChars;
       bad = bad || over;
       flen = over ? -1 : flen;
-      act = act && !term && !over;
-      // std::stod skips blanks in front of the number and ignores whatever
-      // follows it: blanks and tabs in front are passed over here, and a blank
-      // or tab behind a complete number ends it (the rest of the field is not
-      // looked at); a number cut short by one ("1e 5") is the host's
-      const bool blank = ch == ' ' || ch == '\t';
-      const bool first = act && !started && !blank;
-      const bool ends = act && started && !done && blank;
-      bad = bad || (ends && !(ndig > 0 && (st <= 1 || (st == 3 && ed > 0))));
-      const bool live = act && !done && !ends && (started || first);
-      done = done || ends;
-      started = started || first;
+      const bool stop = act && !term && !over && blank(ch);
+      blank_end = blank_end || stop;
+      act = act && !term && !over && !stop;
       const int dv = ch - '0';
       const bool digit = (unsigned)dv <= 9u;
-      const bool mant = live && st <= 1;
+      const bool mant = act && st <= 1;
       const bool mdig = mant && digit;
       m = mdig ? m * 10ull + (unsigned long long)dv : m;
       sig += (mdig && m != 0ull) ? 1 : 0;
       ndig += mdig ? 1 : 0;
       frac += (mdig && st == 1) ? 1 : 0;
-      const bool minus0 = mant && ch == '-' && first;
+      const bool minus0 = mant && ch == '-' && j == 0;
       neg = neg || minus0;
       const bool dot = mant && ch == '.' && st == 0;
       const bool ee = mant && (ch | 0x20) == 'e' && ndig > 0;
-      const bool esign = live && st == 2 && (ch == '+' || ch == '-');
+      const bool esign = act && st == 2 && (ch == '+' || ch == '-');
       eneg = eneg || (esign && ch == '-');
-      const bool edig = live && st >= 2 && digit;
+      const bool edig = act && st >= 2 && digit;
       const int e_next = e10 * 10 + dv;
       e10 = edig ? (e_next > 99999 ? 99999 : e_next) : e10;
       ed += edig ? 1 : 0;
-      bad = bad || (live && !(mdig || minus0 || dot || ee || esign || edig)) || sig > 19;
+      bad = bad || (act && !(mdig || minus0 || dot || ee || esign || edig)) || sig > 19;
       st = dot ? 1 : ee ? 2 : (esign || edig) ? 3 : st;
       flen += act ? 1 : 0;
     }
+    flen = (blank_end || flen < 0) ? -1 : flen + lead;  // as the host will read it, from pos
     if (e10 > 9999) bad = true;
     const int e = (eneg ? -e10 : e10) - frac;
     if (ndig == 0 || st == 2 || (st == 3 && ed == 0) || e < -44 || e > 44) bad = true;

@@ -125,6 +125,9 @@ def test_fields_the_host_converts_and_odd_lines(plr, oracle):
     assert host_converted(plr) == 1
     check_equal(plr, oracle, "1,,2,,,3,1\n4,5,,6,0\n")
     check_equal(plr, oracle, "1;2;1\n3;4;0\n", sep=";")
+    # a blank or a tab as the separator: white space of the other kind still belongs to a field
+    check_equal(plr, oracle, "1.5\t2.5\t1\n 3\t4 \t0\n\t5\t\t6\t1\n", sep="\t")
+    check_equal(plr, oracle, "1.5 2.5 1\n\t3 4\t 0\n", sep=" ")
     nan_line = "nan,1,1\n"
     n, d = plr.set_data_csv(nan_line.encode())
     X, y = plr.get_data()
