@@ -102,16 +102,15 @@ inline bool plan_width(int64_t d, Plan& p, int64_t n = -1) {
       const int64_t widest = p.team_blk_chunks + (p.team_blk_extra ? 1 : 0);
       p.team_nch = (int)ceil_div(widest, kTeamWaves);  // 7 or 8: more than 152 chunks in >= 3 blocks
       if (p.team_nch < kTeamMinNch) p.team_nch = kTeamMinNch;
-      // How many steps a row's update trails its dot product.  Two steps hide the
-      // exchange of the partial dots better (measured on 12 GB shards, one
-      // session, fraction of 8 TB/s with one step -> two: 20000 columns 0.80 ->
-      // 0.82, 40000 0.83 -> 0.85, 50000 0.79 -> 0.82, 65536 0.855 -> 0.87,
-      // 100000 0.73 -> 0.80, 131072 0.81 -> 0.88, 262144 0.73 -> 0.84, 524288
-      // 0.67 -> 0.76) but cost a fourth row buffer; where every wave owns all 8
-      // chunks and the team is small (24576, 32768 columns) the two are within
-      // 1 % of each other in either direction, and one step needs no spill.
-      const bool full = chunks == blocks * kTeamWaves * kTeamNch;
-      p.team_lag = (full && blocks <= 4) ? 1 : 2;
+      // How many steps a row's update trails its dot product.  Two steps give the
+      // exchange of the partial dots more time but cost a fourth row buffer.
+      // Measured on 12 GB shards, one session, fraction of 8 TB/s with one step
+      // -> two: teams of 3 (19457 columns 0.83 -> 0.81, 20000 0.83 -> 0.82, 24576
+      // 0.85 -> 0.83) and 4 (32768 0.85 -> 0.84) are better off with one; from 5
+      // on two pay, the more the larger the team (40000 0.83 -> 0.85, 50000 0.82
+      // -> 0.85, 65536 0.85 -> 0.86, 100000 0.72 -> 0.83, 131072 0.76 -> 0.88,
+      // 262144 0.67 -> 0.87, 524288 0.62 -> 0.79).
+      p.team_lag = blocks <= 4 ? 1 : 2;
     }
     // one more chunk of padding: the page of zeros an unowned chunk slot reads
     p.theta_len += kChunkCols;
