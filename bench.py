@@ -63,12 +63,12 @@ MEASURED_TRAFFIC = {
         200000,
         "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=0> nch_rt=16 tail=0 pitch=16384 "
         "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        26261494892, "profiles/shard_pass_c4_wide_200k_x_16384.md"),
+        26261494888, "profiles/shard_pass_c4_wide_200k_x_16384.md"),
     "c4b_wide_200k_x_16385": (
         200000,
         "shard_pass<NCH=16,R=1,WCOL=8,WROW=1,ALLCH=1,TL=1> nch_rt=16 tail=16 pitch=16400 "
         "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        26287135758, "profiles/shard_pass_c4b_wide_200k_x_16385.md"),
+        26287135754, "profiles/shard_pass_c4b_wide_200k_x_16385.md"),
     "c5_e2e_2m_x_512": (
         2000000,
         "shard_pass<NCH=4,R=16,WCOL=1,WROW=2,ALLCH=1,TL=0> nch_rt=4 tail=0 pitch=512 "
@@ -120,22 +120,22 @@ MEASURED_TRAFFIC = {
         250000,
         "shard_pass<NCH=9,R=2,WCOL=8,WROW=1,ALLCH=0,TL=0> nch_rt=9 tail=0 pitch=9008 "
         "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        18190815749, "profiles/shard_pass_x_wide_250k_x_9000.md"),
+        18190815746, "profiles/shard_pass_x_wide_250k_x_9000.md"),
     "x_wide_75k_x_20000": (
         75000,
-        "team_pass<NCH=7,LAG=2> 3 column blocks of 52- chunks, 85 teams, pitch=20000 "
+        "team_pass<NCH=7,LAG=1> 3 column blocks of 52- chunks, 85 teams, pitch=20000 "
         "grid=255 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        12154026131, "profiles/team_pass_x_wide_75k_x_20000.md"),
+        12149365862, "profiles/team_pass_x_wide_75k_x_20000.md"),
     "x_verywide_100k_x_32768": (
         100000,
         "team_pass<NCH=8,LAG=1> 4 column blocks of 64 chunks, 64 teams, pitch=32768 "
         "grid=256 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        26346230791, "profiles/team_pass_x_verywide_100k_x_32768.md"),
+        26348055385, "profiles/team_pass_x_verywide_100k_x_32768.md"),
     "x_wide_30k_x_50000": (
         30000,
         "team_pass<NCH=7,LAG=2> 7 column blocks of 55- chunks, 36 teams, pitch=50000 "
         "grid=252 x 512 threads (occupancy 1 blocks/CU, 256 CUs)",
-        12112114281, "profiles/team_pass_x_wide_30k_x_50000.md"),
+        12111127486, "profiles/team_pass_x_wide_30k_x_50000.md"),
 }
 
 # The other configurations a default run times after the headline.
