@@ -294,6 +294,8 @@ struct plr_ctx {
   // finishing kernel's blocks store the pass number to (FinishArgs::done)
   volatile unsigned long long* h_done = nullptr;
   unsigned long long* h_done_dev = nullptr;
+  volatile unsigned long long* h_status = nullptr;  // behind them: finish_pass's copy of a
+  unsigned long long* h_status_dev = nullptr;       //   team pass's give-up word
   unsigned long long pass_seq = 0;
   int done_blocks = 0;          // > 0: the pass just enqueued reports through h_done
   bool opt_poll_results = true; // plr_set_option("poll_results")
@@ -633,12 +635,14 @@ int alloc_workspace(plr_ctx* c) {
   // results land in host memory straight from the finishing kernel (no
   // device-to-host copy in the step): pinned, mapped, coherent
   const size_t done_at = ((size_t)(d + 1) + 7) / 8 * 8;  // in doubles: the next cache line
-  PLR_HIP(c, hipHostMalloc(&c->h_out, (done_at + kDoneWords) * sizeof(double),
+  PLR_HIP(c, hipHostMalloc(&c->h_out, (done_at + kDoneWords + 8) * sizeof(double),
                            hipHostMallocMapped | hipHostMallocCoherent));
   PLR_HIP(c, hipHostGetDevicePointer(reinterpret_cast<void**>(&c->h_out_dev), c->h_out, 0));
-  memset(c->h_out, 0, (done_at + kDoneWords) * sizeof(double));
+  memset(c->h_out, 0, (done_at + kDoneWords + 8) * sizeof(double));
   c->h_done = reinterpret_cast<volatile unsigned long long*>(c->h_out + done_at);
   c->h_done_dev = reinterpret_cast<unsigned long long*>(c->h_out_dev + done_at);
+  c->h_status = c->h_done + kDoneWords;
+  c->h_status_dev = c->h_done_dev + kDoneWords;
   memset(c->h_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double));
   PLR_HIP(c, hipMemsetAsync(c->d_theta, 0, (size_t)(c->theta_len + 8) * sizeof(double), c->stream));
   PLR_HIP(c, hipStreamSynchronize(c->stream));
@@ -846,6 +850,8 @@ int enqueue_pass(plr_ctx* c, PassKind kind, unsigned loss_mode, double alpha, do
     const int fblocks = grad ? (int)ceil_div(c->dcols, plr::kFinCols) : 1;
     // a pass short enough for the stream's own completion signal to matter
     // reports to the polling host thread as well (run_pass)
+    fa.status_in = team ? reinterpret_cast<const unsigned*>(c->d_zx + c->zx_words) : nullptr;
+    fa.status_out = c->h_status_dev;
     fa.done = nullptr;
     fa.seq = 0;
     if (c->opt_poll_results && out == c->h_out_dev && fblocks <= kDoneWords) {
@@ -899,10 +905,10 @@ int account_timing(plr_ctx* c) {
 int team_gave_up(plr_ctx* c) {
   if (!c->team_check) return 0;
   c->team_check = false;
-  unsigned long long st = 0;
-  PLR_HIP(c, hipMemcpy(&st, c->d_zx + c->zx_words, sizeof st, hipMemcpyDeviceToHost));
-  if ((unsigned)st == 0u) return 0;
-  PLR_HIP(c, hipMemset(c->d_zx + c->zx_words, 0, sizeof st));
+  // (the finishing kernel of every team pass leaves a copy of the word in host memory)
+  if ((unsigned)*c->h_status == 0u) return 0;
+  *c->h_status = 0;
+  PLR_HIP(c, hipMemset(c->d_zx + c->zx_words, 0, sizeof(unsigned long long)));
   return 1;
 }
 
@@ -2350,6 +2356,8 @@ int plr_loss_grad_noalloc(int device_id, void* hip_stream, const double* dX, con
   fa.theta_bias = nullptr;
   fa.done = nullptr;
   fa.seq = 0;
+  fa.status_in = nullptr;
+  fa.status_out = nullptr;
   hipLaunchKernelGGL(plr::finish_pass, dim3((int)ceil_div(d, plr::kFinCols)),
                      dim3(plr::kFinCols * plr::kFinSlices), 0, stream, fa);
   PLR_NA_HIP(hipGetLastError());

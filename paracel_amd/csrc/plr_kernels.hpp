@@ -1602,6 +1602,11 @@ struct FinishArgs {
   // polls these words has the results without waiting for the stream to drain)
   unsigned long long* done;
   unsigned long long seq;
+  // nullable: a team pass's give-up word (device memory) and where to leave a
+  // copy of it for the host (host memory the device can write), so that the
+  // host need not fetch it with a copy of its own after every pass
+  const unsigned* status_in;
+  unsigned long long* status_out;
 };
 
 constexpr int kFinCols = 16;
@@ -1679,6 +1684,7 @@ __global__ __launch_bounds__(kFinCols* kFinSlices) void finish_pass(FinishArgs a
       }
     }
   }
+  if (a.status_in && blockIdx.x == 0 && threadIdx.x == 0) *a.status_out = *a.status_in;
   if (a.done) {
     __syncthreads();  // every store of this block to `out` has been issued ...
     if (threadIdx.x == 0)  // ... and is visible to the host before the word is
